@@ -1,0 +1,184 @@
+"""The engine against the plain implementation, in float32 and bfloat16, under
+every way of cutting the work: whole requests, the last 32 tokens one by
+one, portions of changing size, and mixed batches with so few pages that
+they are used again."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import plain_model
+from conftest import TINY
+from replay_helpers import (check_against_plain, cut, max_live_tokens, random_requests, run_in_process,
+                            run_trace_run, trace_alone, trace_mixed)
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = ["float32", "bfloat16"]
+CONFIGS = ["A", "B", "W"]
+_plain_cache = {}
+_models = {}
+
+
+def get_model(folders, name, dtype):
+    from vt_transformer_amd.engine import load_model
+    key = (name, dtype)
+    if key not in _models:
+        _models[key] = load_model(folders[name], dtype)
+    return _models[key]
+
+
+def runner_for(model, pool_tokens, max_requests=8):
+    from vt_transformer_amd.engine import make_runner
+    return make_runner(model, pool_tokens=pool_tokens, page_size=16, max_requests=max_requests,
+                       max_seq_len=min(model.spec.max_positions, max(pool_tokens, 16)))
+
+
+def report(name, worst):
+    os.makedirs("gpurun_out", exist_ok=True)
+    with open("gpurun_out/engine_errors.txt", "a") as f:
+        f.write(f"{name}: worst relative error {worst:.3e}\n")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("cfg", CONFIGS)
+def test_whole_requests(model_folders, cfg, dtype):
+    """Each request alone and whole, logits at every position."""
+    reqs = random_requests(TINY[cfg]["vocab_size"], [5, 9, 13, 1, 70, 150], seed=1)
+    steps = trace_alone(reqs, {r: [(0, len(t))] for r, t in reqs.items()})
+    runner = runner_for(get_model(model_folders, cfg, dtype), 192)
+    got = run_in_process(runner, steps)
+    worst = check_against_plain(model_folders[cfg], reqs, steps, got, dtype, _plain_cache)
+    report(f"whole {cfg} {dtype}", worst)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("cfg", CONFIGS)
+def test_last_32_one_by_one(model_folders, cfg, dtype):
+    """Most of a request in one step, its last 32 tokens decoded one by one."""
+    reqs = random_requests(TINY[cfg]["vocab_size"], [40, 97, 33], seed=2)
+    portions = {r: [(0, len(t) - 32)] + [(i, i + 1) for i in range(len(t) - 32, len(t))] for r, t in reqs.items()}
+    steps = trace_alone(reqs, portions)
+    runner = runner_for(get_model(model_folders, cfg, dtype), 128)
+    got = run_in_process(runner, steps)
+    worst = check_against_plain(model_folders[cfg], reqs, steps, got, dtype, _plain_cache)
+    report(f"last32 {cfg} {dtype}", worst)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("cfg", CONFIGS)
+def test_portions_of_changing_size(model_folders, cfg, dtype):
+    reqs = random_requests(TINY[cfg]["vocab_size"], [61, 100, 47], seed=3)
+    sizes = {"r0": [7, 2, 5, 3, 2, 16, 2, 9], "r1": [2, 2, 31, 17, 1, 2, 15, 16, 3], "r2": [15, 1, 16, 2, 13]}
+    steps = trace_alone(reqs, {r: cut(t, sizes[r]) for r, t in reqs.items()})
+    runner = runner_for(get_model(model_folders, cfg, dtype), 128)
+    got = run_in_process(runner, steps)
+    worst = check_against_plain(model_folders[cfg], reqs, steps, got, dtype, _plain_cache)
+    report(f"portions {cfg} {dtype}", worst)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("cfg", CONFIGS)
+def test_mixed_batches_with_page_reuse(model_folders, cfg, dtype):
+    """Up to four live requests, portions of some beside decoded tokens of others; the pool is only as large as
+    the trace needs at its peak, so later requests get the pages of finished ones."""
+    lengths = [31, 16, 7, 1, 50, 33, 64, 20, 45, 18]
+    reqs = random_requests(TINY[cfg]["vocab_size"], lengths, seed=4)
+    portions = {}
+    for i, (r, t) in enumerate(reqs.items()):
+        head = [8, 3, 2] if i % 2 == 0 else [5, 11]
+        n_head = max(0, len(t) - 9)
+        parts = [p for p in cut(t[:n_head], head)] if n_head else []
+        parts += [(j, j + 1) for j in range(n_head, len(t))]   # the last tokens one by one
+        portions[r] = parts
+    steps = trace_mixed(reqs, portions, max_live=4, seed=5)
+    pool = max_live_tokens(steps)
+    runner = runner_for(get_model(model_folders, cfg, dtype), pool, max_requests=4)
+    got = run_in_process(runner, steps)
+    worst = check_against_plain(model_folders[cfg], reqs, steps, got, dtype, _plain_cache)
+    report(f"mixed {cfg} {dtype} pool={pool}", worst)
+    assert sum(runner.cache.held_pages()) == 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("cfg", ["A", "W"])
+def test_long_decoding(model_folders, cfg, dtype):
+    """Three tokens of prompt, then 300 tokens one by one, two requests side by side."""
+    reqs = random_requests(TINY[cfg]["vocab_size"], [303, 280], seed=6)
+    portions = {r: [(0, 3)] + [(i, i + 1) for i in range(3, len(t))] for r, t in reqs.items()}
+    steps = trace_mixed(reqs, portions, max_live=2, seed=7, skip_prob=0.0)
+    runner = runner_for(get_model(model_folders, cfg, dtype), 640)
+    got = run_in_process(runner, steps)
+    worst = check_against_plain(model_folders[cfg], reqs, steps, got, dtype, _plain_cache)
+    report(f"long decoding {cfg} {dtype}", worst)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_first_tokens(model_folders, dtype):
+    """The very first positions, each as a step of its own."""
+    reqs = random_requests(TINY["B"]["vocab_size"], [4, 3], seed=8)
+    steps = trace_alone(reqs, {r: [(i, i + 1) for i in range(len(t))] for r, t in reqs.items()})
+    runner = runner_for(get_model(model_folders, "B", dtype), 64)
+    got = run_in_process(runner, steps)
+    check_against_plain(model_folders["B"], reqs, steps, got, dtype, _plain_cache)
+
+
+def test_wanted_rows_equal_rows_of_all(model_folders):
+    """Logits only at the wanted places are the same rows as when every place is wanted."""
+    from vt_transformer_amd.engine import StepEntry
+    model = get_model(model_folders, "B", "float32")
+    toks = random_requests(TINY["B"]["vocab_size"], [23], seed=9)["r0"]
+    r1 = runner_for(model, 64)
+    r1.admit("x")
+    full = r1.step([StepEntry("x", toks, list(range(23)))]).cpu()
+    r2 = runner_for(model, 64)
+    r2.admit("x")
+    some = r2.step([StepEntry("x", toks, [22, 0, 7])]).cpu()
+    assert torch.equal(some, full[[22, 0, 7]])
+    r3 = runner_for(model, 64)
+    r3.admit("x")
+    assert r3.step([StepEntry("x", toks, [])]) is None
+
+
+def test_fp32_does_not_depend_on_cut_or_batch(model_folders):
+    """In float32 the same position gives bit-equal logits whole, token by token, and beside other requests."""
+    from vt_transformer_amd.engine import StepEntry
+    model = get_model(model_folders, "A", "float32")
+    reqs = random_requests(TINY["A"]["vocab_size"], [37, 20], seed=10)
+    a, b = reqs["r0"], reqs["r1"]
+    r = runner_for(model, 256)
+    r.admit("w")
+    whole = r.step([StepEntry("w", a, [36])]).cpu()
+    r.admit("s"); r.admit("o")
+    r.step([StepEntry("s", a[:30], []), StepEntry("o", b[:5], [])])
+    for i in range(30, 36):
+        r.step([StepEntry("s", a[i:i + 1], []), StepEntry("o", b[5 + i - 30:6 + i - 30], [0])])
+    last = r.step([StepEntry("o", b[11:13], [1]), StepEntry("s", a[36:37], [0])]).cpu()
+    assert torch.equal(last[1], whole[0])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_trace_run_program(model_folders, dtype, tmp_path):
+    """The replay program itself, as a child process fed step by step."""
+    cfg = "B"
+    reqs = random_requests(TINY[cfg]["vocab_size"], [20, 35, 9, 41, 12], seed=11)
+    portions = {r: cut(t, [6, 2, 9, 1]) for r, t in reqs.items()}
+    steps = trace_mixed(reqs, portions, max_live=4, seed=12)
+    steps[1]["entries"][0]["want"] = []          # a step may want nothing from an entry
+    got = run_trace_run(model_folders[cfg], dtype, steps, str(tmp_path / "out"), max_live_tokens(steps),
+                        TINY[cfg]["vocab_size"])
+    worst = check_against_plain(model_folders[cfg], reqs, steps, got, dtype, _plain_cache)
+    report(f"trace_run {cfg} {dtype}", worst)
+
+
+def test_random_weights_on_device_match_written_folder(model_folders):
+    """random_model draws on the device; a written folder draws on the host.  Both must be proper models of the
+    configuration (their values differ: the generators do)."""
+    from vt_transformer_amd.config import config_from_dict
+    from vt_transformer_amd.engine import StepEntry, random_model
+    model = random_model(config_from_dict(dict(TINY["A"])), seed=3, dtype="bfloat16")
+    r = runner_for(model, 64)
+    r.admit(0)
+    logits = r.step([StepEntry(0, [1, 2, 3, 4, 5], [4])])
+    assert logits.shape == (1, TINY["A"]["vocab_size"]) and bool(torch.isfinite(logits).all())

@@ -1,0 +1,433 @@
+"""Each HIP kernel alone against a plain float64 reference of the same op,
+at sizes other than the engine tests': widths that are no power of two, odd
+head groups, head sizes from 16 to 256, pages in shuffled order."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda"
+
+
+def ops():
+    from vt_transformer_amd.kernels import ops as o
+    return o
+
+
+def rel_err(got: torch.Tensor, ref: torch.Tensor) -> float:
+    ref = ref.double().cpu()
+    got = got.double().cpu()
+    return float((got - ref).abs().max() / ref.abs().max().clamp_min(1e-30))
+
+
+def bf16_round(x: torch.Tensor) -> torch.Tensor:
+    return x.to(torch.bfloat16).to(torch.float64)
+
+
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("vocab,hidden,n", [(203, 80, 7), (1000, 3584, 33)])
+def test_embed(dtype, vocab, hidden, n):
+    g = torch.Generator().manual_seed(1)
+    table = torch.randn(vocab, hidden, generator=g).to(dtype)
+    ids = torch.randint(0, vocab, (n,), generator=g, dtype=torch.int32)
+    ids[0], ids[-1] = vocab - 1, 0
+    out = torch.empty(n, hidden, dtype=torch.float32, device=DEV)
+    ops().embed(table.to(DEV), ids.to(DEV), out)
+    assert torch.equal(out.cpu(), table.float()[ids.long()])
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("delta_dtype", [None, torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n,hidden,eps", [(5, 80, 1e-5), (3, 3584, 1e-6), (2, 1000, 1e-2)])
+def test_rmsnorm_with_residual(out_dtype, delta_dtype, n, hidden, eps):
+    g = torch.Generator().manual_seed(2)
+    h = torch.randn(n, hidden, generator=g) * 3
+    gain = 1 + 0.1 * torch.randn(hidden, generator=g)
+    delta = None if delta_dtype is None else torch.randn(n, hidden, generator=g).to(delta_dtype)
+    x = h.double() + (delta.double() if delta is not None else 0)
+    ref = gain.double() * x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
+    hd = h.to(DEV)
+    out = torch.empty(n, hidden, dtype=out_dtype, device=DEV)
+    ops().rmsnorm(hd, delta.to(DEV) if delta is not None else None, gain.to(DEV), out, eps)
+    tol = 1e-5 if out_dtype == torch.float32 else 5e-3
+    assert rel_err(out, ref) < tol
+    # the sum went back into the residual stream, in fp32
+    assert rel_err(hd, x) < 1e-6
+    # eps sits inside the root: a large eps must show
+    if eps == 1e-2:
+        wrong = gain.double() * x / (torch.sqrt((x * x).mean(-1, keepdim=True)) + eps)
+        assert rel_err(out, wrong) > 10 * tol or out_dtype == torch.bfloat16
+
+
+def test_rmsnorm_rows_gather():
+    g = torch.Generator().manual_seed(3)
+    h = torch.randn(9, 96, generator=g)
+    delta = torch.randn(9, 96, generator=g)
+    gain = torch.randn(96, generator=g)
+    rows = torch.tensor([8, 0, 3], dtype=torch.int32)
+    x = (h + delta).double()[rows.long()]
+    ref = gain.double() * x / torch.sqrt((x * x).mean(-1, keepdim=True) + 1e-6)
+    hd = h.to(DEV)
+    out = torch.empty(3, 96, dtype=torch.float32, device=DEV)
+    ops().rmsnorm(hd, delta.to(DEV), gain.to(DEV), out, 1e-6, rows=rows.to(DEV))
+    assert rel_err(out, ref) < 1e-5
+    assert torch.equal(hd.cpu(), h)  # a row list never writes the residual
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_silu_mul(dtype):
+    g = torch.Generator().manual_seed(4)
+    n, inter = 5, 200
+    gu = (torch.randn(n, 2 * inter, generator=g) * 4).to(dtype)
+    gate, up = gu[:, :inter].double(), gu[:, inter:].double()
+    ref = gate / (1 + torch.exp(-gate)) * up
+    out = torch.empty(n, inter, dtype=dtype, device=DEV)
+    ops().silu_mul(gu.to(DEV), out)
+    assert rel_err(out, ref) < (1e-6 if dtype == torch.float32 else 5e-3)
+    # gate = 0 gives 0 whatever the up value
+    z = torch.zeros(1, 2 * inter, dtype=dtype)
+    z[:, inter:] = 7
+    out1 = torch.empty(1, inter, dtype=dtype, device=DEV)
+    ops().silu_mul(z.to(DEV), out1)
+    assert float(out1.abs().max()) == 0.0
+
+
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("n,m,k", [(1, 200, 96), (7, 320, 200), (16, 64, 64), (17, 130, 50), (70, 257, 333)])
+def test_linear_f32(n, m, k):
+    g = torch.Generator().manual_seed(5)
+    x, w, b = torch.randn(n, k, generator=g), torch.randn(m, k, generator=g), torch.randn(m, generator=g)
+    out = torch.empty(n, m, dtype=torch.float32, device=DEV)
+    ops().linear_f32(x.to(DEV), w.to(DEV), b.to(DEV), out)
+    assert rel_err(out, x.double() @ w.double().t() + b.double()) < 2e-6
+    out2 = torch.empty(n, m, dtype=torch.float32, device=DEV)
+    ops().linear_f32(x.to(DEV), w.to(DEV), None, out2)
+    assert rel_err(out2, x.double() @ w.double().t()) < 2e-6
+
+
+def test_linear_f32_is_true_fp32_and_batch_invariant():
+    """Values that a reduced-precision matrix mode would lose; and a row's result must not depend on the batch."""
+    g = torch.Generator().manual_seed(6)
+    k, m = 512, 96
+    x = torch.randn(40, k, generator=g) * (1 + 2.0 ** -12)
+    w = torch.randn(m, k, generator=g)
+    big = torch.empty(40, m, dtype=torch.float32, device=DEV)
+    ops().linear_f32(x.to(DEV), w.to(DEV), None, big)
+    assert rel_err(big, x.double() @ w.double().t()) < 2e-6  # tf32/bf16 products would be near 1e-3
+    one = torch.empty(1, m, dtype=torch.float32, device=DEV)
+    ops().linear_f32(x[11:12].to(DEV).contiguous(), w.to(DEV), None, one)
+    assert torch.equal(one[0], big[11])
+
+
+@pytest.mark.parametrize("n", [1, 3, 16, 17, 33, 64, 100])
+@pytest.mark.parametrize("m,k", [(320, 96), (200, 200), (1030, 3584), (96, 18944 // 8)])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+def test_linear_bf16(n, m, k, out_dtype):
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(n, k, generator=g).to(torch.bfloat16)
+    w = (torch.randn(m, k, generator=g) * 0.05).to(torch.bfloat16)
+    b = torch.randn(m, generator=g)
+    ref = x.double() @ w.double().t() + b.double()
+    out = torch.empty(n, m, dtype=out_dtype, device=DEV)
+    ops().linear_bf16(x.to(DEV), w.to(DEV), b.to(DEV), out)
+    assert rel_err(out, ref) < (2e-5 if out_dtype == torch.float32 else 5e-3)
+
+
+def test_linear_bf16_odd_k_uses_plain_kernel():
+    g = torch.Generator().manual_seed(8)
+    n, m, k = 5, 70, 53
+    x = torch.randn(n, k, generator=g).to(torch.bfloat16)
+    w = torch.randn(m, k, generator=g).to(torch.bfloat16)
+    out = torch.empty(n, m, dtype=torch.float32, device=DEV)
+    ops().linear_bf16(x.to(DEV), w.to(DEV), None, out)
+    assert rel_err(out, x.double() @ w.double().t()) < 2e-5
+
+
+def test_linear_bf16_batch_invariant():
+    g = torch.Generator().manual_seed(9)
+    m, k = 640, 1536
+    x = torch.randn(64, k, generator=g).to(torch.bfloat16).to(DEV)
+    w = (torch.randn(m, k, generator=g) * 0.05).to(torch.bfloat16).to(DEV)
+    full = torch.empty(64, m, dtype=torch.float32, device=DEV)
+    ops().linear_bf16(x, w, None, full)
+    for rows in ([5], [0, 63], list(range(20, 37))):
+        sub = torch.empty(len(rows), m, dtype=torch.float32, device=DEV)
+        ops().linear_bf16(x[rows].contiguous(), w, None, sub)
+        assert torch.equal(sub, full[rows]), rows
+
+
+@pytest.mark.parametrize("n", [1, 9, 40, 64])
+@pytest.mark.parametrize("inter,k", [(200, 96), (128, 64), (1184, 3584)])
+def test_gated_linear_bf16(n, inter, k):
+    g = torch.Generator().manual_seed(10)
+    x = torch.randn(n, k, generator=g).to(torch.bfloat16)
+    w = (torch.randn(2 * inter, k, generator=g) * 0.05).to(torch.bfloat16)
+    gate = x.double() @ w[:inter].double().t()
+    up = x.double() @ w[inter:].double().t()
+    ref = gate / (1 + torch.exp(-gate)) * up
+    out = torch.empty(n, inter, dtype=torch.bfloat16, device=DEV)
+    ops().gated_linear_bf16(x.to(DEV), w.to(DEV), out)
+    assert rel_err(out, ref) < 6e-3
+    out32 = torch.empty(n, inter, dtype=torch.float32, device=DEV)
+    ops().gated_linear_bf16(x.to(DEV), w.to(DEV), out32)
+    assert rel_err(out32, ref) < 3e-5
+
+
+# ---------------------------------------------------------------------------
+# paged cache helpers
+# ---------------------------------------------------------------------------
+def make_pages(k, v, lens, page_size, dtype, seed, extra_pages=3):
+    """k, v: lists of [T_e, KVH, D] per entry.  Pages in shuffled order.  Returns k_pages, v_pages, block_table."""
+    kvh, d = k[0].shape[1], k[0].shape[2]
+    n_blocks = [-(-t // page_size) for t in lens]
+    total = sum(n_blocks) + extra_pages
+    perm = np.random.RandomState(seed).permutation(total)
+    kp = torch.full((total, kvh, page_size, d), 1e4, dtype=torch.float32)   # unwritten slots hold a large finite value
+    vp = torch.full((total, kvh, d, page_size), -1e4, dtype=torch.float32)
+    bt = torch.full((len(lens), max(n_blocks) + 2), -1, dtype=torch.int32)
+    nxt = 0
+    for e, t in enumerate(lens):
+        for b in range(n_blocks[e]):
+            pg = int(perm[nxt]); nxt += 1
+            bt[e, b] = pg
+            lo, hi = b * page_size, min(t, (b + 1) * page_size)
+            kp[pg, :, : hi - lo, :] = k[e][lo:hi].permute(1, 0, 2)
+            vp[pg, :, :, : hi - lo] = v[e][lo:hi].permute(1, 2, 0)
+    return kp.to(dtype), vp.to(dtype), bt
+
+
+def ref_attention(q, k, v, pos, window, scale):
+    """q [NH, D] at position pos against k, v [T, KVH, D]; float64."""
+    nh, d = q.shape
+    kvh = k.shape[1]
+    out = torch.zeros(nh, d, dtype=torch.float64)
+    lo = max(0, pos - window + 1) if window > 0 else 0
+    for h in range(nh):
+        kk, vv = k[lo:pos + 1, h // (nh // kvh)].double(), v[lo:pos + 1, h // (nh // kvh)].double()
+        s = (kk @ q[h].double()) * scale
+        p = torch.softmax(s, dim=0)
+        out[h] = p @ vv
+    return out
+
+
+def attention_case(dtype, nh, kvh, d, page_size, window, entries, seed, spike=False):
+    """entries: list of (cached tokens, new tokens).  Returns (got, ref) as [N, NH*D]."""
+    o = ops()
+    g = torch.Generator().manual_seed(seed)
+    lens = [c + n for c, n in entries]
+    ks = [torch.randn(t, kvh, d, generator=g) for t in lens]
+    vs = [torch.randn(t, kvh, d, generator=g) for t in lens]
+    qs = [torch.randn(n, nh, d, generator=g) for _, n in entries]
+    if spike:
+        # one far key that the query must find: its score stands out among hundreds
+        for e, (c, n) in enumerate(entries):
+            far = 3 if window == 0 else max(0, lens[e] - window)  # the oldest key the last token may still see
+            ks[e][far] *= 0
+            ks[e][far, :, 0] = 30.0
+            qs[e][-1] *= 0
+            qs[e][-1, :, 0] = 30.0 * math.sqrt(d) / 30.0 * 2.0
+            vs[e][far] = 5.0
+    if dtype == torch.bfloat16:
+        ks, vs, qs = ([t.to(torch.bfloat16).float() for t in x] for x in (ks, vs, qs))
+    kp, vp, bt = make_pages(ks, vs, lens, page_size, dtype, seed)
+    n_tok = sum(n for _, n in entries)
+    q = torch.cat(qs).reshape(n_tok, nh * d).to(dtype).to(DEV)
+    positions = torch.tensor([c + i for c, n in entries for i in range(n)], dtype=torch.int32)
+    tok_entry = torch.tensor([e for e, (c, n) in enumerate(entries) for _ in range(n)], dtype=torch.int32)
+    out = torch.empty(n_tok, nh * d, dtype=dtype, device=DEV)
+    scale = 1.0 / math.sqrt(d)
+    if dtype == torch.float32:
+        o.attention_f32(q, kp.to(DEV), vp.to(DEV), positions.to(DEV), tok_entry.to(DEV), bt.to(DEV), out, nh, kvh, d,
+                        window, scale)
+    else:
+        from vt_transformer_amd.engine.step import plan_attention_items
+        start = np.cumsum([0] + [n for _, n in entries]).astype(np.int32)
+        pos0 = np.array([c for c, _ in entries], dtype=np.int32)
+        for target in (2048, 10 ** 9):   # without and with the keys split over several items
+            items, citems, n_parts = plan_attention_items(start, pos0, nh // kvh, window, kvh, target_waves=target,
+                                                          min_chunk=16)
+            part_o = torch.full((max(1, n_parts) * kvh * 16 * d,), float("nan"), device=DEV)
+            part_ml = torch.full((max(1, n_parts) * kvh * 32,), float("nan"), device=DEV)
+            out.fill_(float("nan"))
+            o.attention_bf16(q, kp.to(DEV), vp.to(DEV), bt.to(DEV), torch.from_numpy(items).to(DEV).reshape(-1),
+                             items.shape[0], torch.from_numpy(citems).to(DEV).reshape(-1) if len(citems) else None,
+                             len(citems), out, part_o, part_ml, nh, kvh, d, window, scale, max_part=n_parts)
+            if target == 2048:
+                first = out.clone()
+        assert rel_err(out, first) < 1e-2  # split and unsplit agree to rounding
+    ref = torch.cat([ref_attention(qs[e][i], ks[e], vs[e], c + i, window, scale).reshape(1, -1)
+                     for e, (c, n) in enumerate(entries) for i in range(n)])
+    return out, ref
+
+
+ATT_TOL = {torch.float32: 1e-5, torch.bfloat16: 1.5e-2}
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nh,kvh,d", [(4, 2, 16), (3, 3, 32), (5, 1, 48), (14, 2, 64), (7, 7, 80), (28, 4, 128), (2, 1, 256)])
+def test_attention_mixed_batch(dtype, nh, kvh, d):
+    # a whole prompt, a decoded token with a long cache, a portion in the middle of a prompt, a first token
+    entries = [(0, 37), (300, 1), (45, 19), (0, 1), (16, 2)]
+    got, ref = attention_case(dtype, nh, kvh, d, 16, 0, entries, seed=nh * 100 + d)
+    assert rel_err(got, ref) < ATT_TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("page_size", [16, 32, 64])
+def test_attention_page_sizes_and_edges(dtype, page_size):
+    # lengths that end exactly on, one before and one after a page's edge
+    entries = [(page_size - 1, 1), (page_size, 1), (page_size + 1, 1), (2 * page_size - 1, 3), (0, 2 * page_size)]
+    got, ref = attention_case(dtype, 6, 2, 32, page_size, 0, entries, seed=page_size)
+    assert rel_err(got, ref) < ATT_TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("window", [1, 5, 16, 40])
+def test_attention_window_edge(dtype, window):
+    entries = [(0, 70), (130, 1), (window, 1), (window - 1, 1) if window > 1 else (0, 1), (20, 30)]
+    got, ref = attention_case(dtype, 4, 2, 32, 16, window, entries, seed=window, spike=True)
+    assert rel_err(got, ref) < ATT_TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_far_key_among_hundreds(dtype):
+    entries = [(700, 1), (0, 600), (513, 7)]
+    got, ref = attention_case(dtype, 8, 2, 64, 16, 0, entries, seed=77, spike=True)
+    assert rel_err(got, ref) < ATT_TOL[dtype]
+    # the spiked key carries almost all the weight: output of the last token of entry 0 is its value
+    assert abs(float(got[0, 0]) - 5.0) < 0.1
+
+
+def test_attention_fp32_one_key_is_value_row_and_zero_query_is_mean():
+    o = ops()
+    g = torch.Generator().manual_seed(11)
+    nh, kvh, d, t = 2, 1, 16, 9
+    k = [torch.randn(t, kvh, d, generator=g)]
+    v = [torch.randn(t, kvh, d, generator=g)]
+    kp, vp, bt = make_pages(k, v, [t], 16, torch.float32, 5)
+    q = torch.zeros(t, nh * d, device=DEV)
+    out = torch.empty(t, nh * d, device=DEV)
+    pos = torch.arange(t, dtype=torch.int32, device=DEV)
+    o.attention_f32(q, kp.to(DEV), vp.to(DEV), pos, torch.zeros(t, dtype=torch.int32, device=DEV), bt.to(DEV), out, nh,
+                    kvh, d, 0, 0.25)
+    out = out.cpu().reshape(t, nh, d)
+    assert torch.allclose(out[0, 0], v[0][0, 0], atol=1e-6)             # one key: the value row itself
+    assert torch.allclose(out[5, 1], v[0][:6, 0].mean(0), atol=1e-6)    # zero query: mean of the allowed values
+
+
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nh,kvh,d,page_size", [(4, 2, 16, 16), (5, 1, 48, 32), (28, 4, 128, 16)])
+def test_rope_store(dtype, nh, kvh, d, page_size):
+    from vt_transformer_amd.parts.rotary import rotary_table
+    o = ops()
+    g = torch.Generator().manual_seed(12)
+    theta = 10000.0
+    entries = [(0, 20), (33, 1), (page_size - 1, 3)]
+    n = sum(x[1] for x in entries)
+    width = (nh + 2 * kvh) * d
+    qkv = torch.randn(n, width, generator=g)
+    positions = torch.tensor([c + i for c, m in entries for i in range(m)], dtype=torch.int32)
+    tok_entry = torch.tensor([e for e, (c, m) in enumerate(entries) for _ in range(m)], dtype=torch.int32)
+    lens = [c + m for c, m in entries]
+    n_pages = sum(-(-t // page_size) for t in lens) + 2
+    perm = np.random.RandomState(3).permutation(n_pages)
+    bt = torch.full((len(entries), 8), -1, dtype=torch.int32)
+    nxt = 0
+    for e, t in enumerate(lens):
+        for b in range(-(-t // page_size)):
+            bt[e, b] = int(perm[nxt]); nxt += 1
+    cos, sin = rotary_table(64, d, theta)
+    kp = torch.zeros(n_pages, kvh, page_size, d, dtype=dtype, device=DEV)
+    vp = torch.zeros(n_pages, kvh, d, page_size, dtype=dtype, device=DEV)
+    q_out = torch.empty(n, nh * d, dtype=dtype, device=DEV)
+    o.rope_store(qkv.to(DEV), torch.from_numpy(cos).to(DEV), torch.from_numpy(sin).to(DEV), positions.to(DEV),
+                 tok_entry.to(DEV), bt.to(DEV), q_out, kp, vp, nh, kvh, d)
+    # reference: rotate-half pairs (i, i + d/2), float64 angles
+    i = torch.arange(0, d, 2, dtype=torch.float64)
+    ang = positions.double()[:, None] / torch.pow(torch.tensor(theta, dtype=torch.float64), i / d)[None, :]
+    c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+
+    def rot(x):
+        x1, x2 = x[..., : d // 2].double(), x[..., d // 2:].double()
+        return torch.cat([c * x1 - s * x2, c * x2 + s * x1], -1)
+    q_ref = rot(qkv[:, : nh * d].reshape(n, nh, d)).reshape(n, nh * d)
+    k_ref = rot(qkv[:, nh * d:(nh + kvh) * d].reshape(n, kvh, d))
+    v_ref = qkv[:, (nh + kvh) * d:].reshape(n, kvh, d).double()
+    tol = 2e-6 if dtype == torch.float32 else 5e-3
+    assert rel_err(q_out, q_ref) < tol
+    kp, vp = kp.cpu().double(), vp.cpu().double()
+    for t in range(n):
+        e, p = int(tok_entry[t]), int(positions[t])
+        pg, slot = int(bt[e, p // page_size]), p % page_size
+        assert rel_err(kp[pg, :, slot, :], k_ref[t]) < tol
+        assert rel_err(vp[pg, :, :, slot], v_ref[t]) < tol
+    # nothing else was written
+    written = torch.zeros(n_pages, page_size, dtype=torch.bool)
+    for t in range(n):
+        e, p = int(tok_entry[t]), int(positions[t])
+        written[int(bt[e, p // page_size]), p % page_size] = True
+    assert float(kp.abs().sum(dim=(1, 3))[~written].sum()) == 0.0
+
+
+# ---------------------------------------------------------------------------
+def test_sample_greedy_lowest_index_on_ties():
+    o = ops()
+    v = 1003
+    logits = torch.zeros(3, v)
+    logits[0, [17, 500, 900]] = 4.0
+    logits[1, v - 1] = 1.0
+    logits[2] = -1.0
+    out = torch.empty(3, dtype=torch.int32, device=DEV)
+    o.sample(logits.to(DEV), torch.zeros(3, device=DEV), torch.full((3,), -1, dtype=torch.int32, device=DEV),
+             torch.ones(3, device=DEV), torch.rand(3).to(DEV), torch.empty(3 * v, device=DEV), out)
+    assert out.cpu().tolist() == [17, v - 1, 0]
+
+
+def _draw(logits_row, temperature, top_k, top_p, n_draws, seed):
+    o = ops()
+    v = logits_row.numel()
+    logits = logits_row.reshape(1, v).repeat(n_draws, 1).to(DEV)
+    u = torch.rand(n_draws, generator=torch.Generator().manual_seed(seed)).to(DEV)
+    out = torch.empty(n_draws, dtype=torch.int32, device=DEV)
+    o.sample(logits, torch.full((n_draws,), temperature, device=DEV),
+             torch.full((n_draws,), top_k, dtype=torch.int32, device=DEV), torch.full((n_draws,), top_p, device=DEV),
+             u, torch.empty(n_draws * v, device=DEV), out)
+    return out.cpu().long()
+
+
+def test_sample_frequencies_match_softmax():
+    g = torch.Generator().manual_seed(13)
+    v = 37
+    logits = torch.randn(v, generator=g) * 2
+    n = 40000
+    for temp in (0.7, 1.5):
+        draws = _draw(logits, temp, -1, 1.0, n, seed=int(temp * 10))
+        freq = torch.bincount(draws, minlength=v).double() / n
+        p = torch.softmax(logits.double() / temp, 0)
+        assert float((freq - p).abs().max()) < 4 * math.sqrt(0.25 / n) + 1e-3
+
+
+def test_sample_top_k_and_top_p():
+    g = torch.Generator().manual_seed(14)
+    v = 500
+    logits = torch.randn(v, generator=g) * 3
+    p = torch.softmax(logits.double(), 0)
+    order = torch.argsort(p, descending=True)
+    draws = _draw(logits, 1.0, 3, 1.0, 5000, 1)          # the reference's own stochastic mode: the top three
+    assert set(draws.tolist()) <= set(order[:3].tolist())
+    freq = torch.bincount(draws, minlength=v).double()[order[:3]] / 5000
+    assert float((freq - p[order[:3]] / p[order[:3]].sum()).abs().max()) < 0.03
+    draws = _draw(logits, 1.0, -1, 0.5, 5000, 2)
+    cum = torch.cumsum(p[order], 0)
+    keep = int((cum < 0.5).sum()) + 1
+    assert set(draws.tolist()) <= set(order[:keep].tolist())
+    assert len(set(draws.tolist())) == keep or keep > 20
+    # temperature towards zero is the argmax
+    assert set(_draw(logits, 1e-4, -1, 1.0, 100, 3).tolist()) == {int(order[0])}
+    # top_k = 1 is greedy whatever the temperature
+    assert set(_draw(logits, 5.0, 1, 1.0, 100, 4).tolist()) == {int(order[0])}

@@ -1,0 +1,100 @@
+// Shared helpers of the gfx950 kernels: bf16 conversion, wave and block
+// reductions for 64-wide wavefronts, launch checking.
+//
+// Every entry point is extern "C", takes raw device pointers and a stream,
+// launches on that stream and returns 0, or a negative code after writing a
+// message that vt_last_error() hands out.  Shapes are validated on the host
+// before a launch; no kernel reads outside what its arguments describe.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#define VT_WAVE 64
+
+// activation / weight element types
+#define VT_F32 0
+#define VT_BF16 1
+
+typedef uint16_t bf16_t;  // raw bits
+
+// One library = one translation unit, so the error text lives here.
+static char vt_err_buf_[512] = "";
+static int vt_fail(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(vt_err_buf_, sizeof(vt_err_buf_), fmt, ap);
+    va_end(ap);
+    return -1;
+}
+// Each library's source file invokes this once.
+#define VT_DEFINE_LAST_ERROR() \
+    extern "C" const char* vt_last_error() { return vt_err_buf_; }
+
+#define VT_CHECK_LAUNCH(name)                                              \
+    do {                                                                   \
+        hipError_t e_ = hipGetLastError();                                 \
+        if (e_ != hipSuccess) return vt_fail("%s: launch failed: %s", name, hipGetErrorString(e_)); \
+    } while (0)
+
+#define VT_REQUIRE(cond, ...)                   \
+    do {                                        \
+        if (!(cond)) return vt_fail(__VA_ARGS__); \
+    } while (0)
+
+__device__ __forceinline__ float bf16_to_f32(bf16_t v) {
+    return __uint_as_float(((uint32_t)v) << 16);
+}
+
+// round to nearest even; NaN stays NaN
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (bf16_t)(u >> 16);
+}
+
+template <typename T> __device__ __forceinline__ float load_f32(const T* p, size_t i);
+template <> __device__ __forceinline__ float load_f32<float>(const float* p, size_t i) { return p[i]; }
+template <> __device__ __forceinline__ float load_f32<bf16_t>(const bf16_t* p, size_t i) { return bf16_to_f32(p[i]); }
+
+template <typename T> __device__ __forceinline__ void store_f32(T* p, size_t i, float v);
+template <> __device__ __forceinline__ void store_f32<float>(float* p, size_t i, float v) { p[i] = v; }
+template <> __device__ __forceinline__ void store_f32<bf16_t>(bf16_t* p, size_t i, float v) { p[i] = f32_to_bf16(v); }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+
+// Block reductions for blockDim.x a multiple of 64, up to 1024.  `red` is
+// shared memory of at least 16 floats.  The order of the additions depends
+// only on blockDim.x, so a row's sum does not depend on what else is in the
+// launch.
+__device__ __forceinline__ float block_sum(float v, float* red) {
+    v = wave_sum(v);
+    int w = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[w] = v;
+    __syncthreads();
+    float t = 0.f;
+    for (int i = 0; i < nw; ++i) t += red[i];
+    return t;
+}
+__device__ __forceinline__ float block_max(float v, float* red) {
+    v = wave_max(v);
+    int w = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[w] = v;
+    __syncthreads();
+    float t = red[0];
+    for (int i = 1; i < nw; ++i) t = fmaxf(t, red[i]);
+    return t;
+}

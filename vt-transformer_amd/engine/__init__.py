@@ -1,0 +1,5 @@
+from .step import ModelRunner, OutOfPages, StepContext, StepEntry, plan_attention_items
+from .loading import build_model, load_model, make_runner, parse_dtype, random_model
+
+__all__ = ["ModelRunner", "OutOfPages", "StepContext", "StepEntry", "plan_attention_items", "build_model",
+           "load_model", "make_runner", "parse_dtype", "random_model"]

@@ -1,0 +1,257 @@
+"""The step function: run a batch of (request, its next tokens) from the
+cache and return logits at the wanted places.
+
+A step holds any mixture of portions of prompts and single decoded tokens,
+as one flat list of tokens without padding.  The reference's step
+(EngineBase::forward, vt-transformer/core/vt_engine.hpp:34-37, 66) takes a
+batch that is all-prefill or all-decode (:16-22) and returns one sampled
+token per request; its older engine pads a rectangular [B, T] block
+(v1/tensortype/nn_kvcache.cpp:346-420).  Here positions are
+start + i as there (nn_kvcache.cpp:444-448), logits come back instead of
+tokens, and sampling sits above.
+
+Per step the host builds, in one int32 buffer that goes to the device in one
+copy: token ids, positions, the entry of each token, entry starts, state
+slots, the rows whose logits are wanted, and one block table per group of
+layers.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, Hashable, List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+from ..cache.pages import NO_PAGE, CacheError
+from ..cache.storage import CacheStorage
+from ..kernels.ops import ATTN_CITEM_INTS, ATTN_ITEM_INTS
+from ..parts.base import Runtime
+
+
+class OutOfPages(RuntimeError):
+    """The step needs more pages than are free; nothing was changed."""
+
+
+@dataclass
+class StepEntry:
+    rid: Hashable             # a request admitted to the cache manager
+    tokens: Sequence[int]     # its next tokens (>= 1)
+    want: Sequence[int] = ()  # places among these tokens whose logits are wanted
+
+
+@dataclass
+class AttentionPlan:
+    items: torch.Tensor
+    n_items: int
+    citems: Optional[torch.Tensor]
+    n_citems: int
+    part_o: Optional[torch.Tensor]
+    part_ml: Optional[torch.Tensor]
+    n_parts: int
+
+
+def plan_attention_items(entry_start: np.ndarray, entry_pos0: np.ndarray, group: int, window: int, n_kv: int,
+                         target_waves: int = 2048, min_chunk: int = 64) -> Tuple[np.ndarray, np.ndarray, int]:
+    """Work items of the bf16 attention kernel for one step.
+
+    Rows of an entry are (token, query head of a kv group) pairs, token-major; a tile is 16 rows.  Each tile
+    needs keys [key_lo, key_hi).  When the tiles are too few to fill the GPU, a tile's keys are cut at absolute
+    multiples of a chunk length into several items whose partial results a second kernel merges.
+    Returns (items [n, 8], combine items [m, 6], number of partial slots)."""
+    n_entries = len(entry_pos0)
+    q_len = (entry_start[1:] - entry_start[:-1]).astype(np.int64)
+    rows = q_len * group
+    n_tiles = (rows + 15) // 16
+    total = int(n_tiles.sum())
+    if total == 0:
+        return np.zeros((0, ATTN_ITEM_INTS), np.int32), np.zeros((0, ATTN_CITEM_INTS), np.int32), 0
+    ent = np.repeat(np.arange(n_entries), n_tiles)
+    first = np.cumsum(n_tiles) - n_tiles
+    tile_in_entry = np.arange(total) - np.repeat(first, n_tiles)
+    row0 = tile_in_entry * 16
+    e_rows, e_len, e_pos0, e_start = rows[ent], q_len[ent], entry_pos0[ent].astype(np.int64), entry_start[:-1][ent].astype(np.int64)
+    t_first = row0 // group
+    t_last = np.minimum(e_rows - 1, row0 + 15) // group
+    min_p, max_p = e_pos0 + t_first, e_pos0 + t_last
+    lo = np.maximum(0, min_p - window + 1) if window > 0 else np.zeros_like(min_p)
+    key_lo = (lo // 16) * 16
+    key_hi = max_p + 1
+    span = key_hi - key_lo
+    # split keys only if the tiles alone leave most of the GPU idle
+    chunk = 0
+    if total * n_kv < target_waves // 2:
+        keys_total = int(span.sum()) * n_kv
+        chunk = max(min_chunk, -(-keys_total // target_waves))
+        chunk = -(-chunk // 16) * 16
+        if chunk >= int(span.max()):
+            chunk = 0
+    if chunk == 0:
+        items = np.stack([ent, e_start, e_len, e_pos0, row0, key_lo, key_hi, np.full(total, -1)], axis=1)
+        return items.astype(np.int32), np.zeros((0, ATTN_CITEM_INTS), np.int32), 0
+    c_first = key_lo // chunk
+    c_last = (key_hi - 1) // chunk
+    n_parts = (c_last - c_first + 1)
+    tot_parts = int(n_parts.sum())
+    tile_of = np.repeat(np.arange(total), n_parts)
+    p_first = np.cumsum(n_parts) - n_parts
+    c_idx = np.arange(tot_parts) - np.repeat(p_first, n_parts) + c_first[tile_of]
+    p_lo = np.maximum(key_lo[tile_of], c_idx * chunk)
+    p_hi = np.minimum(key_hi[tile_of], (c_idx + 1) * chunk)
+    single = (n_parts == 1)[tile_of]
+    part_id = np.where(single, -1, np.arange(tot_parts))
+    items = np.stack([ent[tile_of], e_start[tile_of], e_len[tile_of], e_pos0[tile_of], row0[tile_of], p_lo, p_hi,
+                      part_id], axis=1).astype(np.int32)
+    multi = np.nonzero(n_parts > 1)[0]
+    citems = np.stack([e_start[multi], e_len[multi], row0[multi], p_first[multi], n_parts[multi],
+                       np.zeros(len(multi), np.int64)], axis=1).astype(np.int32)
+    return items, citems, tot_parts
+
+
+class StepContext:
+    """Everything the parts may read about the step, on host and device."""
+
+    def __init__(self, rt: Runtime, n_positions: int):
+        self.rt = rt
+        self.n_positions = int(n_positions)   # positions are below this (size of position tables)
+        self.n_tokens = 0
+        self.n_entries = 0
+        self.n_logit_rows = 0
+        # host arrays (numpy int32)
+        self.h_token_ids = self.h_positions = self.h_tok_entry = None
+        self.h_entry_start = self.h_entry_pos0 = self.h_state_slots = self.h_logit_rows = None
+        self.h_block_tables: List[np.ndarray] = []
+        # device views
+        self.token_ids = self.positions = self.tok_entry = None
+        self.entry_start = self.entry_pos0 = self.state_slots = self.logit_rows = None
+        self.block_tables: List[torch.Tensor] = []
+        self.fresh: List[bool] = []           # per entry: the request's first step (its state slot was just cleared)
+        self._plans: Dict[Tuple[int, int, int, int], AttentionPlan] = {}
+
+    def attention_plan(self, group: int, window: int, n_kv: int, head_dim: int) -> AttentionPlan:
+        key = (group, window, n_kv, head_dim)
+        plan = self._plans.get(key)
+        if plan is None:
+            plan = self._make_plan(key)
+            self._plans[key] = plan
+        return plan
+
+    def _make_plan(self, key) -> AttentionPlan:
+        group, window, n_kv, head_dim = key
+        items, citems, n_parts = plan_attention_items(self.h_entry_start, self.h_entry_pos0, group, window, n_kv)
+        rt = self.rt
+        tag = f"attnplan.{group}.{window}.{n_kv}.{head_dim}"
+        flat = np.concatenate([items.reshape(-1), citems.reshape(-1)])
+        dev = rt.buffer(tag, (max(flat.size, 1),), torch.int32)
+        if flat.size:
+            dev[:flat.size].copy_(torch.from_numpy(flat))
+        d_items = dev[:items.size]
+        d_citems = dev[items.size:items.size + citems.size] if citems.size else None
+        part_o = part_ml = None
+        if n_parts:
+            part_o = rt.buffer("attn.part_o", (n_parts * n_kv * 16 * head_dim,), torch.float32)
+            part_ml = rt.buffer("attn.part_ml", (n_parts * n_kv * 16 * 2,), torch.float32)
+        return AttentionPlan(d_items, items.shape[0], d_citems, citems.shape[0], part_o, part_ml, n_parts)
+
+
+class ModelRunner:
+    """Owns the model, its cache and the step function."""
+
+    def __init__(self, model, rt: Runtime, page_size: int, pool_tokens: int, max_requests: int, max_seq_len: int):
+        self.model = model
+        self.rt = rt
+        self.max_seq_len = int(max_seq_len)
+        self.storage = CacheStorage(rt, model, page_size, pool_tokens, max_requests, max_seq_len)
+        self.cache = self.storage.manager
+        self.vocab_size = model.spec.vocab_size
+        self.steps = 0
+        self.tokens = 0
+
+    # -- requests -----------------------------------------------------------
+    def admit(self, rid: Hashable) -> bool:
+        return self.cache.admit(rid) is not None
+
+    def release(self, rid: Hashable) -> None:
+        self.cache.release(rid)
+
+    # -- the step -----------------------------------------------------------
+    def build_context(self, entries: Sequence[StepEntry]) -> StepContext:
+        cache, ps = self.cache, self.cache.page_size
+        n_entries = len(entries)
+        lens = np.array([len(e.tokens) for e in entries], dtype=np.int64)
+        if n_entries == 0 or (lens <= 0).any():
+            raise ValueError("a step needs at least one entry and every entry at least one token")
+        n = int(lens.sum())
+        rps = [cache.get(e.rid) for e in entries]
+        pos0 = np.array([rp.length for rp in rps], dtype=np.int64)
+        start = np.zeros(n_entries + 1, dtype=np.int64)
+        np.cumsum(lens, out=start[1:])
+        tok_entry = np.repeat(np.arange(n_entries), lens)
+        positions = np.arange(n) - start[:-1][tok_entry] + pos0[tok_entry]
+        ids = np.fromiter((t for e in entries for t in e.tokens), dtype=np.int64, count=n)
+        if ids.size and (ids.min() < 0 or ids.max() >= self.vocab_size):
+            bad = ids[(ids < 0) | (ids >= self.vocab_size)][0]
+            raise ValueError(f"token id {int(bad)} is outside the vocabulary of {self.vocab_size}")
+        rows = []
+        for i, e in enumerate(entries):
+            for w in e.want:
+                if not 0 <= w < lens[i]:
+                    raise ValueError(f"request {e.rid!r}: wanted place {w} is not among its {lens[i]} tokens")
+                rows.append(start[i] + w)
+        new_len = pos0 + lens
+        max_blocks = int(-(-new_len.max() // ps))
+        max_blocks = -(-max_blocks // 8) * 8
+        tables = []
+        for gi in range(self.storage.n_groups):
+            bt = np.full((n_entries, max_blocks), NO_PAGE, dtype=np.int32)
+            for i, rp in enumerate(rps):
+                t = rp.tables[gi]
+                bt[i, :len(t)] = t
+            tables.append(bt)
+
+        ctx = StepContext(self.rt, self.max_seq_len)
+        ctx.n_tokens, ctx.n_entries, ctx.n_logit_rows = n, n_entries, len(rows)
+        ctx.h_token_ids = ids.astype(np.int32)
+        ctx.h_positions = positions.astype(np.int32)
+        ctx.h_tok_entry = tok_entry.astype(np.int32)
+        ctx.h_entry_start = start.astype(np.int32)
+        ctx.h_entry_pos0 = pos0.astype(np.int32)
+        ctx.h_state_slots = np.array([rp.slot for rp in rps], dtype=np.int32)
+        ctx.h_logit_rows = np.array(rows, dtype=np.int32)
+        ctx.h_block_tables = tables
+        ctx.fresh = [rp.fresh for rp in rps]
+        parts = [ctx.h_token_ids, ctx.h_positions, ctx.h_tok_entry, ctx.h_entry_start, ctx.h_entry_pos0,
+                 ctx.h_state_slots, ctx.h_logit_rows] + [t.reshape(-1) for t in tables]
+        flat = np.concatenate(parts)
+        dev = self.rt.buffer("step.meta", (flat.size,), torch.int32)
+        dev.copy_(torch.from_numpy(flat))
+        views, off = [], 0
+        for p in parts:
+            views.append(dev[off:off + p.size])
+            off += p.size
+        (ctx.token_ids, ctx.positions, ctx.tok_entry, ctx.entry_start, ctx.entry_pos0, ctx.state_slots,
+         ctx.logit_rows) = views[:7]
+        ctx.block_tables = [v.view(n_entries, max_blocks) for v in views[7:]]
+        return ctx
+
+    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        """Run the entries' tokens as one batch.  Returns fp32 logits [wanted places, vocab] on the device in the
+        order of the entries and of their `want`, or None if nothing is wanted.  Raises OutOfPages (with nothing
+        changed) if the cache cannot hold the new tokens."""
+        cache = self.cache
+        targets = [(e.rid, cache.get(e.rid).length + len(e.tokens)) for e in entries]
+        for rid, new_len in targets:
+            if new_len > self.max_seq_len:
+                raise CacheError(f"request {rid!r} would reach {new_len} tokens, the engine is set up for {self.max_seq_len}")
+        if not cache.reserve(targets):
+            raise OutOfPages(f"the step needs more pages than are free ({cache.available_pages()} free per group)")
+        fresh_slots = [cache.get(e.rid).slot for e in entries if cache.get(e.rid).fresh]
+        self.storage.clear_state(fresh_slots)
+        ctx = self.build_context(entries)
+        caches = self.storage.layer_caches(ctx.block_tables)
+        logits = self.model.forward(ctx, caches, self.storage.state)
+        for rid, new_len in targets:
+            cache.commit(rid, new_len)
+        self.steps += 1
+        self.tokens += ctx.n_tokens
+        return logits

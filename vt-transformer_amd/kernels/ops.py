@@ -1,0 +1,281 @@
+"""Python face of the HIP kernels.
+
+Every function checks on the host that the operands are what the kernel and
+its launch grid assume (device, dtype, contiguity, shapes) and raises
+before anything is launched otherwise.  A missing or unloadable library is an
+error, never a reason to compute some other way.
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+from typing import Optional
+
+import torch
+
+from .build import KernelBuildError, load_lib
+
+F32, BF16 = 0, 1
+_CODES = {torch.float32: F32, torch.bfloat16: BF16}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _code(t: torch.Tensor) -> int:
+    try:
+        return _CODES[t.dtype]
+    except KeyError:
+        raise KernelError(f"dtype {t.dtype} is not handled by the kernels (float32 and bfloat16 are)") from None
+
+
+def _chk(t: torch.Tensor, name: str, dtype=None, shape=None) -> None:
+    if not t.is_cuda:
+        raise KernelError(f"{name}: tensor is on {t.device}, the kernels run on the GPU only")
+    if not t.is_contiguous():
+        raise KernelError(f"{name}: tensor is not contiguous")
+    if dtype is not None and t.dtype != dtype:
+        raise KernelError(f"{name}: dtype {t.dtype}, expected {dtype}")
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        raise KernelError(f"{name}: shape {tuple(t.shape)}, expected {tuple(shape)}")
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return ctypes.c_void_p(t.data_ptr() if t is not None else 0)
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _run(lib, fn: str, *args) -> None:
+    rc = getattr(lib, fn)(*args)
+    if rc != 0:
+        raise KernelError(lib.vt_last_error().decode("utf-8", "replace"))
+
+
+def _i(v) -> ctypes.c_int:
+    return ctypes.c_int(int(v))
+
+
+def _f(v) -> ctypes.c_float:
+    return ctypes.c_float(float(v))
+
+
+# ---------------------------------------------------------------------------
+def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    n = ids.numel()
+    vocab, hidden = table.shape
+    _chk(table, "embed.table")
+    _chk(ids, "embed.ids", torch.int32)
+    _chk(out, "embed.out", torch.float32, (n, hidden))
+    _run(load_lib("vt_elementwise"), "vt_embed", _ptr(table), _i(_code(table)), _ptr(ids), _ptr(out), _i(n), _i(hidden),
+         _i(vocab), _stream())
+    return out
+
+
+def rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], gain: torch.Tensor, out: torch.Tensor, eps: float,
+            rows: Optional[torch.Tensor] = None, update_h: bool = True) -> torch.Tensor:
+    """out[r] = gain * x / sqrt(mean(x^2) + eps), x = h[row] + delta[row]; with update_h the sum is written back to h."""
+    hidden = h.shape[-1]
+    _chk(h, "rmsnorm.h", torch.float32)
+    _chk(gain, "rmsnorm.gain", torch.float32, (hidden,))
+    if delta is not None:
+        _chk(delta, "rmsnorm.delta", None, h.shape)
+    if rows is not None:
+        _chk(rows, "rmsnorm.rows", torch.int32)
+        n_out = rows.numel()
+        update_h = False
+    else:
+        n_out = h.shape[0]
+    _chk(out, "rmsnorm.out", None, (n_out, hidden))
+    _run(load_lib("vt_elementwise"), "vt_rmsnorm", _ptr(h), _ptr(delta), _i(_code(delta) if delta is not None else -1),
+         _ptr(gain), _ptr(out), _i(_code(out)), _ptr(rows), _i(n_out), _i(hidden), _f(eps),
+         _i(1 if (update_h and delta is not None) else 0), _stream())
+    return out
+
+
+def residual_add(h: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
+    _chk(h, "residual_add.h", torch.float32)
+    _chk(delta, "residual_add.delta", None, h.shape)
+    _run(load_lib("vt_elementwise"), "vt_residual_add", _ptr(h), _ptr(delta), _i(_code(delta)),
+         ctypes.c_longlong(h.numel()), _stream())
+    return h
+
+
+def silu_mul(gu: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    n, two_i = gu.shape
+    _chk(gu, "silu_mul.gu")
+    _chk(out, "silu_mul.out", None, (n, two_i // 2))
+    if two_i % 2:
+        raise KernelError(f"silu_mul: input width {two_i} is odd")
+    _run(load_lib("vt_elementwise"), "vt_silu_mul", _ptr(gu), _i(_code(gu)), _ptr(out), _i(_code(out)), _i(n),
+         _i(two_i // 2), _stream())
+    return out
+
+
+def gather_rows(x: torch.Tensor, rows: Optional[torch.Tensor], out: torch.Tensor) -> torch.Tensor:
+    _chk(x, "gather_rows.x")
+    n = rows.numel() if rows is not None else x.shape[0]
+    if rows is not None:
+        _chk(rows, "gather_rows.rows", torch.int32)
+    _chk(out, "gather_rows.out", None, (n, x.shape[1]))
+    _run(load_lib("vt_elementwise"), "vt_gather_rows", _ptr(x), _i(_code(x)), _ptr(rows), _ptr(out), _i(_code(out)),
+         _i(n), _i(x.shape[1]), _stream())
+    return out
+
+
+def rope_store(qkv: torch.Tensor, cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], positions: torch.Tensor,
+               tok_entry: torch.Tensor, block_table: Optional[torch.Tensor], q_out: torch.Tensor,
+               k_pages: Optional[torch.Tensor], v_pages: Optional[torch.Tensor], n_heads: int, n_kv: int, head_dim: int,
+               write_kv: bool = True) -> None:
+    """Rotate queries and keys by the tables' angles at `positions`, write the queries to q_out and, with
+    write_kv, keys and values into their pages ([page][kv][slot][D] and [page][kv][D][slot])."""
+    n = qkv.shape[0]
+    width = (n_heads + (2 * n_kv if write_kv else 0)) * head_dim
+    _chk(qkv, "rope_store.qkv")
+    if qkv.shape[1] < width:
+        raise KernelError(f"rope_store.qkv: {qkv.shape[1]} columns, need {width}")
+    _chk(positions, "rope_store.positions", torch.int32, (n,))
+    _chk(tok_entry, "rope_store.tok_entry", torch.int32, (n,))
+    _chk(q_out, "rope_store.q_out", None, (n, n_heads * head_dim))
+    rot = 0
+    max_pos = 0
+    if cos is not None:
+        _chk(cos, "rope_store.cos", torch.float32)
+        _chk(sin, "rope_store.sin", torch.float32, cos.shape)
+        max_pos, half = cos.shape
+        rot = 2 * half
+    page_size = num_pages = max_blocks = 0
+    if write_kv:
+        num_pages, kvh, page_size, d = k_pages.shape
+        if (kvh, d) != (n_kv, head_dim):
+            raise KernelError(f"rope_store.k_pages: shape {tuple(k_pages.shape)} does not fit kv heads {n_kv} x {head_dim}")
+        _chk(k_pages, "rope_store.k_pages", q_out.dtype)
+        _chk(v_pages, "rope_store.v_pages", q_out.dtype, (num_pages, n_kv, head_dim, page_size))
+        _chk(block_table, "rope_store.block_table", torch.int32)
+        max_blocks = block_table.shape[1]
+    _run(load_lib("vt_elementwise"), "vt_rope_store", _ptr(qkv), _i(_code(qkv)), ctypes.c_longlong(qkv.stride(0)),
+         _ptr(cos), _ptr(sin), _i(rot), _i(max_pos), _ptr(positions), _ptr(tok_entry), _ptr(block_table),
+         _i(max_blocks), _ptr(q_out), _ptr(k_pages), _ptr(v_pages), _i(_code(q_out)), _i(page_size), _i(num_pages),
+         _i(n), _i(n_heads), _i(n_kv), _i(head_dim), _i(1 if write_kv else 0), _stream())
+
+
+# ---------------------------------------------------------------------------
+def linear_f32(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor) -> torch.Tensor:
+    n, k = x.shape
+    m = w.shape[0]
+    _chk(x, "linear_f32.x", torch.float32)
+    _chk(w, "linear_f32.w", torch.float32, (m, k))
+    _chk(out, "linear_f32.out", torch.float32, (n, m))
+    if bias is not None:
+        _chk(bias, "linear_f32.bias", torch.float32, (m,))
+    _run(load_lib("vt_gemm_f32"), "vt_linear_f32", _ptr(x), _ptr(w), _ptr(bias), _ptr(out), _i(n), _i(m), _i(k), _stream())
+    return out
+
+
+def linear_bf16(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor) -> torch.Tensor:
+    """Few rows (decoding, short portions): W is read once per 64 rows."""
+    n, k = x.shape
+    m = w.shape[0]
+    _chk(x, "linear_bf16.x", torch.bfloat16)
+    _chk(w, "linear_bf16.w", torch.bfloat16, (m, k))
+    _chk(out, "linear_bf16.out", None, (n, m))
+    if bias is not None:
+        _chk(bias, "linear_bf16.bias", torch.float32, (m,))
+    _run(load_lib("vt_gemm_bf16"), "vt_linear_bf16", _ptr(x), _ptr(w), _ptr(bias), _ptr(out), _i(_code(out)), _i(n), _i(m),
+         _i(k), _stream())
+    return out
+
+
+def gated_linear_bf16(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    n, k = x.shape
+    two_i = w_gate_up.shape[0]
+    _chk(x, "gated_linear_bf16.x", torch.bfloat16)
+    _chk(w_gate_up, "gated_linear_bf16.w", torch.bfloat16, (two_i, k))
+    _chk(out, "gated_linear_bf16.out", None, (n, two_i // 2))
+    _run(load_lib("vt_gemm_bf16"), "vt_gated_linear_bf16", _ptr(x), _ptr(w_gate_up), _ptr(out), _i(_code(out)), _i(n),
+         _i(two_i // 2), _i(k), _stream())
+    return out
+
+
+# ---------------------------------------------------------------------------
+def attention_f32(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, positions: torch.Tensor,
+                  tok_entry: torch.Tensor, block_table: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int,
+                  head_dim: int, window: int, scale: float) -> torch.Tensor:
+    n = q.shape[0]
+    num_pages, kvh, page_size, d = k_pages.shape
+    _chk(q, "attention_f32.q", torch.float32, (n, n_heads * head_dim))
+    _chk(k_pages, "attention_f32.k_pages", torch.float32, (num_pages, n_kv, page_size, head_dim))
+    _chk(v_pages, "attention_f32.v_pages", torch.float32, (num_pages, n_kv, head_dim, page_size))
+    _chk(positions, "attention_f32.positions", torch.int32, (n,))
+    _chk(tok_entry, "attention_f32.tok_entry", torch.int32, (n,))
+    _chk(block_table, "attention_f32.block_table", torch.int32)
+    _chk(out, "attention_f32.out", torch.float32, (n, n_heads * head_dim))
+    _run(load_lib("vt_attn_f32"), "vt_attn_f32", _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(positions), _ptr(tok_entry),
+         _ptr(block_table), _ptr(out), _i(n), _i(n_heads), _i(n_kv), _i(head_dim), _i(page_size),
+         _i(block_table.shape[1]), _i(num_pages), _i(window), _f(scale), _stream())
+    return out
+
+
+ATTN_ITEM_INTS = 8
+ATTN_CITEM_INTS = 6
+
+
+def attention_bf16(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
+                   items: torch.Tensor, n_items: int, citems: Optional[torch.Tensor], n_citems: int, out: torch.Tensor,
+                   part_o: Optional[torch.Tensor], part_ml: Optional[torch.Tensor], n_heads: int, n_kv: int,
+                   head_dim: int, window: int, scale: float, max_part: int = 0) -> torch.Tensor:
+    """`items` [>=n_items, 8] int32: entry, q_tok0, q_len, pos0, q_row0, key_lo, key_hi, part (-1 = final).
+    `citems` [>=n_citems, 6] int32: q_tok0, q_len, q_row0, part0, n_parts, 0.  The planner (engine) makes them;
+    `max_part` is the number of partial slots it used, checked against the workspace here."""
+    n = q.shape[0]
+    num_pages, kvh, page_size, d = k_pages.shape
+    if head_dim % 16 or not 16 <= head_dim <= 256:
+        raise KernelError(f"attention_bf16: head size {head_dim} is not a multiple of 16 in 16..256")
+    _chk(q, "attention_bf16.q", torch.bfloat16, (n, n_heads * head_dim))
+    _chk(k_pages, "attention_bf16.k_pages", torch.bfloat16, (num_pages, n_kv, page_size, head_dim))
+    _chk(v_pages, "attention_bf16.v_pages", torch.bfloat16, (num_pages, n_kv, head_dim, page_size))
+    _chk(block_table, "attention_bf16.block_table", torch.int32)
+    _chk(items, "attention_bf16.items", torch.int32)
+    _chk(out, "attention_bf16.out", torch.bfloat16, (n, n_heads * head_dim))
+    if items.numel() < n_items * ATTN_ITEM_INTS:
+        raise KernelError("attention_bf16: item list shorter than n_items")
+    if n_citems:
+        _chk(citems, "attention_bf16.citems", torch.int32)
+        _chk(part_o, "attention_bf16.part_o", torch.float32)
+        _chk(part_ml, "attention_bf16.part_ml", torch.float32)
+        if citems.numel() < n_citems * ATTN_CITEM_INTS:
+            raise KernelError("attention_bf16: combine list shorter than n_citems")
+        if part_o.numel() < max_part * n_kv * 16 * head_dim or part_ml.numel() < max_part * n_kv * 16 * 2:
+            raise KernelError("attention_bf16: workspace for split keys is too small")
+    lib = load_lib("vt_attn_bf16", head_dim)
+    _run(lib, "vt_attn_bf16", _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(block_table), _ptr(items), _i(n_items),
+         _ptr(citems), _i(n_citems), _ptr(out), _ptr(part_o), _ptr(part_ml), _i(n_heads), _i(n_kv), _i(page_size),
+         _i(block_table.shape[1]), _i(num_pages), _i(window), _f(scale), _stream())
+    return out
+
+
+# ---------------------------------------------------------------------------
+def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
+           uniform: torch.Tensor, work: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    rows, vocab = logits.shape
+    _chk(logits, "sample.logits", torch.float32)
+    _chk(temperature, "sample.temperature", torch.float32, (rows,))
+    _chk(top_k, "sample.top_k", torch.int32, (rows,))
+    _chk(top_p, "sample.top_p", torch.float32, (rows,))
+    _chk(uniform, "sample.uniform", torch.float32, (rows,))
+    _chk(work, "sample.work", torch.float32)
+    if work.numel() < rows * vocab:
+        raise KernelError("sample: workspace smaller than the logits")
+    _chk(out, "sample.out", torch.int32, (rows,))
+    _run(load_lib("vt_sampling"), "vt_sample", _ptr(logits), _i(rows), _i(vocab), _ptr(temperature), _ptr(top_k),
+         _ptr(top_p), _ptr(uniform), _ptr(work), _ptr(out), _stream())
+    return out
+
+
+def require_gpu() -> torch.device:
+    if not torch.cuda.is_available():
+        raise KernelError("no GPU is visible: this engine has no CPU path")
+    return torch.device("cuda", torch.cuda.current_device())

@@ -1,0 +1,122 @@
+"""Attention mixer over paged keys and values: grouped-query heads, optional
+bias on the projections, optional window, position encoding as a part of its
+own.
+
+Per token, in the order of the reference's layer program
+(v1/models/qwen2-7b/inference_fp16.dag:296-322): K, Q and V projections with
+bias (:296, :302, :312), rotary encoding of K and Q (:297, :303), keys and
+values kept for later steps (:298, :313), scores scaled by 1/sqrt(D), causal
+mask, fp32 softmax, weighted sum (:307-318), output projection without bias
+(:322).  The three projections are one matrix product here (rows of Q, then
+K, then V), rotation is fused with the write into the cache pages, and
+scores, mask, softmax and weighted sum are one kernel that reads the pages.
+"""
+from __future__ import annotations
+
+import math
+from typing import Callable, Dict, Optional
+
+import torch
+
+from ..config.base import PartSpec
+from ..kernels import ops
+from .base import MIXERS, POSITIONS, CacheNeed, Part, Runtime, StateNeed, TensorDecl
+from .linear import linear
+
+
+@MIXERS.register("attention")
+class PagedAttention(Part):
+    def __init__(self, *, rt: Runtime, width: int, prefix: str, num_heads: int, num_kv_heads: int, head_dim: int,
+                 qkv_bias: bool = False, out_bias: bool = False, window: int = 0,
+                 position: Optional[PartSpec] = None, scale: Optional[float] = None, shared: Optional[dict] = None,
+                 names: Optional[Dict[str, str]] = None):
+        if num_heads % num_kv_heads:
+            raise ValueError(f"{num_heads} query heads are not a multiple of {num_kv_heads} key/value heads")
+        self.rt = rt
+        self.width = int(width)
+        self.nh, self.nkv, self.d = int(num_heads), int(num_kv_heads), int(head_dim)
+        self.qkv_bias, self.out_bias = bool(qkv_bias), bool(out_bias)
+        self.window = int(window)
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.d)
+        self.prefix = prefix
+        n = {"q": "q_proj", "k": "k_proj", "v": "v_proj", "o": "o_proj"}
+        n.update(names or {})
+        self.names = {k: prefix + v for k, v in n.items()}
+        # one table per distinct position encoding of the model
+        pos_spec = position or PartSpec("none", {})
+        shared = shared if shared is not None else {}
+        key = "position:" + pos_spec.key()
+        if key not in shared:
+            shared[key] = POSITIONS.build(pos_spec, rt=rt)
+        self.position = shared[key]
+        self.w_qkv = self.b_qkv = self.b_qkv_lowp = self.w_o = self.b_o = None
+
+    # -- what the cache manager must hold for this mixer --------------------
+    def cache_need(self) -> Optional[CacheNeed]:
+        return CacheNeed(self.nkv, self.d, self.window)
+
+    def state_need(self) -> Optional[StateNeed]:
+        return None
+
+    # -- weights -------------------------------------------------------------
+    def tensors(self) -> Dict[str, TensorDecl]:
+        nm, d = self.names, self.d
+        t = {
+            nm["q"] + ".weight": TensorDecl((self.nh * d, self.width), "matrix"),
+            nm["k"] + ".weight": TensorDecl((self.nkv * d, self.width), "matrix"),
+            nm["v"] + ".weight": TensorDecl((self.nkv * d, self.width), "matrix"),
+            nm["o"] + ".weight": TensorDecl((self.width, self.nh * d), "matrix"),
+        }
+        if self.qkv_bias:
+            t[nm["q"] + ".bias"] = TensorDecl((self.nh * d,), "bias")
+            t[nm["k"] + ".bias"] = TensorDecl((self.nkv * d,), "bias")
+            t[nm["v"] + ".bias"] = TensorDecl((self.nkv * d,), "bias")
+        if self.out_bias:
+            t[nm["o"] + ".bias"] = TensorDecl((self.width,), "bias")
+        return t
+
+    def load(self, get: Callable[[str], torch.Tensor], rt: Runtime) -> None:
+        nm = self.names
+        self.w_qkv = torch.cat([rt.place(get(nm[k] + ".weight"), "matrix") for k in "qkv"], dim=0).contiguous()
+        if self.qkv_bias:
+            self.b_qkv = torch.cat([rt.place(get(nm[k] + ".bias"), "bias") for k in "qkv"], dim=0).contiguous()
+            self.b_qkv_lowp = self.b_qkv.to(torch.bfloat16)
+        self.w_o = rt.place(get(nm["o"] + ".weight"), "matrix")
+        if self.out_bias:
+            self.b_o = rt.place(get(nm["o"] + ".bias"), "bias")
+
+    # -- one step --------------------------------------------------------------
+    def forward(self, x: torch.Tensor, ctx, cache, state=None) -> torch.Tensor:
+        rt, nh, nkv, d = self.rt, self.nh, self.nkv, self.d
+        n = x.shape[0]
+        nq = nh * d
+        if cache.writes:
+            qkv = linear(rt, x, self.w_qkv, self.b_qkv, "attn.qkv", bias_lowp=self.b_qkv_lowp)
+        else:  # keys and values of another layer: only queries are made
+            bq = self.b_qkv[:nq] if self.b_qkv is not None else None
+            bql = self.b_qkv_lowp[:nq] if self.b_qkv_lowp is not None else None
+            qkv = linear(rt, x, self.w_qkv[:nq], bq, "attn.qonly", bias_lowp=bql)
+        tables = self.position.rotary_tables(ctx.n_positions)
+        if tables is None and hasattr(self.position, "apply") and self.position.dim != 0:
+            # a position encoding that is not a plain rotation: let it rewrite queries and keys, then store unrotated
+            qv = qkv[:, :nq].reshape(n, nh, d)
+            kv = qkv[:, nq:nq + nkv * d].reshape(n, nkv, d) if cache.writes else None
+            q2, k2 = self.position.apply(qv, kv, ctx.positions)
+            qkv = qkv.clone()
+            qkv[:, :nq] = q2.reshape(n, nq).to(qkv.dtype)
+            if cache.writes:
+                qkv[:, nq:nq + nkv * d] = k2.reshape(n, nkv * d).to(qkv.dtype)
+        cos, sin = tables if tables is not None else (None, None)
+        q = rt.buffer("attn.q", (n, nq), rt.dtype)
+        ops.rope_store(qkv, cos, sin, ctx.positions, ctx.tok_entry, cache.block_table, q, cache.k, cache.v, nh, nkv, d,
+                       write_kv=cache.writes)
+        out = rt.buffer("attn.out", (n, nq), rt.dtype)
+        if rt.dtype == torch.float32:
+            ops.attention_f32(q, cache.k, cache.v, ctx.positions, ctx.tok_entry, cache.block_table, out, nh, nkv, d,
+                              self.window, self.scale)
+        else:
+            plan = ctx.attention_plan(nh // nkv, self.window, nkv, d)
+            ops.attention_bf16(q, cache.k, cache.v, cache.block_table, plan.items, plan.n_items, plan.citems,
+                               plan.n_citems, out, plan.part_o, plan.part_ml, nh, nkv, d, self.window, self.scale,
+                               max_part=plan.n_parts)
+        return linear(rt, out, self.w_o, self.b_o, "attn.o")

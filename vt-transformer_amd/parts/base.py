@@ -1,0 +1,145 @@
+"""What a part is, and the registries that parts are chosen from.
+
+A model is put together from parts of five roles.  Each part gets its sizes
+and constants as constructor parameters (from a `PartSpec`), says which
+tensors it needs, and computes on the tokens of one step.  No part knows
+which model it is in, which layer it is, or what the other parts of its
+layer are.
+
+Interfaces (N = tokens of the step, H = model width):
+
+  Norm            forward(h[N,H] fp32, delta[N,H] or None, rows=None) -> normed [N or R, H] in the runtime's dtype.
+                  With `delta`, h += delta happens first (and is stored in h unless `rows` picks rows).
+  PositionEncoding
+                  rotary_tables(n_positions) -> (cos, sin) fp32 [n_positions, dims/2] or None if the
+                  encoding is not a rotation that the fused kernel can apply;
+                  apply(q, k, positions) -> (q, k) otherwise.
+  Mixer           forward(x[N,H], ctx, cache, state) -> [N,H]; cache_need() / state_need() say what the cache
+                  manager has to hold for it (keys and values in pages; fixed-size state per request).
+  FeedForward     forward(x[N,H], ctx) -> [N,H]
+  Block           forward(h, delta, ctx, cache, state) -> (h, delta): arranges two norms, a mixer and a
+                  feed-forward around the fp32 residual stream h.  `delta` is a layer output that has
+                  not been added to h yet, so that the next norm can fuse the addition.
+
+The reference's counterpart is the set of `op.*` words that a model program
+strings together (v1/tensortype/nn_operators.cpp:530-576) and its user words
+with stack parameters (v1/models/qwen2-7b/inference_fp16.dag:287-345).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Any, Callable, Dict, Optional, Tuple
+
+import torch
+
+from ..config.base import ConfigError, PartSpec
+
+
+@dataclass(frozen=True)
+class TensorDecl:
+    """A tensor that a part needs: its shape and what it is.
+
+    role "matrix": kept in the runtime's dtype (bfloat16 or float32);
+    "gain", "bias": small vectors, kept in float32 (exact from bfloat16);
+    "table": integers, kept as int32.  A tensor stored in 32-bit stays so."""
+
+    shape: Tuple[int, ...]
+    role: str
+    optional: bool = False
+
+
+@dataclass(frozen=True)
+class CacheNeed:
+    """Keys and values that a mixer wants kept in pages, per token."""
+
+    kv_heads: int
+    head_dim: int
+    window: int = 0  # 0: every key stays; W: a key is dead once W later tokens exist
+
+    def group_key(self):
+        return (self.kv_heads, self.head_dim, self.window)
+
+
+@dataclass(frozen=True)
+class StateNeed:
+    """Per-request state of fixed size that a mixer wants kept between steps."""
+
+    shape: Tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+class Runtime:
+    """Device, dtype and scratch buffers shared by the parts of one model."""
+
+    def __init__(self, device: torch.device, dtype: torch.dtype):
+        if dtype not in (torch.bfloat16, torch.float32):
+            raise ValueError(f"dtype {dtype} is not supported (bfloat16 and float32 are)")
+        self.device = device
+        self.dtype = dtype
+        self._buffers: Dict[str, torch.Tensor] = {}
+
+    def place(self, t: torch.Tensor, role: str) -> torch.Tensor:
+        """A loaded tensor as the kernels want it, on the device."""
+        if role == "matrix":
+            if t.dtype in (torch.float32, torch.bfloat16, torch.float16, torch.float64):
+                return t.to(device=self.device, dtype=self.dtype).contiguous()
+            raise ValueError(f"matrix of dtype {t.dtype}")
+        if role in ("gain", "bias"):
+            return t.to(device=self.device, dtype=torch.float32).contiguous()
+        if role == "table":
+            return t.to(device=self.device, dtype=torch.int32).contiguous()
+        raise ValueError(f"unknown tensor role {role!r}")
+
+    def buffer(self, name: str, shape, dtype: torch.dtype) -> torch.Tensor:
+        """A scratch tensor that keeps its address between steps (grown when a step needs more)."""
+        n = 1
+        for s in shape:
+            n *= int(s)
+        buf = self._buffers.get(name)
+        if buf is None or buf.dtype != dtype or buf.numel() < n:
+            buf = torch.empty(max(n, 1), dtype=dtype, device=self.device)
+            self._buffers[name] = buf
+        return buf[:n].view(*shape)
+
+
+class Part:
+    """Base of all parts."""
+
+    def tensors(self) -> Dict[str, TensorDecl]:
+        """Full tensor names this part loads, with their shapes."""
+        return {}
+
+    def load(self, get: Callable[[str], torch.Tensor], rt: Runtime) -> None:
+        """Take the tensors named by `tensors()` (get(name) -> CPU or device tensor) onto the device."""
+
+
+class Registry:
+    def __init__(self, role: str):
+        self.role = role
+        self._kinds: Dict[str, Any] = {}
+
+    def register(self, kind: str, cls=None):
+        if cls is None:
+            def deco(c):
+                self._kinds[kind] = c
+                return c
+            return deco
+        self._kinds[kind] = cls
+        return cls
+
+    def kinds(self):
+        return sorted(self._kinds)
+
+    def build(self, spec: PartSpec, **context):
+        if spec.kind not in self._kinds:
+            raise ConfigError(f"no {self.role} of kind '{spec.kind}' is registered (known: {', '.join(self.kinds())})")
+        return self._kinds[spec.kind](**context, **spec.params)
+
+
+NORMS = Registry("norm")
+POSITIONS = Registry("position encoding")
+MIXERS = Registry("mixer")
+FEED_FORWARDS = Registry("feed-forward")
+BLOCKS = Registry("block")
+EMBEDDINGS = Registry("embedding")
+HEADS = Registry("head")

@@ -1,0 +1,59 @@
+"""Gated feed-forward: down( act(gate(x)) * up(x) ), no biases.
+
+The reference's order (v1/models/qwen2-7b/inference_fp16.dag:333-337): up
+projection (mlp.w2), gate projection (mlp.w1), silu(gate) * up
+(v1/tensortype/hip_kernels/silu_product.cpp:8-16), down projection
+(mlp.o_proj); w1 = gate_proj, w2 = up_proj, o_proj = down_proj
+(v1/models/qwen2-7b/dump_from_huggingface.py:89-99).  Gate and up are one
+matrix here (gate rows, then up rows); with few tokens the gating is applied
+to the fp32 accumulators inside the product's kernel.
+"""
+from __future__ import annotations
+
+from typing import Callable, Dict, Optional
+
+import torch
+
+from ..kernels import ops
+from .base import FEED_FORWARDS, Part, Runtime, TensorDecl
+from .linear import SKINNY_MAX_ROWS, linear
+
+
+@FEED_FORWARDS.register("gated_mlp")
+class GatedMLP(Part):
+    def __init__(self, *, rt: Runtime, width: int, prefix: str, intermediate_size: int, activation: str = "silu",
+                 names: Optional[Dict[str, str]] = None):
+        if activation != "silu":
+            raise ValueError(f"activation '{activation}' is not supported (only 'silu')")
+        self.rt = rt
+        self.width = int(width)
+        self.inter = int(intermediate_size)
+        n = {"gate": "gate_proj", "up": "up_proj", "down": "down_proj"}
+        n.update(names or {})
+        self.names = {k: prefix + v for k, v in n.items()}
+        self.w_gu = self.w_down = None
+
+    def tensors(self) -> Dict[str, TensorDecl]:
+        nm = self.names
+        return {
+            nm["gate"] + ".weight": TensorDecl((self.inter, self.width), "matrix"),
+            nm["up"] + ".weight": TensorDecl((self.inter, self.width), "matrix"),
+            nm["down"] + ".weight": TensorDecl((self.width, self.inter), "matrix"),
+        }
+
+    def load(self, get: Callable[[str], torch.Tensor], rt: Runtime) -> None:
+        nm = self.names
+        self.w_gu = torch.cat([rt.place(get(nm["gate"] + ".weight"), "matrix"),
+                               rt.place(get(nm["up"] + ".weight"), "matrix")], dim=0).contiguous()
+        self.w_down = rt.place(get(nm["down"] + ".weight"), "matrix")
+
+    def forward(self, x: torch.Tensor, ctx=None) -> torch.Tensor:
+        rt = self.rt
+        n = x.shape[0]
+        act = rt.buffer("mlp.act", (n, self.inter), rt.dtype)
+        if rt.dtype == torch.bfloat16 and n <= SKINNY_MAX_ROWS:
+            ops.gated_linear_bf16(x, self.w_gu, act)
+        else:
+            gu = linear(rt, x, self.w_gu, None, "mlp.gu")
+            ops.silu_mul(gu, act)
+        return linear(rt, act, self.w_down, None, "mlp.down")

@@ -1,0 +1,43 @@
+"""y = x W^T + b with W stored [out, in], as the reference's op_linear
+(v1/tensortype/hip_tensor.cpp:479-539; layout asserted in
+v1/tensortype/tensortype.cpp:222-229).
+
+float32: the hand-written fp32 kernel, always (no matrix-core mode).
+bfloat16: the hand-written matrix-core kernel while the rows are few enough
+that reading W dominates; above that the GEMM library, which is where the
+reference's engine uses a library too (hipblasGemmEx, hip_tensor.cpp:514-535).
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from ..kernels import ops
+from .base import Runtime
+
+# up to this many rows W is streamed once per 64 rows by the skinny kernel
+SKINNY_MAX_ROWS = 64
+
+
+def linear(rt: Runtime, x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], name: str,
+           out_dtype: Optional[torch.dtype] = None, bias_lowp: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x [N, K] in the runtime's dtype -> [N, M].  `name` keys the output's scratch buffer.
+    Output dtype: float32 from the hand-written kernels unless `out_dtype` says otherwise; the
+    library path returns bfloat16 (its bias, if any, is `bias_lowp`, the same values in bfloat16)."""
+    n, k = x.shape
+    m = w.shape[0]
+    if rt.dtype == torch.float32:
+        out = rt.buffer(name, (n, m), torch.float32)
+        return ops.linear_f32(x, w, bias, out)
+    if n <= SKINNY_MAX_ROWS:
+        out = rt.buffer(name, (n, m), out_dtype or torch.float32)
+        return ops.linear_bf16(x, w, bias, out)
+    out = rt.buffer(name + ".lib", (n, m), torch.bfloat16)
+    if bias is not None:
+        if bias_lowp is None:
+            bias_lowp = bias.to(torch.bfloat16)
+        torch.addmm(bias_lowp, x, w.t(), out=out)
+    else:
+        torch.mm(x, w.t(), out=out)
+    return out
