@@ -1,0 +1,152 @@
+#!/usr/bin/env python3
+"""Decode and prefill throughput of the engine at Qwen2-7B layer sizes, random weights, one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Prints one JSON line.  `value` is decoded tokens per second at batch 8 after 1,024-token prompts (a step is one
+decode step of the whole batch through scheduler, step function and sampler).  The line also carries the
+prefill of one 2,048-token prompt, the decode step's achieved HBM bandwidth against the bytes it has to read,
+and decode at batch 1 and 64.  The reference publishes no number to compare with (vs_baseline is null).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+# Qwen2-7B layer sizes (v1/models/qwen2-7b/inference_fp16.dag:1-15 of the reference)
+QWEN2_7B = dict(architectures=["Qwen2ForCausalLM"], vocab_size=152064, hidden_size=3584, intermediate_size=18944,
+                num_hidden_layers=28, num_attention_heads=28, num_key_value_heads=4, head_dim=128,
+                rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=8192,
+                hidden_act="silu", use_sliding_window=False)
+FULL_LAYERS = 28
+HBM_GBPS = 8000.0          # MI355X HBM3E, published
+PEAK_FLOPS = {"bf16": 2.5e15, "fp16": 2.5e15, "fp8": 5.0e15, "fp32": 157.3e12}   # dense MFMA, published
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--prompt-len", type=int, default=1024)
+    ap.add_argument("--layers", type=int, default=FULL_LAYERS, help="fewer layers than the model has (named in config)")
+    ap.add_argument("--prefill-tokens", type=int, default=2048)
+    ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
+    ap.add_argument("--no-graphs", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this engine runs on one GPU; N > 1 is not measured")
+        return 2
+
+    import numpy as np
+    import torch
+    from vt_transformer_amd.config import config_from_dict
+    from vt_transformer_amd.engine import Engine, StepEntry
+    from vt_transformer_amd.sampling import SamplingParams
+
+    cfg_d = dict(QWEN2_7B)
+    cfg_d["num_hidden_layers"] = args.layers
+    cfg = config_from_dict(cfg_d)
+    ctx_len = cfg.max_position_embeddings
+    max_batch = 64 if not args.no_points else max(args.batch, 1)
+    per_req = -(-(args.prompt_len + args.steps + args.warmup + 32) // 16) * 16
+    pool_tokens = max(max_batch * per_req, args.prefill_tokens + 64)
+    t0 = time.time()
+    eng = Engine(config=cfg, random_weights_seed=0, dtype="bfloat16", page_size=16, num_pages=pool_tokens // 16,
+                 max_running_reqs=max(max_batch, 1), max_seq_len=ctx_len, max_extend_tokens=8192, chunk_size=2048,
+                 decode_graphs=not args.no_graphs)
+    torch.cuda.synchronize()
+    print(f"[bench] model ready in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
+    rs = np.random.RandomState(0)
+
+    def decode_run(batch: int, steps: int, warmup: int):
+        """tokens/s and ms/step of `steps` decode steps at `batch` after prompts of --prompt-len tokens."""
+        sp = SamplingParams(max_tokens=steps + warmup + 8, ignore_eos=True)
+        uids = [eng.add_request(rs.randint(0, cfg.vocab_size, size=args.prompt_len).tolist(), sp) for _ in range(batch)]
+        while any(not eng.requests[u].decoding for u in uids):      # prompts, in portions under the token budget
+            eng.step()
+        for _ in range(warmup):
+            eng.step()
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(steps):
+            eng.step()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t
+        ctx_mid = args.prompt_len + 1 + warmup + steps // 2
+        for u in uids:
+            eng.abort_request(u)
+        while eng.has_work():
+            eng.step()
+        print(f"[bench] decode batch {batch}: {batch * steps / dt:.1f} tok/s, {dt / steps * 1e3:.3f} ms/step",
+              file=sys.stderr, flush=True)
+        return batch * steps / dt, dt / steps * 1e3, ctx_mid
+
+    def prefill_run(tokens: int, reps: int = 3):
+        runner = eng.runner
+        best = None
+        for i in range(reps + 1):
+            rid = f"prefill{i}"
+            runner.admit(rid)
+            ids = rs.randint(0, cfg.vocab_size, size=tokens).tolist()
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            runner.step([StepEntry(rid, ids, [tokens - 1])])
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t
+            runner.release(rid)
+            if i > 0:
+                best = dt if best is None else min(best, dt)
+        print(f"[bench] prefill {tokens} tokens: {best * 1e3:.2f} ms", file=sys.stderr, flush=True)
+        return best
+
+    # ---- sizes for the roofline -------------------------------------------------
+    H, I, V, L = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size, cfg.num_hidden_layers
+    qkv = (cfg.num_attention_heads + 2 * cfg.num_key_value_heads) * cfg.head_dim
+    layer_params = qkv * H + qkv + cfg.num_attention_heads * cfg.head_dim * H + 3 * I * H + 2 * H
+    weight_bytes = 2 * (L * layer_params + V * H + H)                  # every weight the step uses, once (bf16)
+    kv_bytes_per_token = 2 * 2 * L * cfg.num_key_value_heads * cfg.head_dim
+
+    tps, ms, ctx_mid = decode_run(args.batch, args.steps, args.warmup)
+    step_bytes = weight_bytes + args.batch * ctx_mid * kv_bytes_per_token
+    achieved = step_bytes / (ms * 1e-3) / 1e9
+
+    T = args.prefill_tokens
+    p_dt = prefill_run(T)
+    mm_flops = 2.0 * T * L * (qkv * H + cfg.num_attention_heads * cfg.head_dim * H + 3 * I * H) + 2.0 * V * H
+    attn_flops = L * 4.0 * cfg.num_attention_heads * cfg.head_dim * (T * (T + 1) / 2)   # causal: QK^T and PV
+    p_flops = mm_flops + attn_flops
+
+    points = {}
+    if not args.no_points:
+        for b in (1, 64):
+            k = max(16, args.steps // 2)
+            points[f"decode_b{b}"] = round(decode_run(b, k, 8)[0], 1)
+
+    line = {
+        "metric": "decode tok/s at batch 8, Qwen2-7B layer sizes, 1,024-token prompts",
+        "value": round(tps, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic (random weights N(0,0.02), uniform random token ids)",
+        "config": {"model": "Qwen2-7B sizes", "layers": L, "layers_full": FULL_LAYERS, "hidden": H,
+                   "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
+                   "intermediate": I, "vocab": V, "global_batch": args.batch, "seq_len": args.prompt_len,
+                   "prompt_len": args.prompt_len, "context_len": ctx_len, "kv_block": 16, "rope_theta": cfg.rope_theta,
+                   "parallelism": "1 GPU", "decode_graphs": not args.no_graphs},
+        "prefill": {"value": round(T / p_dt, 1), "tokens": T, "ms": round(p_dt * 1e3, 3),
+                    "frac": round(p_flops / p_dt / PEAK_FLOPS["bf16"], 4)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBPS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_GBPS, 4)},
+        "points": points,
+    }
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -182,3 +182,80 @@ def test_random_weights_on_device_match_written_folder(model_folders):
     r.admit(0)
     logits = r.step([StepEntry(0, [1, 2, 3, 4, 5], [4])])
     assert logits.shape == (1, TINY["A"]["vocab_size"]) and bool(torch.isfinite(logits).all())
+
+
+# ---------------------------------------------------------------------------
+# the entry point: scheduler, step function and sampler together
+# ---------------------------------------------------------------------------
+def test_greedy_generation_through_entry_point(model_folders):
+    from vt_transformer_amd.engine import Engine
+    from vt_transformer_amd.sampling import SamplingParams
+    cfg = "A"
+    pc, pw = plain_model.read_folder(model_folders[cfg])
+    prompts = list(random_requests(TINY[cfg]["vocab_size"], [5, 9, 13], seed=20).values())
+    want = [plain_model.greedy(pc, pw, p, 8) for p in prompts]
+    eng = Engine(model_folders[cfg], dtype="float32", num_pages=12, max_running_reqs=3, max_seq_len=64)
+    got = eng.generate(prompts, SamplingParams(max_tokens=8, ignore_eos=True))
+    assert got == want
+    assert sum(eng.runner.cache.held_pages()) == 0
+    # bfloat16: every chosen token is the plain model's best or within rounding of it
+    eng = Engine(model_folders[cfg], dtype="bfloat16", num_pages=12, max_running_reqs=3, max_seq_len=64)
+    got = eng.generate(prompts, SamplingParams(max_tokens=8, ignore_eos=True))
+    for p, g in zip(prompts, got):
+        logits = plain_model.forward(pc, pw, p + g)
+        for i, tok in enumerate(g):
+            row = logits[len(p) - 1 + i]
+            assert float(row.max() - row[tok]) <= 3e-2 * float(row.abs().max())
+
+
+def test_chunked_prompts_mixed_with_decoding_and_temperature(model_folders):
+    """Prompts of 1/7/16/31 tokens in portions of 8 beside decoding requests, temperature 0.8 from a fixed seed:
+    the same tokens whatever the batch looks like (alone, together, preempted)."""
+    from vt_transformer_amd.engine import Engine
+    from vt_transformer_amd.sampling import SamplingParams
+    cfg = "B"
+    prompts = list(random_requests(TINY[cfg]["vocab_size"], [1, 7, 16, 31], seed=21).values())
+    sp = [SamplingParams(temperature=0.8, max_tokens=8, ignore_eos=True, seed=1000 + i) for i in range(4)]
+    together = Engine(model_folders[cfg], dtype="float32", num_pages=32, max_running_reqs=4, max_seq_len=128,
+                      chunk_size=8, max_extend_tokens=12)
+    got = together.generate(prompts, sp)
+    for i, p in enumerate(prompts):
+        alone = Engine(model_folders[cfg], dtype="float32", num_pages=8, max_running_reqs=1, max_seq_len=128)
+        assert alone.generate([p], [sp[i]])[0] == got[i]
+    # so few pages that decoding requests are preempted and recomputed: still the same tokens
+    tight = Engine(model_folders[cfg], dtype="float32", num_pages=5, max_running_reqs=4, max_seq_len=128,
+                   chunk_size=8, max_extend_tokens=12)
+    assert tight.generate(prompts, sp) == got
+    assert tight.scheduler.counters["preemptions"] > 0
+
+
+def test_decode_graph_replays_match_eager(model_folders):
+    """Captured decoding steps against the same steps launched one by one: several replays, with eager work
+    (prompt portions of other requests, synchronisations) between them, all equal."""
+    from vt_transformer_amd.engine import StepEntry
+    model = get_model(model_folders, "A", "bfloat16")
+    reqs = random_requests(TINY["A"]["vocab_size"], [60, 45, 30], seed=22)
+    eager, graph = runner_for(model, 512), runner_for(model, 512)
+    graph.decode_graphs = True
+    for r in (eager, graph):
+        for rid, toks in reqs.items():
+            r.admit(rid)
+            r.step([StepEntry(rid, toks[:20], [])])
+    for i in range(20, 30):
+        entries = [StepEntry(rid, toks[i:i + 1], [0]) for rid, toks in reqs.items()]
+        a = eager.step(entries).clone()
+        b = graph.step(entries).clone()
+        torch.cuda.synchronize()
+        assert torch.equal(a, b), f"decode step {i}"
+        if i % 3 == 0:   # eager work between replays: another request's portion through both runners
+            for r in (eager, graph):
+                r.admit(f"x{i}")
+                r.step([StepEntry(f"x{i}", reqs["r0"][:17], [16])])
+                r.release(f"x{i}")
+    # fewer entries than the captured batch: the padding entries must not disturb the real ones
+    e2 = [StepEntry("r0", reqs["r0"][30:31], [0]), StepEntry("r1", reqs["r1"][30:31], [0])]
+    e3 = e2 + [StepEntry("r2", reqs["r2"][29:30] if False else [reqs["r2"][29]], [0])]
+    a = eager.step(e3).clone()
+    b = graph.step(e3).clone()
+    assert torch.equal(a, b)
+    assert len(graph._graphs) >= 1

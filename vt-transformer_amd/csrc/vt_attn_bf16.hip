@@ -52,6 +52,11 @@ struct AttnArgs {
     float* part_ml;         // [parts][n_kv][16][2]
     int n_items, n_heads, n_kv, page_size, max_blocks, num_pages, window;
     float scale_log2;       // scale * log2(e)
+    // decode mode: one token per entry, items are computed here from the entries' positions
+    const int* entry_pos0;  // [entries] position of each entry's token
+    const int* dec_params;  // [0] = chunk: keys per item (a multiple of 16), read from memory so that a
+                            //       captured launch can be replayed with another value
+    int p_max;              // items per entry
 };
 
 union U8 { uint2 u; bf16x4_t v; };
@@ -61,14 +66,31 @@ __device__ __forceinline__ unsigned pack2(float a, float b) {
     return (unsigned)f32_to_bf16(a) | ((unsigned)f32_to_bf16(b) << 16);
 }
 
+template <bool DECODE>
 __global__ __launch_bounds__(256) void attn_bf16_kernel(AttnArgs a) {
     const int wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int item = blockIdx.x * 4 + wv;
     if (item >= a.n_items) return;
-    const int* it = a.items + (size_t)item * ITEM_INTS;
-    const int entry = it[0], q_tok0 = it[1], q_len = it[2], pos0 = it[3], q_row0 = it[4];
-    const int key_lo = it[5], key_hi = it[6], part = it[7];
-    if (entry < 0) return;
+    int entry, q_tok0, q_len, pos0, q_row0, key_lo, key_hi, part;
+    if (DECODE) {
+        // item = (entry, part p): keys [p*chunk, (p+1)*chunk) of the entry's one token
+        const int chunk = a.dec_params[0];
+        entry = item / a.p_max;
+        const int pi = item - entry * a.p_max;
+        q_tok0 = entry; q_len = 1; q_row0 = 0;
+        pos0 = a.entry_pos0[entry];
+        const int lo = a.window > 0 ? max(0, pos0 - a.window + 1) : 0;
+        const int p_first = ((lo >> 4) << 4) / chunk, p_last = pos0 / chunk;
+        if (pi < p_first || pi > p_last) return;
+        key_lo = max((lo >> 4) << 4, pi * chunk);
+        key_hi = min(pos0 + 1, (pi + 1) * chunk);
+        part = (p_first == p_last) ? -1 : item;
+    } else {
+        const int* it = a.items + (size_t)item * ITEM_INTS;
+        entry = it[0]; q_tok0 = it[1]; q_len = it[2]; pos0 = it[3]; q_row0 = it[4];
+        key_lo = it[5]; key_hi = it[6]; part = it[7];
+        if (entry < 0) return;
+    }
     const int kvh = blockIdx.y;
     const int G = a.n_heads / a.n_kv;
     const int r = lane & 15, g = lane >> 4;
@@ -185,11 +207,25 @@ __global__ __launch_bounds__(256) void attn_bf16_kernel(AttnArgs a) {
 
 // Merge the partial results of a row tile whose keys were split.
 // citems: [n][6] = q_tok0, q_len, q_row0, part0, n_parts, unused.  One block per (tile, kv head), 16 rows x D.
+template <bool DECODE>
 __global__ void attn_combine_kernel(const int* __restrict__ citems, const float* __restrict__ part_o,
-                                    const float* __restrict__ part_ml, bf16_t* __restrict__ out, int n_heads, int n_kv) {
-    const int* it = citems + (size_t)blockIdx.x * 6;
-    const int q_tok0 = it[0], q_len = it[1], q_row0 = it[2], part0 = it[3], n_parts = it[4];
-    if (n_parts <= 0) return;
+                                    const float* __restrict__ part_ml, bf16_t* __restrict__ out, int n_heads, int n_kv,
+                                    const int* __restrict__ entry_pos0, const int* __restrict__ dec_params, int p_max,
+                                    int window) {
+    int q_tok0, q_len, q_row0, part0, n_parts;
+    if (DECODE) {
+        const int e = blockIdx.x, chunk = dec_params[0], pos0 = entry_pos0[e];
+        const int lo = window > 0 ? max(0, pos0 - window + 1) : 0;
+        const int p_first = ((lo >> 4) << 4) / chunk, p_last = pos0 / chunk;
+        q_tok0 = e; q_len = 1; q_row0 = 0;
+        part0 = e * p_max + p_first;
+        n_parts = p_last - p_first + 1;
+        if (n_parts <= 1) return;   // a single item wrote the output itself
+    } else {
+        const int* it = citems + (size_t)blockIdx.x * 6;
+        q_tok0 = it[0]; q_len = it[1]; q_row0 = it[2]; part0 = it[3]; n_parts = it[4];
+        if (n_parts <= 0) return;
+    }
     const int kvh = blockIdx.y, G = n_heads / n_kv;
     for (int idx = threadIdx.x; idx < 16 * D; idx += blockDim.x) {
         int r = idx / D, d = idx - r * D;
@@ -228,11 +264,43 @@ extern "C" int vt_attn_bf16(const void* q, const void* k_pages, const void* v_pa
     a.block_table = block_table; a.items = items; a.out = (bf16_t*)out; a.part_o = part_o; a.part_ml = part_ml;
     a.n_items = n_items; a.n_heads = n_heads; a.n_kv = n_kv; a.page_size = page_size; a.max_blocks = max_blocks;
     a.num_pages = num_pages; a.window = window; a.scale_log2 = scale * 1.4426950408889634f;
-    attn_bf16_kernel<<<dim3((n_items + 3) / 4, n_kv), 256, 0, stream>>>(a);
+    a.entry_pos0 = nullptr; a.dec_params = nullptr; a.p_max = 0;
+    attn_bf16_kernel<false><<<dim3((n_items + 3) / 4, n_kv), 256, 0, stream>>>(a);
     VT_CHECK_LAUNCH("vt_attn_bf16");
     if (n_citems > 0) {
-        attn_combine_kernel<<<dim3(n_citems, n_kv), 256, 0, stream>>>(citems, part_o, part_ml, (bf16_t*)out, n_heads, n_kv);
+        attn_combine_kernel<false><<<dim3(n_citems, n_kv), 256, 0, stream>>>(citems, part_o, part_ml, (bf16_t*)out,
+                                                                            n_heads, n_kv, nullptr, nullptr, 0, window);
         VT_CHECK_LAUNCH("vt_attn_bf16(combine)");
     }
+    return 0;
+}
+
+// Decoding: one token per entry (token i belongs to entry i, at position entry_pos0[i]).  Every entry gets p_max
+// items of dec_params[0] keys each; items beyond the entry's keys exit at once.  Nothing here depends on values
+// that change between steps except through device memory, so the launches can be captured once and replayed.
+// The workspace holds n_entries * p_max partial slots.
+extern "C" int vt_attn_bf16_decode(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
+                                   const int* entry_pos0, const int* dec_params, int n_entries, int p_max, void* out,
+                                   float* part_o, float* part_ml, int n_heads, int n_kv, int page_size, int max_blocks,
+                                   int num_pages, int window, float scale, hipStream_t stream) {
+    VT_REQUIRE(n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "vt_attn_bf16_decode: bad heads %d/%d", n_heads, n_kv);
+    VT_REQUIRE(n_heads / n_kv <= 16, "vt_attn_bf16_decode: %d query heads per kv head do not fit one tile of 16 rows",
+               n_heads / n_kv);
+    VT_REQUIRE(page_size > 0 && page_size % 16 == 0, "vt_attn_bf16_decode: page size %d is not a multiple of 16", page_size);
+    VT_REQUIRE(max_blocks > 0 && num_pages > 0 && p_max > 0, "vt_attn_bf16_decode: bad sizes");
+    VT_REQUIRE(n_kv <= 65535, "vt_attn_bf16_decode: too many kv heads (%d)", n_kv);
+    VT_REQUIRE(part_o && part_ml && entry_pos0 && dec_params, "vt_attn_bf16_decode: missing buffers");
+    if (n_entries <= 0) return 0;
+    AttnArgs a;
+    a.q = (const bf16_t*)q; a.k_pages = (const bf16_t*)k_pages; a.v_pages = (const bf16_t*)v_pages;
+    a.block_table = block_table; a.items = nullptr; a.out = (bf16_t*)out; a.part_o = part_o; a.part_ml = part_ml;
+    a.n_items = n_entries * p_max; a.n_heads = n_heads; a.n_kv = n_kv; a.page_size = page_size; a.max_blocks = max_blocks;
+    a.num_pages = num_pages; a.window = window; a.scale_log2 = scale * 1.4426950408889634f;
+    a.entry_pos0 = entry_pos0; a.dec_params = dec_params; a.p_max = p_max;
+    attn_bf16_kernel<true><<<dim3((a.n_items + 3) / 4, n_kv), 256, 0, stream>>>(a);
+    VT_CHECK_LAUNCH("vt_attn_bf16_decode");
+    attn_combine_kernel<true><<<dim3(n_entries, n_kv), 256, 0, stream>>>(nullptr, part_o, part_ml, (bf16_t*)out, n_heads,
+                                                                        n_kv, entry_pos0, dec_params, p_max, window);
+    VT_CHECK_LAUNCH("vt_attn_bf16_decode(combine)");
     return 0;
 }

@@ -3,3 +3,7 @@ from .loading import build_model, load_model, make_runner, parse_dtype, random_m
 
 __all__ = ["ModelRunner", "OutOfPages", "StepContext", "StepEntry", "plan_attention_items", "build_model",
            "load_model", "make_runner", "parse_dtype", "random_model"]
+from .scheduler import ReqResult, Request, Scheduled, Scheduler, SchedulerConfig  # noqa: E402
+from .engine import Engine  # noqa: E402
+
+__all__ += ["ReqResult", "Request", "Scheduled", "Scheduler", "SchedulerConfig", "Engine"]

@@ -1,0 +1,114 @@
+"""The engine a user holds: requests in, tokens out.
+
+`Engine.step()` is the reference's scheduler step (FullScheduler::step,
+vt-transformer/core/vt_scheduler.cpp:96-141): choose a batch, run the step
+function, take the results, finish and free; `generate()` is the loop its
+back end runs (vt_backend.cpp:94-103) without the sockets.  Token ids go in
+and come out; text is the front end's business, as in the reference where
+sglfront tokenises and the engine sees ids only.
+"""
+from __future__ import annotations
+
+import time
+from typing import Dict, Hashable, Iterable, List, Optional, Sequence, Union
+
+import torch
+
+from ..config import ModelConfig, load_config
+from ..sampling import Sampler, SamplingParams, request_seed
+from .loading import load_model, make_runner, random_model
+from .scheduler import ReqResult, Request, Scheduled, Scheduler, SchedulerConfig
+from .step import ModelRunner, StepEntry
+
+
+class Engine:
+    def __init__(self, model: Optional[str] = None, *, config: Optional[ModelConfig] = None,
+                 random_weights_seed: Optional[int] = None, dtype: str = "bfloat16", seed: int = 0,
+                 scheduler_config: Optional[SchedulerConfig] = None, decode_graphs: bool = True, **options):
+        """model: a folder with config.json and model.safetensors.  Or `config` with `random_weights_seed`
+        for random weights drawn on the device.  `options` override fields of SchedulerConfig
+        (max_running_reqs, num_pages, max_seq_len, page_size, max_extend_tokens, default_max_output, chunk_size)."""
+        sc = scheduler_config or SchedulerConfig()
+        for k, v in options.items():
+            if not hasattr(sc, k):
+                raise TypeError(f"unknown engine option '{k}'")
+            setattr(sc, k, v)
+        if model is not None:
+            self.model = load_model(model, dtype)
+        elif config is not None and random_weights_seed is not None:
+            self.model = random_model(config, random_weights_seed, dtype)
+        else:
+            raise ValueError("give a model folder, or a config and random_weights_seed")
+        spec = self.model.spec
+        sc.max_seq_len = min(sc.max_seq_len, spec.max_positions)
+        self.config = sc
+        self.runner: ModelRunner = make_runner(self.model, pool_tokens=sc.num_pages * sc.page_size,
+                                               page_size=sc.page_size, max_requests=sc.max_running_reqs,
+                                               max_seq_len=sc.max_seq_len)
+        self.runner.decode_graphs = bool(decode_graphs)
+        self.scheduler = Scheduler(sc, self.runner.cache, spec.eos_token_ids)
+        self.sampler = Sampler(self.model.rt)
+        self.seed = int(seed)
+        self._next_uid = 0
+        self.requests: Dict[Hashable, Request] = {}
+
+    # -- requests ------------------------------------------------------------
+    def add_request(self, prompt: Sequence[int], params: Optional[SamplingParams] = None,
+                    uid: Optional[Hashable] = None) -> Hashable:
+        if uid is None:
+            uid = self._next_uid
+            self._next_uid += 1
+        if uid in self.requests and self.requests[uid].state != "finished":
+            raise ValueError(f"request id {uid!r} is in use")
+        params = params or SamplingParams(max_tokens=self.config.default_max_output)
+        vocab = self.model.spec.vocab_size
+        for t in prompt:
+            if not 0 <= int(t) < vocab:
+                raise ValueError(f"token id {t} is outside the vocabulary of {vocab}")
+        seed = params.seed if params.seed is not None else request_seed(self.seed, uid)
+        req = Request(uid, [int(t) for t in prompt], params, seed)
+        self.requests[uid] = req
+        self.scheduler.add_request(req)
+        return uid
+
+    def abort_request(self, uid: Hashable) -> bool:
+        return self.scheduler.abort_request(uid)
+
+    def has_work(self) -> bool:
+        return self.scheduler.has_work()
+
+    # -- one step ------------------------------------------------------------
+    def step(self) -> List[ReqResult]:
+        plan = self.scheduler.schedule()
+        sampled: Dict[Hashable, int] = {}
+        if plan:
+            entries = []
+            for s in plan:
+                toks = s.request.tokens[s.start:s.start + s.n_tokens]
+                entries.append(StepEntry(s.request.uid, toks, [s.n_tokens - 1] if s.sample else []))
+            logits = self.runner.step(entries)
+            rows = [(s.request.params, s.request.seed, len(s.request.output)) for s in plan if s.sample]
+            if rows:
+                toks = self.sampler.sample(logits, rows)
+                for s, t in zip((s for s in plan if s.sample), toks):
+                    sampled[s.request.uid] = t
+        return self.scheduler.update(plan, sampled)
+
+    # -- the whole loop --------------------------------------------------------
+    def generate(self, prompts: Union[Sequence[int], Sequence[Sequence[int]]],
+                 params: Union[None, SamplingParams, Sequence[SamplingParams]] = None) -> List[List[int]]:
+        """Token ids in, generated token ids out (one list per prompt, in order)."""
+        single = len(prompts) > 0 and not isinstance(prompts[0], (list, tuple))
+        plist = [prompts] if single else list(prompts)
+        if params is None or isinstance(params, SamplingParams):
+            params = [params] * len(plist)
+        uids = [self.add_request(p, sp) for p, sp in zip(plist, params)]
+        while self.has_work():
+            results = self.step()
+            if not results and not self.scheduler.running and self.scheduler.waiting:
+                raise RuntimeError("the scheduler cannot place the waiting requests (pool too small?)")
+        outs = [self.requests[u].output for u in uids]
+        return outs[0:1] if single else outs
+
+    def finish_reason(self, uid: Hashable) -> Optional[str]:
+        return self.requests[uid].finish_reason

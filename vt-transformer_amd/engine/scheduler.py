@@ -1,0 +1,266 @@
+"""Admission, portions of prompts under a token budget, decoding, finishing
+and freeing; and what happens when pages run out.
+
+After the reference's FullScheduler (vt-transformer/core/vt_scheduler.cpp):
+requests wait in arrival order (pending_) and run until they finish
+(running_) (vt_scheduler.hpp:132-141); a step's new tokens are bounded by
+max_extend_tokens (vt_scheduler.hpp:37); a request finishes on the end token
+or at its output limit (vt_scheduler.cpp:431-437); results are
+(uid, next_token, finished) (vt_scheduler.hpp:94-103); abort frees at once
+(vt_scheduler.cpp:47-88).  Request bookkeeping follows vt_request.hpp:12-33:
+the newest output token has no keys and values yet, the next step writes them.
+
+Where it differs: the reference runs either prompts or decoding in a step
+(vt_scheduler.cpp:102-110, 305-311), never cuts a prompt (:277, 292-294), and
+reserves the whole output budget at admission (:257-299); when a decode step
+cannot get a page it simply does not run and is tried again for ever
+(:112-117, 365-371).  Here every step carries all decoding requests plus
+portions of prompts; a prompt is cut to the budget; and when a decoding
+request cannot get a page the youngest running request is preempted: it
+gives everything back, returns to the head of the waiting line and is later
+recomputed from its prompt and the tokens it has produced.  A request that
+could never fit is finished with an error instead of waiting for ever.
+"""
+from __future__ import annotations
+
+from collections import deque
+from dataclasses import dataclass, field
+from typing import Deque, Dict, Hashable, List, Optional, Sequence, Tuple
+
+from ..cache.pages import CacheManager
+from ..sampling.params import SamplingParams
+
+
+@dataclass
+class SchedulerConfig:
+    """Names and defaults of the reference's SchedulerConfig (vt_scheduler.hpp:28-39) where it has them."""
+
+    max_running_reqs: int = 128     # live requests at a time (= state slots)
+    num_pages: int = 1024           # pages per group of layers
+    max_seq_len: int = 4096         # prompt + output of one request
+    page_size: int = 16             # tokens per page (the reference defaults to 1)
+    max_extend_tokens: int = 8192   # new tokens per step, prompts and decoding together
+    default_max_output: int = 1024  # output limit of a request that names none
+    chunk_size: int = 2048          # longest portion of one prompt in a step
+
+
+WAITING, RUNNING, FINISHED = "waiting", "running", "finished"
+
+
+@dataclass
+class Request:
+    uid: Hashable
+    prompt: List[int]
+    params: SamplingParams
+    seed: int = 0
+    output: List[int] = field(default_factory=list)
+    state: str = WAITING
+    computed: int = 0            # tokens whose keys and values are in the cache
+    arrival: int = 0
+    finish_reason: Optional[str] = None
+    preemptions: int = 0
+
+    @property
+    def tokens(self) -> List[int]:
+        return self.prompt + self.output
+
+    @property
+    def total_len(self) -> int:
+        return len(self.prompt) + len(self.output)
+
+    @property
+    def decoding(self) -> bool:
+        """All but the newest token are in the cache: the next step is one token."""
+        return self.state == RUNNING and len(self.output) > 0 and self.computed == self.total_len - 1
+
+
+@dataclass
+class Scheduled:
+    request: Request
+    start: int        # first token of the portion (= request.computed)
+    n_tokens: int
+    sample: bool      # the portion ends at the request's newest token: its last logits give the next token
+
+
+@dataclass
+class ReqResult:
+    uid: Hashable
+    next_token: Optional[int]
+    finished: bool
+    reason: Optional[str] = None
+
+
+class Scheduler:
+    def __init__(self, config: SchedulerConfig, cache: CacheManager, eos_token_ids: Sequence[int] = ()):
+        self.config = config
+        self.cache = cache
+        self.eos = set(int(e) for e in eos_token_ids)
+        self.waiting: Deque[Request] = deque()
+        self.running: List[Request] = []
+        self._arrivals = 0
+        self.finished_early: List[ReqResult] = []   # requests refused before they ever ran
+        self.counters = {"steps": 0, "tokens": 0, "preemptions": 0, "refused": 0}
+
+    # -- requests in and out -------------------------------------------------
+    def add_request(self, req: Request) -> None:
+        if not req.prompt:
+            raise ValueError(f"request {req.uid!r} has an empty prompt")
+        req.state, req.computed, req.arrival = WAITING, 0, self._arrivals
+        self._arrivals += 1
+        self.waiting.append(req)
+
+    def abort_request(self, uid: Hashable) -> bool:
+        for r in list(self.waiting):
+            if r.uid == uid:
+                self.waiting.remove(r)
+                r.state, r.finish_reason = FINISHED, "abort"
+                return True
+        for r in self.running:
+            if r.uid == uid:
+                self._finish(r, "abort")
+                return True
+        return False
+
+    def has_work(self) -> bool:
+        return bool(self.waiting or self.running or self.finished_early)
+
+    # -- one step's decisions ------------------------------------------------
+    def _capacity_tokens(self) -> int:
+        return min(p.num_pages for p in self.cache.pools) * self.cache.page_size
+
+    def _fits(self, items: List[Tuple[Request, int]]) -> bool:
+        need = [0] * len(self.cache.pools)
+        for r, new_len in items:
+            for gi, n in enumerate(self.cache.pages_needed(self.cache.get(r.uid), new_len)):
+                need[gi] += n
+        return all(n <= p.available for n, p in zip(need, self.cache.pools))
+
+    def _preempt(self, r: Request) -> None:
+        self.cache.release(r.uid)
+        self.running.remove(r)
+        r.state, r.computed = WAITING, 0
+        r.preemptions += 1
+        self.counters["preemptions"] += 1
+        self.waiting.appendleft(r)
+
+    def _finish(self, r: Request, reason: str) -> None:
+        if r.state == RUNNING:
+            self.cache.release(r.uid)
+            self.running.remove(r)
+        r.state, r.finish_reason = FINISHED, reason
+
+    def _refuse(self, r: Request, reason: str) -> None:
+        r.state, r.finish_reason = FINISHED, reason
+        self.counters["refused"] += 1
+        self.finished_early.append(ReqResult(r.uid, None, True, reason))
+
+    def schedule(self) -> List[Scheduled]:
+        """Choose the step's portions.  Pages are not taken here: the step function reserves them, and this
+        choice is made so that it will succeed."""
+        cfg = self.config
+        budget = cfg.max_extend_tokens
+        plan: List[Scheduled] = []
+        planned: List[Tuple[Request, int]] = []
+
+        # 1. every decoding request gets its one token; if pages run out, the youngest running request goes
+        decoding = sorted((r for r in self.running if r.decoding), key=lambda r: r.arrival)
+        while decoding:
+            items = [(r, r.computed + 1) for r in decoding[:budget]]
+            if self._fits(items):
+                break
+            victim = max(self.running, key=lambda r: r.arrival)
+            if len(self.running) == 1:
+                # alone and still no page: it can never go on
+                self._finish(victim, "out_of_pages")
+                self.finished_early.append(ReqResult(victim.uid, None, True, "out_of_pages"))
+            else:
+                self._preempt(victim)
+            decoding = [r for r in decoding if r is not victim]
+        for r in decoding[:budget]:
+            plan.append(Scheduled(r, r.computed, 1, True))
+            planned.append((r, r.computed + 1))
+        budget -= len(plan)
+
+        # 2. running requests still inside their prompt (or being recomputed), oldest first
+        for r in sorted((r for r in self.running if not r.decoding), key=lambda r: r.arrival):
+            if budget <= 0:
+                break
+            n = min(r.total_len - r.computed, cfg.chunk_size, budget)
+            if n <= 0 or not self._fits(planned + [(r, r.computed + n)]):
+                continue   # it waits for pages; decoding requests will free some or be preempted
+            plan.append(Scheduled(r, r.computed, n, r.computed + n == r.total_len))
+            planned.append((r, r.computed + n))
+            budget -= n
+
+        # 3. admit from the waiting line, in order, while a slot, budget and pages for a first portion are there
+        while self.waiting and budget > 0 and len(self.running) < cfg.max_running_reqs:
+            r = self.waiting[0]
+            limit = min(cfg.max_seq_len, self._capacity_tokens())
+            if r.total_len > limit:
+                self.waiting.popleft()
+                self._refuse(r, "too_long")
+                continue
+            if self.cache.slots.available == 0:
+                break
+            n = min(r.total_len - r.computed, cfg.chunk_size, budget)
+            rp = self.cache.admit(r.uid)
+            # head-room: one page per running request, so that admission does not starve decoding at once
+            reserve_pages = len(self.running)
+            ok = self._fits(planned + [(r, n)]) and all(
+                p.available - need >= reserve_pages for p, need in zip(
+                    self.cache.pools, self._need(planned + [(r, n)])))
+            if not ok:
+                self.cache.release(r.uid)
+                if not self.running and not plan:
+                    # nothing else holds pages and it still does not fit: cut the portion to what fits
+                    n_fit = min(n, min(p.available for p in self.cache.pools) * self.cache.page_size)
+                    if n_fit <= 0:
+                        self.waiting.popleft()
+                        self._refuse(r, "out_of_pages")
+                        continue
+                    self.cache.admit(r.uid)
+                    n = n_fit
+                else:
+                    break
+            self.waiting.popleft()
+            r.state = RUNNING
+            self.running.append(r)
+            plan.append(Scheduled(r, 0, n, n == r.total_len))
+            planned.append((r, n))
+            budget -= n
+        return plan
+
+    def _need(self, items: List[Tuple[Request, int]]) -> List[int]:
+        need = [0] * len(self.cache.pools)
+        for r, new_len in items:
+            for gi, k in enumerate(self.cache.pages_needed(self.cache.get(r.uid), new_len)):
+                need[gi] += k
+        return need
+
+    # -- after the step ------------------------------------------------------
+    def update(self, plan: List[Scheduled], sampled: Dict[Hashable, int]) -> List[ReqResult]:
+        """Record what the step stored and the tokens sampled for the portions that asked; finish and free."""
+        results: List[ReqResult] = list(self.finished_early)
+        self.finished_early = []
+        self.counters["steps"] += 1
+        for s in plan:
+            r = s.request
+            if r.state != RUNNING:
+                continue   # aborted while the step ran
+            r.computed = s.start + s.n_tokens
+            self.counters["tokens"] += s.n_tokens
+            if not s.sample:
+                continue
+            tok = int(sampled[r.uid])
+            r.output.append(tok)
+            reason = None
+            if tok in self.eos and not r.params.ignore_eos:
+                reason = "eos"
+            elif len(r.output) >= r.params.max_tokens:
+                reason = "max_tokens"
+            elif r.total_len >= self.config.max_seq_len:
+                reason = "max_seq_len"
+            if reason:
+                self._finish(r, reason)
+            results.append(ReqResult(r.uid, tok, reason is not None, reason))
+        return results

@@ -126,6 +126,10 @@ class StepContext:
         self.entry_start = self.entry_pos0 = self.state_slots = self.logit_rows = None
         self.block_tables: List[torch.Tensor] = []
         self.fresh: List[bool] = []           # per entry: the request's first step (its state slot was just cleared)
+        # set when every entry brings exactly one token (decoding): int32 device array whose [0] is the number of
+        # keys per attention item, and the number of items per entry
+        self.decode_params: Optional[torch.Tensor] = None
+        self.decode_p_max = 0
         self._plans: Dict[Tuple[int, int, int, int], AttentionPlan] = {}
 
     def attention_plan(self, group: int, window: int, n_kv: int, head_dim: int) -> AttentionPlan:
@@ -154,6 +158,28 @@ class StepContext:
         return AttentionPlan(d_items, items.shape[0], d_citems, citems.shape[0], part_o, part_ml, n_parts)
 
 
+def decode_chunk(kv_lens: np.ndarray, p_max: int, target_items: int = 1024, min_chunk: int = 64) -> int:
+    """Keys per attention item of a decoding step: small enough to fill the GPU, large enough that the longest
+    entry needs at most p_max items; a multiple of 16."""
+    total = int(kv_lens.sum())
+    chunk = max(min_chunk, -(-total // target_items), -(-int(kv_lens.max()) // p_max))
+    return -(-chunk // 16) * 16
+
+
+class _DecodeGraph:
+    """A captured decoding step for a fixed number of entries."""
+
+    def __init__(self):
+        self.graph = None
+        self.ctx: Optional[StepContext] = None
+        self.meta: Optional[torch.Tensor] = None
+        self.logits: Optional[torch.Tensor] = None
+        self.layout = None
+
+
+GRAPH_BATCHES = (1, 2, 4, 8, 16, 32, 64)
+
+
 class ModelRunner:
     """Owns the model, its cache and the step function."""
 
@@ -166,6 +192,12 @@ class ModelRunner:
         self.vocab_size = model.spec.vocab_size
         self.steps = 0
         self.tokens = 0
+        self.decode_p_max = max(1, min(64, -(-self.max_seq_len // 64)))
+        # Decoding steps of a bfloat16 model are captured once per batch size and replayed, unless a mixer keeps
+        # state of its own between steps (the warm-up run before a capture would advance it twice).
+        self.decode_graphs = False
+        self._graphs: Dict[int, _DecodeGraph] = {}
+        self._stateless = all(s is None for s in self.storage.state)
 
     # -- requests -----------------------------------------------------------
     def admit(self, rid: Hashable) -> bool:
@@ -175,7 +207,7 @@ class ModelRunner:
         self.cache.release(rid)
 
     # -- the step -----------------------------------------------------------
-    def build_context(self, entries: Sequence[StepEntry]) -> StepContext:
+    def _host_arrays(self, entries: Sequence[StepEntry], pad_to: int = 0, fixed_blocks: int = 0):
         cache, ps = self.cache, self.cache.page_size
         n_entries = len(entries)
         lens = np.array([len(e.tokens) for e in entries], dtype=np.int64)
@@ -184,14 +216,22 @@ class ModelRunner:
         n = int(lens.sum())
         rps = [cache.get(e.rid) for e in entries]
         pos0 = np.array([rp.length for rp in rps], dtype=np.int64)
-        start = np.zeros(n_entries + 1, dtype=np.int64)
-        np.cumsum(lens, out=start[1:])
-        tok_entry = np.repeat(np.arange(n_entries), lens)
-        positions = np.arange(n) - start[:-1][tok_entry] + pos0[tok_entry]
         ids = np.fromiter((t for e in entries for t in e.tokens), dtype=np.int64, count=n)
-        if ids.size and (ids.min() < 0 or ids.max() >= self.vocab_size):
+        if ids.min() < 0 or ids.max() >= self.vocab_size:
             bad = ids[(ids < 0) | (ids >= self.vocab_size)][0]
             raise ValueError(f"token id {int(bad)} is outside the vocabulary of {self.vocab_size}")
+        slots = np.array([rp.slot for rp in rps], dtype=np.int64)
+        n_pad = max(0, pad_to - n_entries)   # padding entries: one token at position 0 with no pages
+        if n_pad:
+            lens = np.concatenate([lens, np.ones(n_pad, np.int64)])
+            pos0 = np.concatenate([pos0, np.zeros(n_pad, np.int64)])
+            ids = np.concatenate([ids, np.zeros(n_pad, np.int64)])
+            slots = np.concatenate([slots, np.zeros(n_pad, np.int64)])
+        n_all = n_entries + n_pad
+        start = np.zeros(n_all + 1, dtype=np.int64)
+        np.cumsum(lens, out=start[1:])
+        tok_entry = np.repeat(np.arange(n_all), lens)
+        positions = np.arange(n + n_pad) - start[:-1][tok_entry] + pos0[tok_entry]
         rows = []
         for i, e in enumerate(entries):
             for w in e.want:
@@ -199,31 +239,37 @@ class ModelRunner:
                     raise ValueError(f"request {e.rid!r}: wanted place {w} is not among its {lens[i]} tokens")
                 rows.append(start[i] + w)
         new_len = pos0 + lens
-        max_blocks = int(-(-new_len.max() // ps))
-        max_blocks = -(-max_blocks // 8) * 8
+        if fixed_blocks:
+            max_blocks = fixed_blocks
+        else:
+            max_blocks = int(-(-new_len.max() // ps))
+            max_blocks = -(-max_blocks // 8) * 8
         tables = []
         for gi in range(self.storage.n_groups):
-            bt = np.full((n_entries, max_blocks), NO_PAGE, dtype=np.int32)
+            bt = np.full((n_all, max_blocks), NO_PAGE, dtype=np.int32)
             for i, rp in enumerate(rps):
                 t = rp.tables[gi]
                 bt[i, :len(t)] = t
             tables.append(bt)
+        return dict(n=n + n_pad, n_entries=n_all, ids=ids.astype(np.int32), positions=positions.astype(np.int32),
+                    tok_entry=tok_entry.astype(np.int32), start=start.astype(np.int32), pos0=pos0.astype(np.int32),
+                    slots=slots.astype(np.int32), rows=np.array(rows, dtype=np.int32), tables=tables,
+                    fresh=[rp.fresh for rp in rps] + [False] * n_pad, kv_lens=new_len, max_blocks=max_blocks)
 
-        ctx = StepContext(self.rt, self.max_seq_len)
-        ctx.n_tokens, ctx.n_entries, ctx.n_logit_rows = n, n_entries, len(rows)
-        ctx.h_token_ids = ids.astype(np.int32)
-        ctx.h_positions = positions.astype(np.int32)
-        ctx.h_tok_entry = tok_entry.astype(np.int32)
-        ctx.h_entry_start = start.astype(np.int32)
-        ctx.h_entry_pos0 = pos0.astype(np.int32)
-        ctx.h_state_slots = np.array([rp.slot for rp in rps], dtype=np.int32)
-        ctx.h_logit_rows = np.array(rows, dtype=np.int32)
-        ctx.h_block_tables = tables
-        ctx.fresh = [rp.fresh for rp in rps]
+    def _fill_context(self, ctx: StepContext, h: dict, rows: np.ndarray, dev: torch.Tensor, decode: bool) -> None:
+        """Lay the host arrays out in one int32 buffer, copy it to `dev`, and point the context at the pieces."""
+        ctx.n_tokens, ctx.n_entries, ctx.n_logit_rows = h["n"], h["n_entries"], len(rows)
+        ctx.h_token_ids, ctx.h_positions, ctx.h_tok_entry = h["ids"], h["positions"], h["tok_entry"]
+        ctx.h_entry_start, ctx.h_entry_pos0, ctx.h_state_slots = h["start"], h["pos0"], h["slots"]
+        ctx.h_logit_rows, ctx.h_block_tables, ctx.fresh = rows, h["tables"], h["fresh"]
+        dec = np.zeros(4, np.int32)
+        if decode:
+            dec[0] = decode_chunk(h["kv_lens"], self.decode_p_max)
         parts = [ctx.h_token_ids, ctx.h_positions, ctx.h_tok_entry, ctx.h_entry_start, ctx.h_entry_pos0,
-                 ctx.h_state_slots, ctx.h_logit_rows] + [t.reshape(-1) for t in tables]
+                 ctx.h_state_slots, ctx.h_logit_rows, dec] + [t.reshape(-1) for t in h["tables"]]
         flat = np.concatenate(parts)
-        dev = self.rt.buffer("step.meta", (flat.size,), torch.int32)
+        if dev.numel() != flat.size:
+            raise RuntimeError("step metadata does not fit its device buffer")
         dev.copy_(torch.from_numpy(flat))
         views, off = [], 0
         for p in parts:
@@ -231,7 +277,20 @@ class ModelRunner:
             off += p.size
         (ctx.token_ids, ctx.positions, ctx.tok_entry, ctx.entry_start, ctx.entry_pos0, ctx.state_slots,
          ctx.logit_rows) = views[:7]
-        ctx.block_tables = [v.view(n_entries, max_blocks) for v in views[7:]]
+        ctx.decode_params = views[7] if decode else None
+        ctx.decode_p_max = self.decode_p_max if decode else 0
+        ctx.block_tables = [v.view(h["n_entries"], h["max_blocks"]) for v in views[8:]]
+
+    def _meta_size(self, h: dict, n_rows: int) -> int:
+        return 3 * h["n"] + (h["n_entries"] + 1) + 2 * h["n_entries"] + n_rows + 4 + \
+            self.storage.n_groups * h["n_entries"] * h["max_blocks"]
+
+    def build_context(self, entries: Sequence[StepEntry]) -> StepContext:
+        h = self._host_arrays(entries)
+        decode = self.rt.dtype == torch.bfloat16 and all(len(e.tokens) == 1 for e in entries)
+        ctx = StepContext(self.rt, self.max_seq_len)
+        dev = self.rt.buffer("step.meta", (self._meta_size(h, len(h["rows"])),), torch.int32)
+        self._fill_context(ctx, h, h["rows"], dev, decode)
         return ctx
 
     def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
@@ -247,11 +306,47 @@ class ModelRunner:
             raise OutOfPages(f"the step needs more pages than are free ({cache.available_pages()} free per group)")
         fresh_slots = [cache.get(e.rid).slot for e in entries if cache.get(e.rid).fresh]
         self.storage.clear_state(fresh_slots)
-        ctx = self.build_context(entries)
-        caches = self.storage.layer_caches(ctx.block_tables)
-        logits = self.model.forward(ctx, caches, self.storage.state)
+        use_graph = (self.decode_graphs and self._stateless and self.rt.dtype == torch.bfloat16
+                     and len(entries) <= GRAPH_BATCHES[-1] and all(len(e.tokens) == 1 for e in entries))
+        if use_graph:
+            logits = self._step_decode_graph(entries)
+        else:
+            ctx = self.build_context(entries)
+            caches = self.storage.layer_caches(ctx.block_tables)
+            logits = self.model.forward(ctx, caches, self.storage.state)
         for rid, new_len in targets:
             cache.commit(rid, new_len)
         self.steps += 1
-        self.tokens += ctx.n_tokens
+        self.tokens += sum(len(e.tokens) for e in entries)
         return logits
+
+    # -- decoding through a captured graph ---------------------------------------
+    def _step_decode_graph(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        n = len(entries)
+        b = next(x for x in GRAPH_BATCHES if x >= n)
+        fixed_blocks = -(-self.max_seq_len // self.cache.page_size)
+        h = self._host_arrays(entries, pad_to=b, fixed_blocks=fixed_blocks)
+        all_rows = np.arange(b, dtype=np.int32)     # logits of every entry; the wanted ones are picked afterwards
+        g = self._graphs.get(b)
+        with self.rt.scoped(f"graph{b}:"):
+            if g is None:
+                g = _DecodeGraph()
+                g.meta = self.rt.buffer("step.meta", (self._meta_size(h, b),), torch.int32)
+                g.ctx = StepContext(self.rt, self.max_seq_len)
+                self._fill_context(g.ctx, h, all_rows, g.meta, decode=True)
+                caches = self.storage.layer_caches(g.ctx.block_tables)
+                # once eagerly: loads the libraries and makes every scratch buffer, so the capture allocates nothing
+                self.model.forward(g.ctx, caches, self.storage.state)
+                torch.cuda.synchronize()
+                g.graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g.graph):
+                    g.logits = self.model.forward(g.ctx, caches, self.storage.state)
+                self._graphs[b] = g
+            else:
+                self._fill_context(g.ctx, h, all_rows, g.meta, decode=True)
+            g.graph.replay()
+        if len(h["rows"]) == 0:
+            return None
+        if (h["rows"] == all_rows[:len(h["rows"])]).all():
+            return g.logits[:len(h["rows"])]     # the first entries in order: a view, no copy
+        return g.logits.index_select(0, torch.from_numpy(h["rows"].astype(np.int64)).to(self.rt.device))

@@ -114,6 +114,12 @@ class PagedAttention(Part):
         if rt.dtype == torch.float32:
             ops.attention_f32(q, cache.k, cache.v, ctx.positions, ctx.tok_entry, cache.block_table, out, nh, nkv, d,
                               self.window, self.scale)
+        elif ctx.decode_params is not None and nh // nkv <= 16:
+            # one token per entry: the kernel cuts the keys itself from the positions on the device
+            part_o = rt.buffer("attn.dec_part_o", (n * ctx.decode_p_max * nkv * 16 * d,), torch.float32)
+            part_ml = rt.buffer("attn.dec_part_ml", (n * ctx.decode_p_max * nkv * 32,), torch.float32)
+            ops.attention_bf16_decode(q, cache.k, cache.v, cache.block_table, ctx.entry_pos0, ctx.decode_params,
+                                      ctx.decode_p_max, out, part_o, part_ml, nh, nkv, d, self.window, self.scale)
         else:
             plan = ctx.attention_plan(nh // nkv, self.window, nkv, d)
             ops.attention_bf16(q, cache.k, cache.v, cache.block_table, plan.items, plan.n_items, plan.citems,

@@ -77,6 +77,7 @@ class Runtime:
         self.device = device
         self.dtype = dtype
         self._buffers: Dict[str, torch.Tensor] = {}
+        self._scope = ""
 
     def place(self, t: torch.Tensor, role: str) -> torch.Tensor:
         """A loaded tensor as the kernels want it, on the device."""
@@ -95,11 +96,30 @@ class Runtime:
         n = 1
         for s in shape:
             n *= int(s)
+        name = self._scope + name
         buf = self._buffers.get(name)
         if buf is None or buf.dtype != dtype or buf.numel() < n:
+            if self._scope and torch.cuda.is_current_stream_capturing():
+                raise RuntimeError(f"scratch buffer '{name}' would be allocated while a graph is being captured")
             buf = torch.empty(max(n, 1), dtype=dtype, device=self.device)
             self._buffers[name] = buf
         return buf[:n].view(*shape)
+
+    def scoped(self, prefix: str):
+        """Scratch buffers asked for inside this context are a set of their own: a captured graph keeps the
+        addresses of its buffers, so they must never be regrown by steps of another shape."""
+        rt = self
+
+        class _Scope:
+            def __enter__(self_inner):
+                self_inner.prev = rt._scope
+                rt._scope = prefix
+                return rt
+
+            def __exit__(self_inner, *exc):
+                rt._scope = self_inner.prev
+                return False
+        return _Scope()
 
 
 class Part:
