@@ -222,11 +222,26 @@ def test_chunked_prompts_mixed_with_decoding_and_temperature(model_folders):
     for i, p in enumerate(prompts):
         alone = Engine(model_folders[cfg], dtype="float32", num_pages=8, max_running_reqs=1, max_seq_len=128)
         assert alone.generate([p], [sp[i]])[0] == got[i]
-    # so few pages that decoding requests are preempted and recomputed: still the same tokens
-    tight = Engine(model_folders[cfg], dtype="float32", num_pages=5, max_running_reqs=4, max_seq_len=128,
-                   chunk_size=8, max_extend_tokens=12)
-    assert tight.generate(prompts, sp) == got
+
+
+def test_preemption_recomputes_the_same_tokens(model_folders):
+    """Three pages for two requests that each grow into a second page while decoding: the younger one is
+    preempted, gives its pages back, waits, and is recomputed from its prompt and the tokens it had produced.
+    Its tokens are those it produces alone."""
+    from vt_transformer_amd.engine import Engine
+    from vt_transformer_amd.sampling import SamplingParams
+    cfg = "B"
+    prompts = list(random_requests(TINY[cfg]["vocab_size"], [15, 16], seed=23).values())
+    sp = [SamplingParams(temperature=0.8, max_tokens=8, ignore_eos=True, seed=2000 + i) for i in range(2)]
+    alone = []
+    for i, p in enumerate(prompts):
+        eng = Engine(model_folders[cfg], dtype="float32", num_pages=4, max_running_reqs=1, max_seq_len=128)
+        alone.append(eng.generate([p], [sp[i]])[0])
+    tight = Engine(model_folders[cfg], dtype="float32", num_pages=3, max_running_reqs=4, max_seq_len=128)
+    assert tight.generate(prompts, sp) == alone
     assert tight.scheduler.counters["preemptions"] > 0
+    assert tight.requests[1].preemptions > 0 and tight.requests[0].preemptions == 0
+    assert sum(tight.runner.cache.held_pages()) == 0
 
 
 def test_decode_graph_replays_match_eager(model_folders):
