@@ -1,0 +1,65 @@
+"""Host-side pieces of the step: the attention work planner, the decode chunk, the sampler's uniform numbers."""
+import numpy as np
+import pytest
+
+from vt_transformer_amd.engine.step import decode_chunk, plan_attention_items
+from vt_transformer_amd.sampling import SamplingParams, request_seed, uniform
+
+
+@pytest.mark.parametrize("group,window", [(1, 0), (7, 0), (2, 5), (5, 40), (3, 16)])
+@pytest.mark.parametrize("target", [0, 2048, 10 ** 9])
+def test_every_row_gets_every_key_it_may_see_exactly_once(group, window, target):
+    lens = np.array([1, 37, 1, 2, 19, 130])
+    pos0 = np.array([300, 0, 0, 16, 45, 7])
+    start = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    items, citems, n_parts = plan_attention_items(start, pos0.astype(np.int32), group, window, 2, target_waves=target,
+                                                  min_chunk=16)
+    covered = {}
+    for entry, q_tok0, q_len, p0, row0, lo, hi, part in items.tolist():
+        assert q_tok0 == start[entry] and q_len == lens[entry] and p0 == pos0[entry]
+        assert lo % 16 == 0 and lo < hi
+        for r in range(row0, min(row0 + 16, q_len * group)):
+            p = p0 + r // group
+            first = max(0, p - window + 1) if window else 0
+            keys = covered.setdefault((entry, r), [])
+            keys.extend(j for j in range(lo, hi) if first <= j <= p)
+    for e in range(len(lens)):
+        for r in range(lens[e] * group):
+            p = pos0[e] + r // group
+            first = max(0, p - window + 1) if window else 0
+            assert sorted(covered[(e, r)]) == list(range(first, p + 1)), (e, r)
+    # partial slots: each used by one item; every split tile is merged once over exactly its slots
+    parts = [it[7] for it in items.tolist() if it[7] >= 0]
+    assert len(parts) == len(set(parts)) and all(p < n_parts for p in parts)
+    merged = sorted(p for c in citems.tolist() for p in range(c[3], c[3] + c[4]))
+    assert merged == sorted(parts)
+    if target == 0:
+        assert len(citems) == 0
+
+
+def test_decode_chunk():
+    assert decode_chunk(np.array([1]), 64) == 64
+    assert decode_chunk(np.array([8192]), 64) % 16 == 0 and decode_chunk(np.array([8192]), 64) * 64 >= 8192
+    c = decode_chunk(np.full(64, 1024), 64)
+    assert c % 16 == 0 and 64 <= c <= 128
+
+
+def test_uniform_numbers_depend_only_on_seed_and_counter():
+    a = [uniform(5, i) for i in range(2000)]
+    assert a == [uniform(5, i) for i in range(2000)]
+    assert all(0.0 <= x < 1.0 for x in a)
+    assert abs(np.mean(a) - 0.5) < 0.03 and abs(np.var(a) - 1 / 12) < 0.01
+    assert np.float32(a[7]) == a[7]                       # exact in float32
+    assert uniform(6, 0) != uniform(5, 0)
+    assert request_seed(1, "a") != request_seed(1, "b") and request_seed(1, "a") == request_seed(1, "a")
+
+
+def test_sampling_params_follow_the_front_end():
+    """sglfront/sglfront/core.py:6-16."""
+    p = SamplingParams()
+    assert (p.temperature, p.top_k, p.top_p, p.ignore_eos, p.max_tokens) == (0.0, -1, 1.0, False, 1024)
+    assert p.is_greedy and SamplingParams(temperature=0.7, top_k=1).is_greedy
+    assert not SamplingParams(temperature=0.7).is_greedy and not SamplingParams(top_p=0.9).is_greedy
+    for bad in (dict(top_p=0.0), dict(top_k=0), dict(max_tokens=0)):
+        with pytest.raises(ValueError):
+            SamplingParams(**bad)

@@ -1,0 +1,197 @@
+"""The scheduler's decisions, driven without a GPU: a stand-in for the step function reserves and commits pages
+as the real one does and hands out made-up tokens."""
+import random
+
+import pytest
+
+from vt_transformer_amd.cache import CacheManager, GroupSpec
+from vt_transformer_amd.engine.scheduler import (FINISHED, RUNNING, WAITING, Request, Scheduler, SchedulerConfig)
+from vt_transformer_amd.sampling import SamplingParams
+
+EOS = 7
+
+
+class FakeEngine:
+    """Scheduler + cache manager + a step that only does the bookkeeping of the real step function."""
+
+    def __init__(self, num_pages=64, page_size=4, windows=(0,), token=lambda req: 1, **cfg):
+        self.cfg = SchedulerConfig(num_pages=num_pages, page_size=page_size, **cfg)
+        self.cache = CacheManager([GroupSpec(i, w, num_pages) for i, w in enumerate(windows)], page_size,
+                                  self.cfg.max_running_reqs, self.cfg.max_seq_len)
+        self.sched = Scheduler(self.cfg, self.cache, [EOS])
+        self.token = token
+        self.plans = []
+
+    def add(self, uid, n_prompt, **sp):
+        r = Request(uid, list(range(10, 10 + n_prompt)), SamplingParams(**sp))
+        self.sched.add_request(r)
+        return r
+
+    def step(self):
+        plan = self.sched.schedule()
+        self.plans.append([(s.request.uid, s.start, s.n_tokens, s.sample) for s in plan])
+        if plan:
+            items = [(s.request.uid, s.start + s.n_tokens) for s in plan]
+            assert self.cache.reserve(items), "the scheduler chose a step that the cache cannot hold"
+            for uid, n in items:
+                self.cache.commit(uid, n)
+        sampled = {s.request.uid: self.token(s.request) for s in plan if s.sample}
+        out = self.sched.update(plan, sampled)
+        self.cache.check()
+        return out
+
+    def run(self, limit=10000):
+        results = []
+        for _ in range(limit):
+            if not self.sched.has_work():
+                break
+            results.extend(self.step())
+        assert not self.sched.has_work(), "the scheduler did not finish"
+        return results
+
+
+def test_three_decode_steps_give_three_results_none_finished():
+    """vt-transformer/test/vt_backend_test.cpp:313-333."""
+    e = FakeEngine()
+    r = e.add("a", 5, max_tokens=10)
+    first = e.step()                       # the prompt: its last logits give the first token
+    assert [(x.uid, x.finished) for x in first] == [("a", False)]
+    for _ in range(3):
+        res = e.step()
+        assert len(res) == 1 and res[0].uid == "a" and not res[0].finished
+    # request bookkeeping of vt_request.hpp:12-33: the newest output token is not in the cache yet
+    assert len(r.output) == 4 and r.computed == r.total_len - 1 and r.decoding
+    assert e.plans[0] == [("a", 0, 5, True)] and e.plans[1] == [("a", 5, 1, True)]
+
+
+def test_finish_on_end_token_or_output_limit():
+    """vt_scheduler.cpp:431-437."""
+    e = FakeEngine(token=lambda r: EOS if len(r.output) == 2 else 1)
+    a = e.add("a", 3, max_tokens=10)
+    b = e.add("b", 3, max_tokens=10, ignore_eos=True)
+    c = e.add("c", 3, max_tokens=2)
+    res = e.run()
+    assert (a.finish_reason, len(a.output)) == ("eos", 3)
+    assert (b.finish_reason, len(b.output)) == ("max_tokens", 10)
+    assert (c.finish_reason, len(c.output)) == ("max_tokens", 2)
+    assert sum(1 for r in res if r.finished) == 3
+    assert e.cache.held_pages() == [0] and e.cache.slots.available == e.cfg.max_running_reqs
+
+
+def test_context_length_stops_a_request():
+    e = FakeEngine(max_seq_len=12)
+    a = e.add("a", 8, max_tokens=100)
+    e.run()
+    assert a.finish_reason == "max_seq_len" and a.total_len == 12
+
+
+def test_abort_frees_and_gives_no_further_results():
+    """vt_backend_test.cpp:338-360."""
+    e = FakeEngine()
+    e.add("a", 6, max_tokens=50)
+    e.add("b", 6, max_tokens=50)
+    e.step(); e.step()
+    assert e.sched.abort_request("a")
+    assert e.cache.held_pages()[0] == sum(1 for p in e.cache.get("b").tables[0] if p >= 0)   # only b holds pages
+    for _ in range(3):
+        assert all(r.uid == "b" for r in e.step())
+    assert not e.sched.abort_request("zzz")
+    e.add("c", 3)
+    assert e.sched.abort_request("c")            # still waiting: just leaves the line
+    assert e.sched.abort_request("b")
+    assert not e.sched.has_work() and e.cache.held_pages() == [0]
+
+
+def test_prompts_are_cut_under_the_token_budget_and_decoding_goes_first():
+    e = FakeEngine(num_pages=256, max_extend_tokens=10, chunk_size=6)
+    e.add("a", 4, max_tokens=20)
+    e.step()                                        # a: whole prompt
+    e.add("b", 20, max_tokens=20)
+    e.step()
+    # a decodes (1 token) and b gets a portion of at most chunk_size within what is left of the budget
+    assert e.plans[1] == [("a", 4, 1, True), ("b", 0, 6, False)]
+    e.add("c", 9, max_tokens=20)
+    e.step()
+    # budget 10: a 1, b 6 (older), c the 3 that are left
+    assert e.plans[2] == [("a", 5, 1, True), ("b", 6, 6, False), ("c", 0, 3, False)]
+    e.step()
+    assert e.plans[3] == [("a", 6, 1, True), ("b", 12, 6, False), ("c", 3, 3, False)]
+    e.step()
+    # b's last portion is short and ends at its newest token: it samples
+    assert e.plans[4] == [("a", 7, 1, True), ("b", 18, 2, True), ("c", 6, 3, True)]
+    assert all(sum(n for _, _, n, _ in p) <= 10 for p in e.plans)
+
+
+def test_running_requests_are_bounded_by_slots():
+    e = FakeEngine(max_running_reqs=2)
+    for i in range(5):
+        e.add(i, 3, max_tokens=3)
+    e.step()
+    assert len(e.sched.running) == 2 and len(e.sched.waiting) == 3
+    e.run()
+    assert all(e.sched.counters[k] >= 0 for k in e.sched.counters)
+
+
+def test_when_pages_run_out_the_youngest_is_preempted_and_recomputed():
+    # 3 pages of 4: two prompts of 4 tokens take one page each; both then need a second page
+    e = FakeEngine(num_pages=3, page_size=4)
+    a = e.add("a", 4, max_tokens=6)
+    b = e.add("b", 4, max_tokens=6)
+    e.step()
+    assert len(e.sched.running) == 2
+    e.step()                                        # both try to decode: a gets the last page, b must go
+    assert b.state == WAITING and b.preemptions == 1 and b.computed == 0 and len(b.output) == 1
+    assert e.sched.waiting[0] is b                  # at the head of the line
+    assert e.cache.held_pages() == [2]
+    e.run()
+    assert (a.finish_reason, b.finish_reason) == ("max_tokens", "max_tokens")
+    assert len(a.output) == 6 and len(b.output) == 6
+    assert a.preemptions == 0
+    # b was recomputed from its prompt and what it had produced: one portion of 5 tokens that samples
+    assert any(p == [("b", 0, 5, True)] for p in e.plans)
+    assert e.cache.held_pages() == [0]
+
+
+def test_a_request_that_can_never_fit_is_refused_not_waited_for():
+    e = FakeEngine(num_pages=2, page_size=4, max_seq_len=100)       # the pool holds 8 tokens
+    big = e.add("big", 9)
+    ok = e.add("ok", 3, max_tokens=2)
+    res = e.run()
+    assert big.state == FINISHED and big.finish_reason == "too_long"
+    assert [r for r in res if r.uid == "big"][0].finished and [r for r in res if r.uid == "big"][0].next_token is None
+    assert ok.finish_reason == "max_tokens"
+    e2 = FakeEngine(max_seq_len=8)
+    long = e2.add("long", 9)
+    e2.run()
+    assert long.finish_reason == "too_long"
+
+
+def test_a_lone_request_that_outgrows_the_pool_ends_with_an_error():
+    e = FakeEngine(num_pages=2, page_size=4)
+    a = e.add("a", 6, max_tokens=50)
+    e.run()
+    assert a.finish_reason == "out_of_pages" and a.total_len == 9    # 8 tokens in the cache, the 9th had no page
+    assert e.cache.held_pages() == [0]
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_load_always_drains(seed):
+    rng = random.Random(seed)
+    e = FakeEngine(num_pages=rng.randint(8, 30), page_size=rng.choice([2, 4, 16]), windows=(0, rng.choice([0, 6])),
+                   max_running_reqs=rng.randint(1, 6), max_extend_tokens=rng.randint(4, 40), chunk_size=rng.randint(2, 16),
+                   max_seq_len=64, token=lambda r: rng.choice([1, 2, 3, EOS]))
+    reqs = []
+    for step in range(300):
+        if rng.random() < 0.3:
+            reqs.append(e.add(len(reqs), rng.randint(1, 40), max_tokens=rng.randint(1, 12),
+                              ignore_eos=rng.random() < 0.3))
+        if rng.random() < 0.05 and reqs:
+            e.sched.abort_request(rng.choice(reqs).uid)
+        e.step()
+    e.run()
+    assert all(r.state == FINISHED for r in reqs)
+    assert all(r.finish_reason in ("eos", "max_tokens", "max_seq_len", "abort", "too_long", "out_of_pages") for r in reqs)
+    assert e.cache.held_pages() == [0, 0]
+    for r in reqs:
+        if r.finish_reason == "max_tokens":
+            assert len(r.output) == r.params.max_tokens

@@ -9,6 +9,7 @@ else is in the batch and however often it was preempted.
 """
 from __future__ import annotations
 
+import hashlib
 from typing import List, Sequence, Tuple
 
 import numpy as np
@@ -36,7 +37,9 @@ def uniform(seed: int, counter: int) -> float:
 
 
 def request_seed(engine_seed: int, request_key) -> int:
-    return _splitmix64((engine_seed & _M64) ^ _splitmix64(hash(str(request_key)) & _M64))
+    """The same for the same (engine seed, request id) in every process (Python's own hash of a string is not)."""
+    key = int.from_bytes(hashlib.sha256(str(request_key).encode()).digest()[:8], "little")
+    return _splitmix64((engine_seed & _M64) ^ _splitmix64(key))
 
 
 class Sampler:
