@@ -227,6 +227,8 @@ class CacheManager:
     def available_tokens(self) -> int:
         """Tokens that still fit, in the reference's unit (pages x page size, vt_cache.hpp:54-57),
         for the group with the fewest free pages."""
+        if not self.pools:
+            return self.max_seq_len * self.slots.n     # no layer keeps pages: nothing to run out of
         return min(p.available for p in self.pools) * self.page_size
 
     def held_pages(self) -> List[int]:

@@ -126,6 +126,8 @@ class Scheduler:
 
     # -- one step's decisions ------------------------------------------------
     def _capacity_tokens(self) -> int:
+        if not self.cache.pools:
+            return self.config.max_seq_len
         return min(p.num_pages for p in self.cache.pools) * self.cache.page_size
 
     def _fits(self, items: List[Tuple[Request, int]]) -> bool:
@@ -213,7 +215,7 @@ class Scheduler:
                 self.cache.release(r.uid)
                 if not self.running and not plan:
                     # nothing else holds pages and it still does not fit: cut the portion to what fits
-                    n_fit = min(n, min(p.available for p in self.cache.pools) * self.cache.page_size)
+                    n_fit = min(n, self.cache.available_tokens())
                     if n_fit <= 0:
                         self.waiting.popleft()
                         self._refuse(r, "out_of_pages")

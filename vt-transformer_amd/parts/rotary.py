@@ -1,13 +1,15 @@
 """Rotary position encoding: the table of angles.
 
-As the reference builds it on the host (v1/tensortype/common.cpp:6-24):
-inv_freq[i] = 1 / base^(2i/D) for i < D/2, rounded to float; the angle of
-position l is l * inv_freq[i], computed in double and rounded to float; cosine
-and sine of that float angle, computed in double and rounded to float.  Dims i
+The reference builds it on the host (v1/tensortype/common.cpp:6-24):
+inv_freq[i] = 1 / base^(2i/D) for i < D/2, the angle of position l is
+l * inv_freq[i], and the table holds its cosine and sine as floats.  Dims i
 and i + D/2 share an angle and form a rotated pair
 (v1/tensortype/hip_kernels/rotary_embed.cpp:20-26); the rotation itself is
 fused into the kernel that writes keys and values into their pages.
 
+The reference rounds inv_freq and the angle to float before taking cosine
+and sine, which costs about position * 1e-7 radians; here everything up to
+the final cosine and sine is computed in double and rounded to float once.
 The reference's table has 10000 rows (v1/models/qwen2-7b/inference_fp16.dag:38);
 here it has as many as the longest sequence the engine is set up for.
 """
@@ -24,10 +26,9 @@ from .base import POSITIONS, Part, Runtime
 def rotary_table(n_positions: int, dims: int, theta: float) -> Tuple[np.ndarray, np.ndarray]:
     """(cos, sin), float32 [n_positions, dims/2]."""
     i = np.arange(0, dims, 2, dtype=np.float64)
-    inv = (1.0 / np.power(np.float64(theta), i / dims)).astype(np.float32)
-    ang = (np.arange(n_positions, dtype=np.float64)[:, None] * inv.astype(np.float64)[None, :]).astype(np.float32)
-    a64 = ang.astype(np.float64)
-    return np.cos(a64).astype(np.float32), np.sin(a64).astype(np.float32)
+    inv = 1.0 / np.power(np.float64(theta), i / dims)
+    ang = np.arange(n_positions, dtype=np.float64)[:, None] * inv[None, :]
+    return np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
 
 
 @POSITIONS.register("rotary")
