@@ -247,18 +247,20 @@ def attention_case(dtype, nh, kvh, d, page_size, window, entries, seed, spike=Fa
         from vt_transformer_amd.engine.step import plan_attention_items
         start = np.cumsum([0] + [n for _, n in entries]).astype(np.int32)
         pos0 = np.array([c for c, _ in entries], dtype=np.int32)
-        for target in (2048, 10 ** 9):   # without and with the keys split over several items
+        first = None
+        for target, rt in ((0, 1), (10 ** 9, 1), (0, 2), (10 ** 9, 4), (0, 4)):   # keys unsplit and split; 1, 2, 4 row tiles
             items, citems, n_parts = plan_attention_items(start, pos0, nh // kvh, window, kvh, target_waves=target,
-                                                          min_chunk=16)
-            part_o = torch.full((max(1, n_parts) * kvh * 16 * d,), float("nan"), device=DEV)
-            part_ml = torch.full((max(1, n_parts) * kvh * 32,), float("nan"), device=DEV)
+                                                          min_chunk=16, rt=rt)
+            part_o = torch.full((max(1, n_parts) * rt * kvh * 16 * d,), float("nan"), device=DEV)
+            part_ml = torch.full((max(1, n_parts) * rt * kvh * 32,), float("nan"), device=DEV)
             out.fill_(float("nan"))
             o.attention_bf16(q, kp.to(DEV), vp.to(DEV), bt.to(DEV), torch.from_numpy(items).to(DEV).reshape(-1),
                              items.shape[0], torch.from_numpy(citems).to(DEV).reshape(-1) if len(citems) else None,
-                             len(citems), out, part_o, part_ml, nh, kvh, d, window, scale, max_part=n_parts)
-            if target == 2048:
+                             len(citems), out, part_o, part_ml, nh, kvh, d, window, scale, max_part=n_parts, rt=rt)
+            if first is None:
                 first = out.clone()
-        assert rel_err(out, first) < 1e-2  # split and unsplit agree to rounding
+            assert bool(torch.isfinite(out).all()), (target, rt)
+            assert rel_err(out, first) < 1e-2, (target, rt)  # every way of cutting the work agrees to rounding
     ref = torch.cat([ref_attention(qs[e][i], ks[e], vs[e], c + i, window, scale).reshape(1, -1)
                      for e, (c, n) in enumerate(entries) for i in range(n)])
     return out, ref
@@ -431,3 +433,32 @@ def test_sample_top_k_and_top_p():
     assert set(_draw(logits, 1e-4, -1, 1.0, 100, 3).tolist()) == {int(order[0])}
     # top_k = 1 is greedy whatever the temperature
     assert set(_draw(logits, 5.0, 1, 1.0, 100, 4).tolist()) == {int(order[0])}
+
+
+@pytest.mark.parametrize("nh,kvh,d", [(28, 4, 128), (4, 2, 16), (16, 1, 48)])
+@pytest.mark.parametrize("window", [0, 37])
+@pytest.mark.parametrize("chunk", [16, 64, 256])
+def test_attention_decode_kernel(nh, kvh, d, window, chunk):
+    """One token per entry, the keys cut into items on the device from the positions in memory."""
+    o = ops()
+    g = torch.Generator().manual_seed(nh + d + chunk)
+    cached = [0, 15, 16, 17, 300, 63, 1000]
+    lens = [c + 1 for c in cached]
+    ks = [torch.randn(t, kvh, d, generator=g).to(torch.bfloat16).float() for t in lens]
+    vs = [torch.randn(t, kvh, d, generator=g).to(torch.bfloat16).float() for t in lens]
+    qs = [torch.randn(1, nh, d, generator=g).to(torch.bfloat16).float() for _ in lens]
+    kp, vp, bt = make_pages(ks, vs, lens, 16, torch.bfloat16, 9)
+    n = len(lens)
+    q = torch.cat(qs).reshape(n, nh * d).to(torch.bfloat16).to(DEV)
+    p_max = 64
+    if -(-max(lens) // chunk) > p_max:
+        pytest.skip("the host never chooses a chunk that needs more items than p_max")
+    part_o = torch.full((n * p_max * kvh * 16 * d,), float("nan"), device=DEV)
+    part_ml = torch.full((n * p_max * kvh * 32,), float("nan"), device=DEV)
+    out = torch.full((n, nh * d), float("nan"), dtype=torch.bfloat16, device=DEV)
+    scale = 1.0 / math.sqrt(d)
+    o.attention_bf16_decode(q, kp.to(DEV), vp.to(DEV), bt.to(DEV), torch.tensor(cached, dtype=torch.int32, device=DEV),
+                            torch.tensor([chunk, 0, 0, 0], dtype=torch.int32, device=DEV), p_max, out, part_o, part_ml,
+                            nh, kvh, d, window, scale)
+    ref = torch.cat([ref_attention(qs[e][0], ks[e], vs[e], cached[e], window, scale).reshape(1, -1) for e in range(n)])
+    assert rel_err(out, ref) < ATT_TOL[torch.bfloat16]

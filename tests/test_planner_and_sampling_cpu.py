@@ -8,17 +8,18 @@ from vt_transformer_amd.sampling import SamplingParams, request_seed, uniform
 
 @pytest.mark.parametrize("group,window", [(1, 0), (7, 0), (2, 5), (5, 40), (3, 16)])
 @pytest.mark.parametrize("target", [0, 2048, 10 ** 9])
-def test_every_row_gets_every_key_it_may_see_exactly_once(group, window, target):
+@pytest.mark.parametrize("rt", [1, 2, 4])
+def test_every_row_gets_every_key_it_may_see_exactly_once(group, window, target, rt):
     lens = np.array([1, 37, 1, 2, 19, 130])
     pos0 = np.array([300, 0, 0, 16, 45, 7])
     start = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
     items, citems, n_parts = plan_attention_items(start, pos0.astype(np.int32), group, window, 2, target_waves=target,
-                                                  min_chunk=16)
+                                                  min_chunk=16, rt=rt)
     covered = {}
     for entry, q_tok0, q_len, p0, row0, lo, hi, part in items.tolist():
         assert q_tok0 == start[entry] and q_len == lens[entry] and p0 == pos0[entry]
         assert lo % 16 == 0 and lo < hi
-        for r in range(row0, min(row0 + 16, q_len * group)):
+        for r in range(row0, min(row0 + 16 * rt, q_len * group)):
             p = p0 + r // group
             first = max(0, p - window + 1) if window else 0
             keys = covered.setdefault((entry, r), [])
@@ -28,11 +29,20 @@ def test_every_row_gets_every_key_it_may_see_exactly_once(group, window, target)
             p = pos0[e] + r // group
             first = max(0, p - window + 1) if window else 0
             assert sorted(covered[(e, r)]) == list(range(first, p + 1)), (e, r)
-    # partial slots: each used by one item; every split tile is merged once over exactly its slots
+    # partial indices: each used by one item; every 16-row tile of a split item is merged once over exactly its items
     parts = [it[7] for it in items.tolist() if it[7] >= 0]
     assert len(parts) == len(set(parts)) and all(p < n_parts for p in parts)
-    merged = sorted(p for c in citems.tolist() for p in range(c[3], c[3] + c[4]))
-    assert merged == sorted(parts)
+    by_part = {it[7]: it for it in items.tolist() if it[7] >= 0}
+    merged = {}
+    for q_tok0, q_len, r0, part0, n, sub in citems.tolist():
+        assert 2 <= n <= 128 and 0 <= sub < rt
+        for pi in range(part0, part0 + n):
+            it = by_part[pi]
+            assert it[1] == q_tok0 and it[4] + 16 * sub == r0 and r0 < q_len * group
+            merged.setdefault(pi, []).append(sub)
+    for pi, it in by_part.items():
+        tiles = [s_ for s_ in range(rt) if it[4] + 16 * s_ < it[2] * group]
+        assert sorted(merged[pi]) == tiles
     if target == 0:
         assert len(citems) == 0
 

@@ -66,7 +66,40 @@ __device__ __forceinline__ unsigned pack2(float a, float b) {
     return (unsigned)f32_to_bf16(a) | ((unsigned)f32_to_bf16(b) << 16);
 }
 
-template <bool DECODE>
+constexpr bool WIDE = (D % 32 == 0);           // 16x16x32 instruction for the scores when the head size allows
+constexpr int QSTEPS = WIDE ? D / 32 : D / 16;
+constexpr int DT = D / 16;
+
+// Keys and values of one block of 16 keys as this lane needs them for the two A operands.
+struct KVBlock {
+    uint4 k8[WIDE ? QSTEPS : 1];
+    uint2 k4[WIDE ? 1 : QSTEPS];
+    uint2 v[DT];
+    bool ok;
+};
+
+__device__ __forceinline__ void load_block(KVBlock& b, const AttnArgs& a, const int* bt, int j0, int kvh, int r, int g) {
+    const int ps = a.page_size;
+    const int blk = j0 / ps;
+    const int pg = bt[blk];
+    b.ok = pg >= 0 && pg < a.num_pages;   // a page the window has passed: its keys are masked for every row
+    if (!b.ok) return;
+    const int off = j0 - blk * ps;
+    const bf16_t* kb = a.k_pages + (((size_t)pg * a.n_kv + kvh) * ps + off + r) * D;
+    if constexpr (WIDE) {
+#pragma unroll
+        for (int st = 0; st < QSTEPS; ++st) b.k8[st] = *(const uint4*)(kb + st * 32 + g * 8);
+    } else {
+#pragma unroll
+        for (int st = 0; st < QSTEPS; ++st) b.k4[st] = *(const uint2*)(kb + st * 16 + g * 4);
+    }
+    const bf16_t* vb = a.v_pages + (((size_t)pg * a.n_kv + kvh) * D + r) * ps + off + 4 * g;
+#pragma unroll
+    for (int t = 0; t < DT; ++t) b.v[t] = *(const uint2*)(vb + (size_t)t * 16 * ps);
+}
+
+// RT row tiles of 16 rows per wave share every key/value block they read.
+template <bool DECODE, int RT>
 __global__ __launch_bounds__(256) void attn_bf16_kernel(AttnArgs a) {
     const int wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int item = blockIdx.x * 4 + wv;
@@ -94,169 +127,216 @@ __global__ __launch_bounds__(256) void attn_bf16_kernel(AttnArgs a) {
     const int kvh = blockIdx.y;
     const int G = a.n_heads / a.n_kv;
     const int r = lane & 15, g = lane >> 4;
-    const int ps = a.page_size;
-
     const int n_rows = q_len * G;
-    const int row = q_row0 + r;
-    const bool row_ok = row < n_rows;
-    const int rowc = row_ok ? row : n_rows - 1;
-    const int ti = rowc / G, head = kvh * G + (rowc - ti * G);
-    const int p = pos0 + ti;                                  // this row's position
-    const int p_lo = a.window > 0 ? p - a.window + 1 : 0;     // first key it sees
 
-    // queries of this lane's row: the B operand of S^T, kept for the whole item
-    const bf16_t* qrow = a.q + ((size_t)(q_tok0 + ti) * a.n_heads + head) * D;
-    constexpr bool WIDE = (D % 32 == 0);
-    constexpr int QSTEPS = WIDE ? D / 32 : D / 16;
-    bf16x8_t q8[WIDE ? QSTEPS : 1];
-    bf16x4_t q4[WIDE ? 1 : QSTEPS];
-    if constexpr (WIDE) {
+    bool row_ok[RT];
+    int ti[RT], head[RT], p[RT], p_lo[RT], tile_hi[RT], tile_lo[RT];
+    bf16x8_t q8[RT][WIDE ? QSTEPS : 1];
+    bf16x4_t q4[RT][WIDE ? 1 : QSTEPS];
+    f32x4_t o[RT][DT];
+    float m[RT], l[RT];
 #pragma unroll
-        for (int s = 0; s < QSTEPS; ++s) { U16 t; t.u = *(const uint4*)(qrow + s * 32 + g * 8); q8[s] = t.v; }
-    } else {
-#pragma unroll
-        for (int s = 0; s < QSTEPS; ++s) { U8 t; t.u = *(const uint2*)(qrow + s * 16 + g * 4); q4[s] = t.v; }
-    }
-
-    f32x4_t o[D / 16];
-#pragma unroll
-    for (int t = 0; t < D / 16; ++t) o[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
-    float m = -INFINITY, l = 0.f;
-
-    const int* bt = a.block_table + (size_t)entry * a.max_blocks;
-    for (int j0 = key_lo; j0 < key_hi; j0 += 16) {
-        const int blk = j0 / ps;
-        int pg = bt[blk];
-        if (pg < 0 || pg >= a.num_pages) continue;  // a page the window has passed; its keys are masked for every row
-        const int off = j0 - blk * ps;
-        const bf16_t* kb = a.k_pages + (((size_t)pg * a.n_kv + kvh) * ps + off + r) * D;
-        f32x4_t s = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+    for (int rt = 0; rt < RT; ++rt) {
+        const int row = q_row0 + rt * 16 + r;
+        row_ok[rt] = row < n_rows;
+        const int rowc = row_ok[rt] ? row : n_rows - 1;
+        ti[rt] = rowc / G;
+        head[rt] = kvh * G + (rowc - ti[rt] * G);
+        p[rt] = pos0 + ti[rt];                                   // this row's position
+        p_lo[rt] = a.window > 0 ? p[rt] - a.window + 1 : 0;      // first key it sees
+        // keys that any row of the tile may see (the same for every lane)
+        const int last_row = min(n_rows - 1, q_row0 + rt * 16 + 15), first_row = min(n_rows - 1, q_row0 + rt * 16);
+        tile_hi[rt] = (q_row0 + rt * 16 < n_rows) ? pos0 + last_row / G : -1;
+        tile_lo[rt] = a.window > 0 ? pos0 + first_row / G - a.window + 1 : 0;
+        const bf16_t* qrow = a.q + ((size_t)(q_tok0 + ti[rt]) * a.n_heads + head[rt]) * D;
         if constexpr (WIDE) {
 #pragma unroll
-            for (int st = 0; st < QSTEPS; ++st) {
-                U16 t; t.u = *(const uint4*)(kb + st * 32 + g * 8);
-                s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(t.v, q8[st], s, 0, 0, 0);
-            }
+            for (int s = 0; s < QSTEPS; ++s) { U16 t; t.u = *(const uint4*)(qrow + s * 32 + g * 8); q8[rt][s] = t.v; }
         } else {
 #pragma unroll
-            for (int st = 0; st < QSTEPS; ++st) {
-                U8 t; t.u = *(const uint2*)(kb + st * 16 + g * 4);
-                s = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(t.v, q4[st], s, 0, 0, 0);
+            for (int s = 0; s < QSTEPS; ++s) { U8 t; t.u = *(const uint2*)(qrow + s * 16 + g * 4); q4[rt][s] = t.v; }
+        }
+#pragma unroll
+        for (int t = 0; t < DT; ++t) o[rt][t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+        m[rt] = -INFINITY;
+        l[rt] = 0.f;
+    }
+
+    const int* bt = a.block_table + (size_t)entry * a.max_blocks;
+    KVBlock cur, nxt;
+    nxt.ok = false;
+    load_block(cur, a, bt, key_lo, kvh, r, g);
+    for (int j0 = key_lo; j0 < key_hi; j0 += 16) {
+        // the next block's loads are in flight while this one is computed
+        if (j0 + 16 < key_hi) load_block(nxt, a, bt, j0 + 16, kvh, r, g);
+        if (cur.ok) {
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+                if (j0 > tile_hi[rt] || j0 + 15 < tile_lo[rt]) continue;   // every key masked for every row of the tile
+                f32x4_t s = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+                if constexpr (WIDE) {
+#pragma unroll
+                    for (int st = 0; st < QSTEPS; ++st) {
+                        U16 t; t.u = cur.k8[st];
+                        s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(t.v, q8[rt][st], s, 0, 0, 0);
+                    }
+                } else {
+#pragma unroll
+                    for (int st = 0; st < QSTEPS; ++st) {
+                        U8 t; t.u = cur.k4[st];
+                        s = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(t.v, q4[rt][st], s, 0, 0, 0);
+                    }
+                }
+                // s[i] is key j0 + 4 g + i against row r of the tile
+                float sv[4];
+                bool ok[4];
+                float mb = -INFINITY;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int j = j0 + 4 * g + i;
+                    ok[i] = (j <= p[rt]) && (j >= p_lo[rt]);
+                    sv[i] = s[i] * a.scale_log2;
+                    if (ok[i]) mb = fmaxf(mb, sv[i]);
+                }
+                mb = fmaxf(mb, __shfl_xor(mb, 16, 64));
+                mb = fmaxf(mb, __shfl_xor(mb, 32, 64));
+                const float m_new = fmaxf(m[rt], mb);
+                const float alpha = (m[rt] == -INFINITY) ? 0.f : exp2f(m[rt] - m_new);
+                float pv[4], psum = 0.f;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    pv[i] = ok[i] ? exp2f(sv[i] - m_new) : 0.f;
+                    psum += pv[i];
+                }
+                l[rt] = l[rt] * alpha + psum;
+                m[rt] = m_new;
+                U8 pf;
+                pf.u.x = pack2(pv[0], pv[1]);
+                pf.u.y = pack2(pv[2], pv[3]);
+#pragma unroll
+                for (int t = 0; t < DT; ++t) {
+                    U8 vf; vf.u = cur.v[t];
+                    o[rt][t] *= alpha;
+                    o[rt][t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf.v, pf.v, o[rt][t], 0, 0, 0);
+                }
             }
         }
-        // s[i] is key j0 + 4 g + i against row r
-        float sv[4];
-        bool ok[4];
-        float mb = -INFINITY;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            int j = j0 + 4 * g + i;
-            ok[i] = (j <= p) && (j >= p_lo);
-            sv[i] = s[i] * a.scale_log2;
-            if (ok[i]) mb = fmaxf(mb, sv[i]);
-        }
-        mb = fmaxf(mb, __shfl_xor(mb, 16, 64));
-        mb = fmaxf(mb, __shfl_xor(mb, 32, 64));
-        const float m_new = fmaxf(m, mb);
-        const float alpha = (m == -INFINITY) ? 0.f : exp2f(m - m_new);
-        float pv[4], psum = 0.f;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            pv[i] = ok[i] ? exp2f(sv[i] - m_new) : 0.f;
-            psum += pv[i];
-        }
-        l = l * alpha + psum;
-        m = m_new;
-        U8 pf;
-        pf.u.x = pack2(pv[0], pv[1]);
-        pf.u.y = pack2(pv[2], pv[3]);
-        const bf16_t* vb = a.v_pages + (((size_t)pg * a.n_kv + kvh) * D + r) * ps + off + 4 * g;
-#pragma unroll
-        for (int t = 0; t < D / 16; ++t) {
-            U8 vf; vf.u = *(const uint2*)(vb + (size_t)t * 16 * ps);
-            o[t] *= alpha;
-            o[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf.v, pf.v, o[t], 0, 0, 0);
-        }
+        cur = nxt;
     }
-    l += __shfl_xor(l, 16, 64);
-    l += __shfl_xor(l, 32, 64);
 
-    if (part < 0) {
-        if (!row_ok) return;
-        const float inv = l > 0.f ? 1.f / l : 0.f;
-        bf16_t* orow = a.out + ((size_t)(q_tok0 + ti) * a.n_heads + head) * D;
 #pragma unroll
-        for (int t = 0; t < D / 16; ++t) {
-            uint2 w;
-            w.x = pack2(o[t][0] * inv, o[t][1] * inv);
-            w.y = pack2(o[t][2] * inv, o[t][3] * inv);
-            *(uint2*)(orow + t * 16 + 4 * g) = w;
-        }
-    } else {
-        if (!row_ok) return;
-        const size_t slot = ((size_t)part * a.n_kv + kvh) * 16 + r;
-        float* po = a.part_o + slot * D;
+    for (int rt = 0; rt < RT; ++rt) {
+        float lt = l[rt];
+        lt += __shfl_xor(lt, 16, 64);
+        lt += __shfl_xor(lt, 32, 64);
+        if (!row_ok[rt]) continue;
+        if (part < 0) {
+            const float inv = lt > 0.f ? 1.f / lt : 0.f;
+            bf16_t* orow = a.out + ((size_t)(q_tok0 + ti[rt]) * a.n_heads + head[rt]) * D;
 #pragma unroll
-        for (int t = 0; t < D / 16; ++t) *(f32x4_t*)(po + t * 16 + 4 * g) = o[t];
-        if (g == 0) {
-            a.part_ml[slot * 2] = m;
-            a.part_ml[slot * 2 + 1] = l;
+            for (int t = 0; t < DT; ++t) {
+                uint2 w;
+                w.x = pack2(o[rt][t][0] * inv, o[rt][t][1] * inv);
+                w.y = pack2(o[rt][t][2] * inv, o[rt][t][3] * inv);
+                *(uint2*)(orow + t * 16 + 4 * g) = w;
+            }
+        } else {
+            // partial slots of an item: RT consecutive tiles of 16 rows
+            const size_t slot = (((size_t)part * RT + rt) * a.n_kv + kvh) * 16 + r;
+            float* po = a.part_o + slot * D;
+#pragma unroll
+            for (int t = 0; t < DT; ++t) *(f32x4_t*)(po + t * 16 + 4 * g) = o[rt][t];
+            if (g == 0) {
+                a.part_ml[slot * 2] = m[rt];
+                a.part_ml[slot * 2 + 1] = lt;
+            }
         }
     }
 }
 
-// Merge the partial results of a row tile whose keys were split.
-// citems: [n][6] = q_tok0, q_len, q_row0, part0, n_parts, unused.  One block per (tile, kv head), 16 rows x D.
+// Merge the partial results of a tile of 16 rows whose keys were split over several items.
+// citems: [n][6] = q_tok0, q_len, first row of the tile, first item's partial index, number of items, tile index
+// within its items (each item holds `rt_per_item` tiles).  One block per (tile, kv head).
+#define MAX_PARTS 128
 template <bool DECODE>
-__global__ void attn_combine_kernel(const int* __restrict__ citems, const float* __restrict__ part_o,
-                                    const float* __restrict__ part_ml, bf16_t* __restrict__ out, int n_heads, int n_kv,
-                                    const int* __restrict__ entry_pos0, const int* __restrict__ dec_params, int p_max,
-                                    int window) {
-    int q_tok0, q_len, q_row0, part0, n_parts;
+__global__ __launch_bounds__(256) void attn_combine_kernel(const int* __restrict__ citems, const float* __restrict__ part_o,
+                                                          const float* __restrict__ part_ml, bf16_t* __restrict__ out,
+                                                          int n_heads, int n_kv, const int* __restrict__ entry_pos0,
+                                                          const int* __restrict__ dec_params, int p_max, int window,
+                                                          int rt_per_item) {
+    __shared__ float sm[MAX_PARTS][16];   // m of (part, row), then the row's normalised weight of the part
+    __shared__ float sl[MAX_PARTS][16];
+    int q_tok0, q_len, q_row0, part0, n_parts, rt;
     if (DECODE) {
         const int e = blockIdx.x, chunk = dec_params[0], pos0 = entry_pos0[e];
         const int lo = window > 0 ? max(0, pos0 - window + 1) : 0;
         const int p_first = ((lo >> 4) << 4) / chunk, p_last = pos0 / chunk;
-        q_tok0 = e; q_len = 1; q_row0 = 0;
+        q_tok0 = e; q_len = 1; q_row0 = 0; rt = 0;
         part0 = e * p_max + p_first;
         n_parts = p_last - p_first + 1;
         if (n_parts <= 1) return;   // a single item wrote the output itself
     } else {
         const int* it = citems + (size_t)blockIdx.x * 6;
-        q_tok0 = it[0]; q_len = it[1]; q_row0 = it[2]; part0 = it[3]; n_parts = it[4];
+        q_tok0 = it[0]; q_len = it[1]; q_row0 = it[2]; part0 = it[3]; n_parts = it[4]; rt = it[5];
         if (n_parts <= 0) return;
     }
-    const int kvh = blockIdx.y, G = n_heads / n_kv;
-    for (int idx = threadIdx.x; idx < 16 * D; idx += blockDim.x) {
-        int r = idx / D, d = idx - r * D;
-        int row = q_row0 + r;
-        if (row >= q_len * G) continue;
+    n_parts = min(n_parts, MAX_PARTS);   // the host never plans more
+    const int kvh = blockIdx.y, G = n_heads / n_kv, tid = threadIdx.x;
+    const int n_valid = min(16, q_len * G - q_row0);
+    // slot of (part pi, row r) = (((part0 + pi) * rt_per_item + rt) * n_kv + kvh) * 16 + r
+    const size_t slot0 = (((size_t)part0 * rt_per_item + rt) * n_kv + kvh) * 16;
+    const size_t slot_step = (size_t)rt_per_item * n_kv * 16;
+    for (int i = tid; i < n_parts * 16; i += 256) {
+        const int pi = i >> 4, r = i & 15;
+        const size_t sl_ = slot0 + pi * slot_step + r;
+        const bool ok = r < n_valid;
+        sm[pi][r] = ok ? part_ml[sl_ * 2] : -INFINITY;
+        sl[pi][r] = ok ? part_ml[sl_ * 2 + 1] : 0.f;
+    }
+    __syncthreads();
+    if (tid < 16) {
         float mx = -INFINITY;
-        for (int pi = 0; pi < n_parts; ++pi)
-            mx = fmaxf(mx, part_ml[((((size_t)(part0 + pi)) * n_kv + kvh) * 16 + r) * 2]);
-        float num = 0.f, den = 0.f;
+        for (int pi = 0; pi < n_parts; ++pi) mx = fmaxf(mx, sm[pi][tid]);
+        float den = 0.f;
         for (int pi = 0; pi < n_parts; ++pi) {
-            size_t slot = (((size_t)(part0 + pi)) * n_kv + kvh) * 16 + r;
-            float mp = part_ml[slot * 2];
-            float w = (mp == -INFINITY) ? 0.f : exp2f(mp - mx);
-            num += w * part_o[slot * D + d];
-            den += w * part_ml[slot * 2 + 1];
+            const float w = (sm[pi][tid] == -INFINITY) ? 0.f : exp2f(sm[pi][tid] - mx);
+            den += w * sl[pi][tid];
+            sm[pi][tid] = w;
         }
-        int ti = row / G, head = kvh * G + (row - ti * G);
-        out[((size_t)(q_tok0 + ti) * n_heads + head) * D + d] = f32_to_bf16(den > 0.f ? num / den : 0.f);
+        const float inv = den > 0.f ? 1.f / den : 0.f;
+        for (int pi = 0; pi < n_parts; ++pi) sm[pi][tid] *= inv;
+    }
+    __syncthreads();
+    for (int idx = tid; idx < n_valid * D; idx += 256) {
+        const int r = idx / D, d = idx - r * D;
+        const float* po = part_o + (slot0 + r) * D + d;
+        float acc = 0.f;
+#pragma unroll 4
+        for (int pi = 0; pi < n_parts; ++pi) acc += sm[pi][r] * po[(size_t)pi * slot_step * D];
+        const int row = q_row0 + r;
+        const int ti = row / G, head = kvh * G + (row - ti * G);
+        out[((size_t)(q_tok0 + ti) * n_heads + head) * D + d] = f32_to_bf16(acc);
     }
 }
 
 extern "C" int vt_attn_bf16_head_dim() { return D; }
 
+static int check_common(const char* who, int n_heads, int n_kv, int page_size, int max_blocks, int num_pages) {
+    VT_REQUIRE(n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "%s: bad heads %d/%d", who, n_heads, n_kv);
+    VT_REQUIRE(page_size > 0 && page_size % 16 == 0, "%s: page size %d is not a multiple of 16", who, page_size);
+    VT_REQUIRE(max_blocks > 0 && num_pages > 0, "%s: bad cache sizes", who);
+    VT_REQUIRE(n_kv <= 65535, "%s: too many kv heads (%d)", who, n_kv);
+    return 0;
+}
+
+// items: [n_items][8] = entry, q_tok0, q_len, pos0, first row, key_lo, key_hi, partial index (-1: writes the output).
+// Each item covers 16 * rt rows (rt = 1, 2 or 4).  The partial workspace holds (partial indices) * rt * n_kv * 16 rows.
 extern "C" int vt_attn_bf16(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
-                            const int* items, int n_items, const int* citems, int n_citems, void* out, float* part_o,
-                            float* part_ml, int n_heads, int n_kv, int page_size, int max_blocks, int num_pages,
-                            int window, float scale, hipStream_t stream) {
-    VT_REQUIRE(n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "vt_attn_bf16: bad heads %d/%d", n_heads, n_kv);
-    VT_REQUIRE(page_size > 0 && page_size % 16 == 0, "vt_attn_bf16: page size %d is not a multiple of 16", page_size);
-    VT_REQUIRE(max_blocks > 0 && num_pages > 0, "vt_attn_bf16: bad cache sizes");
-    VT_REQUIRE(n_kv <= 65535, "vt_attn_bf16: too many kv heads (%d)", n_kv);
+                            const int* items, int n_items, int rt, const int* citems, int n_citems, void* out,
+                            float* part_o, float* part_ml, int n_heads, int n_kv, int page_size, int max_blocks,
+                            int num_pages, int window, float scale, hipStream_t stream) {
+    if (check_common("vt_attn_bf16", n_heads, n_kv, page_size, max_blocks, num_pages)) return -1;
+    VT_REQUIRE(rt == 1 || rt == 2 || rt == 4, "vt_attn_bf16: %d row tiles per item (1, 2 or 4)", rt);
     VT_REQUIRE(n_citems == 0 || (part_o && part_ml), "vt_attn_bf16: split keys but no workspace");
     if (n_items <= 0) return 0;
     AttnArgs a;
@@ -265,11 +345,14 @@ extern "C" int vt_attn_bf16(const void* q, const void* k_pages, const void* v_pa
     a.n_items = n_items; a.n_heads = n_heads; a.n_kv = n_kv; a.page_size = page_size; a.max_blocks = max_blocks;
     a.num_pages = num_pages; a.window = window; a.scale_log2 = scale * 1.4426950408889634f;
     a.entry_pos0 = nullptr; a.dec_params = nullptr; a.p_max = 0;
-    attn_bf16_kernel<false><<<dim3((n_items + 3) / 4, n_kv), 256, 0, stream>>>(a);
+    dim3 grid((n_items + 3) / 4, n_kv);
+    if (rt == 1) attn_bf16_kernel<false, 1><<<grid, 256, 0, stream>>>(a);
+    else if (rt == 2) attn_bf16_kernel<false, 2><<<grid, 256, 0, stream>>>(a);
+    else attn_bf16_kernel<false, 4><<<grid, 256, 0, stream>>>(a);
     VT_CHECK_LAUNCH("vt_attn_bf16");
     if (n_citems > 0) {
         attn_combine_kernel<false><<<dim3(n_citems, n_kv), 256, 0, stream>>>(citems, part_o, part_ml, (bf16_t*)out,
-                                                                            n_heads, n_kv, nullptr, nullptr, 0, window);
+                                                                            n_heads, n_kv, nullptr, nullptr, 0, window, rt);
         VT_CHECK_LAUNCH("vt_attn_bf16(combine)");
     }
     return 0;
@@ -283,12 +366,10 @@ extern "C" int vt_attn_bf16_decode(const void* q, const void* k_pages, const voi
                                    const int* entry_pos0, const int* dec_params, int n_entries, int p_max, void* out,
                                    float* part_o, float* part_ml, int n_heads, int n_kv, int page_size, int max_blocks,
                                    int num_pages, int window, float scale, hipStream_t stream) {
-    VT_REQUIRE(n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "vt_attn_bf16_decode: bad heads %d/%d", n_heads, n_kv);
+    if (check_common("vt_attn_bf16_decode", n_heads, n_kv, page_size, max_blocks, num_pages)) return -1;
     VT_REQUIRE(n_heads / n_kv <= 16, "vt_attn_bf16_decode: %d query heads per kv head do not fit one tile of 16 rows",
                n_heads / n_kv);
-    VT_REQUIRE(page_size > 0 && page_size % 16 == 0, "vt_attn_bf16_decode: page size %d is not a multiple of 16", page_size);
-    VT_REQUIRE(max_blocks > 0 && num_pages > 0 && p_max > 0, "vt_attn_bf16_decode: bad sizes");
-    VT_REQUIRE(n_kv <= 65535, "vt_attn_bf16_decode: too many kv heads (%d)", n_kv);
+    VT_REQUIRE(p_max > 0 && p_max <= MAX_PARTS, "vt_attn_bf16_decode: %d items per entry (1..%d)", p_max, MAX_PARTS);
     VT_REQUIRE(part_o && part_ml && entry_pos0 && dec_params, "vt_attn_bf16_decode: missing buffers");
     if (n_entries <= 0) return 0;
     AttnArgs a;
@@ -297,10 +378,10 @@ extern "C" int vt_attn_bf16_decode(const void* q, const void* k_pages, const voi
     a.n_items = n_entries * p_max; a.n_heads = n_heads; a.n_kv = n_kv; a.page_size = page_size; a.max_blocks = max_blocks;
     a.num_pages = num_pages; a.window = window; a.scale_log2 = scale * 1.4426950408889634f;
     a.entry_pos0 = entry_pos0; a.dec_params = dec_params; a.p_max = p_max;
-    attn_bf16_kernel<true><<<dim3((a.n_items + 3) / 4, n_kv), 256, 0, stream>>>(a);
+    attn_bf16_kernel<true, 1><<<dim3((a.n_items + 3) / 4, n_kv), 256, 0, stream>>>(a);
     VT_CHECK_LAUNCH("vt_attn_bf16_decode");
     attn_combine_kernel<true><<<dim3(n_entries, n_kv), 256, 0, stream>>>(nullptr, part_o, part_ml, (bf16_t*)out, n_heads,
-                                                                        n_kv, entry_pos0, dec_params, p_max, window);
+                                                                        n_kv, entry_pos0, dec_params, p_max, window, 1);
     VT_CHECK_LAUNCH("vt_attn_bf16_decode(combine)");
     return 0;
 }

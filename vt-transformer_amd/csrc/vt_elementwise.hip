@@ -72,15 +72,90 @@ __global__ void rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__ del
     }
 }
 
+// The same, for widths that are a multiple of 4 and at most 256 * 4 * RMS_MAXV: every value is read once with
+// 16-byte loads and kept in registers between the sum and the scaling.  The sum of squares is taken in the same
+// order whatever the number of rows.
+#define RMS_MAXV 16
+__device__ __forceinline__ float4 load4(const float* p) { return *(const float4*)p; }
+__device__ __forceinline__ float4 load4(const bf16_t* p) {
+    uint2 u = *(const uint2*)p;
+    return make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u), __uint_as_float(u.y << 16),
+                       __uint_as_float(u.y & 0xffff0000u));
+}
+__device__ __forceinline__ void store4(float* p, float4 v) { *(float4*)p = v; }
+__device__ __forceinline__ void store4(bf16_t* p, float4 v) {
+    uint2 u;
+    u.x = (unsigned)f32_to_bf16(v.x) | ((unsigned)f32_to_bf16(v.y) << 16);
+    u.y = (unsigned)f32_to_bf16(v.z) | ((unsigned)f32_to_bf16(v.w) << 16);
+    *(uint2*)p = u;
+}
+
+template <typename TD, typename TO, bool HAS_DELTA, int NV>
+__global__ __launch_bounds__(256) void rmsnorm_vec_kernel(float* __restrict__ h, const TD* __restrict__ delta,
+                                                         const float* __restrict__ gain, TO* __restrict__ out,
+                                                         const int* __restrict__ rows, int hidden, float eps, int update) {
+    __shared__ float red[16];
+    const int r = blockIdx.x, tid = threadIdx.x;
+    const size_t src = rows ? (size_t)rows[r] : (size_t)r;
+    float* hr = h + src * hidden;
+    const TD* dr = HAS_DELTA ? delta + src * hidden : nullptr;
+    const int nq = hidden >> 2;
+    float4 x[NV];
+    float ss = 0.f;
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        const int qi = tid + v * 256;
+        if (qi < nq) {
+            x[v] = load4(hr + 4 * qi);
+            if (HAS_DELTA) {
+                float4 d = load4(dr + 4 * qi);
+                x[v].x += d.x; x[v].y += d.y; x[v].z += d.z; x[v].w += d.w;
+                if (update) store4(hr + 4 * qi, x[v]);
+            }
+            ss += x[v].x * x[v].x + x[v].y * x[v].y + x[v].z * x[v].z + x[v].w * x[v].w;
+        }
+    }
+    ss = block_sum(ss, red);
+    const float rinv = 1.0f / sqrtf(ss / (float)hidden + eps);
+    TO* o = out + (size_t)r * hidden;
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        const int qi = tid + v * 256;
+        if (qi < nq) {
+            float4 g = load4(gain + 4 * qi);
+            store4(o + 4 * qi, make_float4((g.x * x[v].x) * rinv, (g.y * x[v].y) * rinv, (g.z * x[v].z) * rinv,
+                                           (g.w * x[v].w) * rinv));
+        }
+    }
+}
+
+template <typename TD, typename TO, bool HD>
+static void launch_rmsnorm(float* h, const void* delta, const float* gain, void* out, const int* rows, int n_out,
+                           int hidden, float eps, int update_h, hipStream_t stream) {
+    const bool aligned = (hidden % 4 == 0) && !((uintptr_t)h & 15) && !((uintptr_t)gain & 15) && !((uintptr_t)out & 15) &&
+                         !((uintptr_t)delta & 15);
+    const int nq = hidden / 4;
+#define VT_RNV(NV) rmsnorm_vec_kernel<TD, TO, HD, NV><<<n_out, 256, 0, stream>>>(h, (const TD*)delta, gain, (TO*)out, \
+                                                                               rows, hidden, eps, update_h)
+    if (aligned && nq <= 256 * 1) VT_RNV(1);
+    else if (aligned && nq <= 256 * 2) VT_RNV(2);
+    else if (aligned && nq <= 256 * 4) VT_RNV(4);
+    else if (aligned && nq <= 256 * 8) VT_RNV(8);
+    else if (aligned && nq <= 256 * RMS_MAXV) VT_RNV(RMS_MAXV);
+    else {
+        int threads = hidden >= 2048 ? 512 : 256;
+        rmsnorm_kernel<TD, TO, HD><<<n_out, threads, 0, stream>>>(h, (const TD*)delta, gain, (TO*)out, rows, hidden, eps,
+                                                                 update_h);
+    }
+#undef VT_RNV
+}
+
 extern "C" int vt_rmsnorm(float* h, const void* delta, int delta_dtype, const float* gain, void* out, int out_dtype,
                           const int* rows, int n_out, int hidden, float eps, int update_h, hipStream_t stream) {
     VT_REQUIRE(n_out >= 0 && hidden > 0, "vt_rmsnorm: bad sizes n=%d hidden=%d", n_out, hidden);
     VT_REQUIRE(!(update_h && rows), "vt_rmsnorm: cannot update the residual through a row list");
     if (n_out == 0) return 0;
-    int threads = hidden >= 2048 ? 512 : 256;
-#define VT_RN(TD, TO, HD)                                                                                       \
-    rmsnorm_kernel<TD, TO, HD><<<n_out, threads, 0, stream>>>(h, (const TD*)delta, gain, (TO*)out, rows, hidden, \
-                                                              eps, update_h)
+#define VT_RN(TD, TO, HD) launch_rmsnorm<TD, TO, HD>(h, delta, gain, out, rows, n_out, hidden, eps, update_h, stream)
     if (!delta) {
         if (out_dtype == VT_F32) VT_RN(float, float, false);
         else if (out_dtype == VT_BF16) VT_RN(float, bf16_t, false);
@@ -134,21 +209,35 @@ __global__ void silu_mul_kernel(const TI* __restrict__ gu, TO* __restrict__ out,
     store_f32<TO>(out + (size_t)t * inter, i, g / (1.f + expf(-g)) * u);
 }
 
+// four values per thread with 8- or 16-byte accesses, for widths that are a multiple of 4
+template <typename TI, typename TO>
+__global__ void silu_mul_vec_kernel(const TI* __restrict__ gu, TO* __restrict__ out, int inter) {
+    int t = blockIdx.y;
+    int i = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
+    if (i >= inter) return;
+    const TI* row = gu + (size_t)t * 2 * inter;
+    float4 g = load4(row + i), u = load4(row + inter + i);
+    store4(out + (size_t)t * inter + i, make_float4(g.x / (1.f + expf(-g.x)) * u.x, g.y / (1.f + expf(-g.y)) * u.y,
+                                                   g.z / (1.f + expf(-g.z)) * u.z, g.w / (1.f + expf(-g.w)) * u.w));
+}
+
+template <typename TI, typename TO>
+static void launch_silu_mul(const void* gu, void* out, int n, int inter, hipStream_t stream) {
+    if (inter % 4 == 0 && !((uintptr_t)gu & 15) && !((uintptr_t)out & 15))
+        silu_mul_vec_kernel<TI, TO><<<dim3((inter / 4 + 255) / 256, n), 256, 0, stream>>>((const TI*)gu, (TO*)out, inter);
+    else
+        silu_mul_kernel<TI, TO><<<dim3((inter + 255) / 256, n), 256, 0, stream>>>((const TI*)gu, (TO*)out, inter);
+}
+
 extern "C" int vt_silu_mul(const void* gu, int in_dtype, void* out, int out_dtype, int n, int inter, hipStream_t stream) {
     VT_REQUIRE(n >= 0 && inter > 0, "vt_silu_mul: bad sizes n=%d inter=%d", n, inter);
     if (n == 0) return 0;
     VT_REQUIRE(n <= 65535, "vt_silu_mul: more than 65535 rows (%d)", n);
-    dim3 grid((inter + 255) / 256, n);
-    if (in_dtype == VT_F32 && out_dtype == VT_F32)
-        silu_mul_kernel<float, float><<<grid, 256, 0, stream>>>((const float*)gu, (float*)out, inter);
-    else if (in_dtype == VT_F32 && out_dtype == VT_BF16)
-        silu_mul_kernel<float, bf16_t><<<grid, 256, 0, stream>>>((const float*)gu, (bf16_t*)out, inter);
-    else if (in_dtype == VT_BF16 && out_dtype == VT_BF16)
-        silu_mul_kernel<bf16_t, bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, inter);
-    else if (in_dtype == VT_BF16 && out_dtype == VT_F32)
-        silu_mul_kernel<bf16_t, float><<<grid, 256, 0, stream>>>((const bf16_t*)gu, (float*)out, inter);
-    else
-        return vt_fail("vt_silu_mul: unknown dtypes %d -> %d", in_dtype, out_dtype);
+    if (in_dtype == VT_F32 && out_dtype == VT_F32) launch_silu_mul<float, float>(gu, out, n, inter, stream);
+    else if (in_dtype == VT_F32 && out_dtype == VT_BF16) launch_silu_mul<float, bf16_t>(gu, out, n, inter, stream);
+    else if (in_dtype == VT_BF16 && out_dtype == VT_BF16) launch_silu_mul<bf16_t, bf16_t>(gu, out, n, inter, stream);
+    else if (in_dtype == VT_BF16 && out_dtype == VT_F32) launch_silu_mul<bf16_t, float>(gu, out, n, inter, stream);
+    else return vt_fail("vt_silu_mul: unknown dtypes %d -> %d", in_dtype, out_dtype);
     VT_CHECK_LAUNCH("vt_silu_mul");
     return 0;
 }
@@ -224,6 +313,58 @@ __global__ void rope_store_kernel(RopeStoreArgs a) {
     }
 }
 
+// Four dims per thread with 8- or 16-byte accesses, one block per token; for head sizes that are a multiple of 4
+// and rotary dims that are a multiple of 8.
+template <typename TI, typename TO>
+__global__ __launch_bounds__(256) void rope_store_vec_kernel(RopeStoreArgs a) {
+    const int t = blockIdx.x;
+    const int D = a.D, half = a.rot >> 1, qd = D >> 2;
+    const int pos = a.positions[t];
+    const int tp = pos < a.max_pos ? (pos < 0 ? 0 : pos) : a.max_pos - 1;
+    const float* c = a.cos_t + (size_t)tp * half;
+    const float* s = a.sin_t + (size_t)tp * half;
+    const int n_heads_all = a.n_heads + (a.write_kv ? 2 * a.n_kv : 0);
+    const TI* in = (const TI*)a.qkv + (size_t)t * a.in_stride;
+    long long page = -1;
+    int slot = 0;
+    if (a.write_kv) {
+        const int e = a.tok_entry[t];
+        const int blk = pos / a.page_size;
+        slot = pos - blk * a.page_size;
+        const int pg = (blk < a.max_blocks) ? a.block_table[(size_t)e * a.max_blocks + blk] : -1;
+        if (pg >= 0 && pg < a.num_pages) page = pg;
+    }
+    for (int q = threadIdx.x; q < n_heads_all * qd; q += 256) {
+        const int head = q / qd, i = (q - head * qd) * 4;
+        const bool is_q = head < a.n_heads, is_v = head >= a.n_heads + a.n_kv;
+        if (!is_q && page < 0) continue;   // no page: the host never asks for this
+        const TI* hp = in + (size_t)head * D;
+        float4 x = load4(hp + i), o = x;
+        if (!is_v && i < a.rot) {
+            if (i < half) {
+                float4 y = load4(hp + i + half), cc = load4(c + i), sn = load4(s + i);
+                o = make_float4(cc.x * x.x - sn.x * y.x, cc.y * x.y - sn.y * y.y, cc.z * x.z - sn.z * y.z, cc.w * x.w - sn.w * y.w);
+            } else {
+                float4 y = load4(hp + i - half), cc = load4(c + i - half), sn = load4(s + i - half);
+                o = make_float4(cc.x * x.x + sn.x * y.x, cc.y * x.y + sn.y * y.y, cc.z * x.z + sn.z * y.z, cc.w * x.w + sn.w * y.w);
+            }
+        }
+        if (is_q) {
+            store4((TO*)a.q_out + ((size_t)t * a.n_heads + head) * D + i, o);
+        } else if (!is_v) {
+            const int kvh = head - a.n_heads;
+            store4((TO*)a.k_pages + (((size_t)page * a.n_kv + kvh) * a.page_size + slot) * D + i, o);
+        } else {
+            const int kvh = head - a.n_heads - a.n_kv;
+            TO* vp = (TO*)a.v_pages + (((size_t)page * a.n_kv + kvh) * D + i) * a.page_size + slot;
+            store_f32<TO>(vp, 0, o.x);
+            store_f32<TO>(vp, (size_t)a.page_size, o.y);
+            store_f32<TO>(vp, (size_t)2 * a.page_size, o.z);
+            store_f32<TO>(vp, (size_t)3 * a.page_size, o.w);
+        }
+    }
+}
+
 extern "C" int vt_rope_store(const void* qkv, int in_dtype, long long in_stride, const float* cos_t, const float* sin_t,
                              int rot, int max_pos, const int* positions, const int* tok_entry, const int* block_table,
                              int max_blocks, void* q_out, void* k_pages, void* v_pages, int out_dtype, int page_size,
@@ -239,13 +380,23 @@ extern "C" int vt_rope_store(const void* qkv, int in_dtype, long long in_stride,
     a.block_table = block_table; a.q_out = q_out; a.k_pages = k_pages; a.v_pages = v_pages;
     a.in_stride = in_stride; a.rot = rot; a.max_pos = max_pos; a.max_blocks = max_blocks;
     a.page_size = page_size; a.num_pages = num_pages; a.n_heads = n_heads; a.n_kv = n_kv; a.D = D; a.write_kv = write_kv;
+    const int isz = in_dtype == VT_F32 ? 4 : 2;
+    const bool vec = (D % 4 == 0) && (rot % 8 == 0) && (in_stride % 4 == 0) && !((uintptr_t)qkv & 15) &&
+                     !((uintptr_t)q_out & 15) && !((uintptr_t)k_pages & 15) && !((uintptr_t)cos_t & 15) &&
+                     !((uintptr_t)sin_t & 15) && (((size_t)D * isz) % 8 == 0);
     dim3 grid(n, n_heads + (write_kv ? 2 * n_kv : 0));
     VT_REQUIRE(grid.y <= 65535, "vt_rope_store: too many heads (%u)", grid.y);
     int threads = D <= 64 ? 64 : (D <= 128 ? 128 : 256);
-    if (in_dtype == VT_F32 && out_dtype == VT_F32) rope_store_kernel<float, float><<<grid, threads, 0, stream>>>(a);
-    else if (in_dtype == VT_F32 && out_dtype == VT_BF16) rope_store_kernel<float, bf16_t><<<grid, threads, 0, stream>>>(a);
-    else if (in_dtype == VT_BF16 && out_dtype == VT_BF16) rope_store_kernel<bf16_t, bf16_t><<<grid, threads, 0, stream>>>(a);
+#define VT_RS(TI, TO)                                                                    \
+    do {                                                                                 \
+        if (vec) rope_store_vec_kernel<TI, TO><<<n, 256, 0, stream>>>(a);                \
+        else rope_store_kernel<TI, TO><<<grid, threads, 0, stream>>>(a);                 \
+    } while (0)
+    if (in_dtype == VT_F32 && out_dtype == VT_F32) VT_RS(float, float);
+    else if (in_dtype == VT_F32 && out_dtype == VT_BF16) VT_RS(float, bf16_t);
+    else if (in_dtype == VT_BF16 && out_dtype == VT_BF16) VT_RS(bf16_t, bf16_t);
     else return vt_fail("vt_rope_store: unsupported dtypes %d -> %d", in_dtype, out_dtype);
+#undef VT_RS
     VT_CHECK_LAUNCH("vt_rope_store");
     return 0;
 }

@@ -49,40 +49,58 @@ class AttentionPlan:
     part_o: Optional[torch.Tensor]
     part_ml: Optional[torch.Tensor]
     n_parts: int
+    rt: int = 1
+
+
+MAX_PARTS = 128     # the merge kernel holds the weights of at most this many items per row tile
+
+
+def choose_row_tiles(entry_start: np.ndarray, group: int, n_kv: int, min_items: int = 768) -> int:
+    """Row tiles (of 16 rows) per attention item: as many as still leave enough items to fill the GPU.  More tiles
+    per item means every key/value block read serves more rows."""
+    rows = int(((entry_start[1:] - entry_start[:-1]).astype(np.int64) * group).sum())
+    for rt in (4, 2):
+        q_len = (entry_start[1:] - entry_start[:-1]).astype(np.int64)
+        items = int(((q_len * group + 16 * rt - 1) // (16 * rt)).sum()) * n_kv
+        if items >= min_items:
+            return rt
+    return 1
 
 
 def plan_attention_items(entry_start: np.ndarray, entry_pos0: np.ndarray, group: int, window: int, n_kv: int,
-                         target_waves: int = 2048, min_chunk: int = 64) -> Tuple[np.ndarray, np.ndarray, int]:
+                         target_waves: int = 2048, min_chunk: int = 64, rt: int = 1) -> Tuple[np.ndarray, np.ndarray, int]:
     """Work items of the bf16 attention kernel for one step.
 
-    Rows of an entry are (token, query head of a kv group) pairs, token-major; a tile is 16 rows.  Each tile
-    needs keys [key_lo, key_hi).  When the tiles are too few to fill the GPU, a tile's keys are cut at absolute
-    multiples of a chunk length into several items whose partial results a second kernel merges.
-    Returns (items [n, 8], combine items [m, 6], number of partial slots)."""
+    Rows of an entry are (token, query head of a kv group) pairs, token-major.  An item is 16 * rt rows (rt row
+    tiles) against the keys [key_lo, key_hi) that any of them may see.  When the items are too few to fill the
+    GPU, an item's keys are cut at absolute multiples of a chunk length into several items whose partial results
+    a second kernel merges, tile by tile.
+    Returns (items [n, 8], combine items [m, 6], number of partial indices)."""
     n_entries = len(entry_pos0)
+    rpi = 16 * rt
     q_len = (entry_start[1:] - entry_start[:-1]).astype(np.int64)
     rows = q_len * group
-    n_tiles = (rows + 15) // 16
+    n_tiles = (rows + rpi - 1) // rpi
     total = int(n_tiles.sum())
     if total == 0:
         return np.zeros((0, ATTN_ITEM_INTS), np.int32), np.zeros((0, ATTN_CITEM_INTS), np.int32), 0
     ent = np.repeat(np.arange(n_entries), n_tiles)
     first = np.cumsum(n_tiles) - n_tiles
     tile_in_entry = np.arange(total) - np.repeat(first, n_tiles)
-    row0 = tile_in_entry * 16
+    row0 = tile_in_entry * rpi
     e_rows, e_len, e_pos0, e_start = rows[ent], q_len[ent], entry_pos0[ent].astype(np.int64), entry_start[:-1][ent].astype(np.int64)
     t_first = row0 // group
-    t_last = np.minimum(e_rows - 1, row0 + 15) // group
+    t_last = np.minimum(e_rows - 1, row0 + rpi - 1) // group
     min_p, max_p = e_pos0 + t_first, e_pos0 + t_last
     lo = np.maximum(0, min_p - window + 1) if window > 0 else np.zeros_like(min_p)
     key_lo = (lo // 16) * 16
     key_hi = max_p + 1
     span = key_hi - key_lo
-    # split keys only if the tiles alone leave most of the GPU idle
+    # split keys only if the items alone leave most of the GPU idle
     chunk = 0
     if total * n_kv < target_waves // 2:
         keys_total = int(span.sum()) * n_kv
-        chunk = max(min_chunk, -(-keys_total // target_waves))
+        chunk = max(min_chunk, -(-keys_total // target_waves), -(-int(span.max() + 15) // MAX_PARTS))
         chunk = -(-chunk // 16) * 16
         if chunk >= int(span.max()):
             chunk = 0
@@ -102,9 +120,15 @@ def plan_attention_items(entry_start: np.ndarray, entry_pos0: np.ndarray, group:
     part_id = np.where(single, -1, np.arange(tot_parts))
     items = np.stack([ent[tile_of], e_start[tile_of], e_len[tile_of], e_pos0[tile_of], row0[tile_of], p_lo, p_hi,
                       part_id], axis=1).astype(np.int32)
+    # one merge per 16-row tile of every item whose keys were split
     multi = np.nonzero(n_parts > 1)[0]
-    citems = np.stack([e_start[multi], e_len[multi], row0[multi], p_first[multi], n_parts[multi],
-                       np.zeros(len(multi), np.int64)], axis=1).astype(np.int32)
+    cl = []
+    for sub in range(rt):
+        r0 = row0[multi] + 16 * sub
+        keep = r0 < e_rows[multi]
+        m = multi[keep]
+        cl.append(np.stack([e_start[m], e_len[m], r0[keep], p_first[m], n_parts[m], np.full(len(m), sub)], axis=1))
+    citems = np.concatenate(cl).astype(np.int32) if cl else np.zeros((0, ATTN_CITEM_INTS), np.int32)
     return items, citems, tot_parts
 
 
@@ -142,7 +166,9 @@ class StepContext:
 
     def _make_plan(self, key) -> AttentionPlan:
         group, window, n_kv, head_dim = key
-        items, citems, n_parts = plan_attention_items(self.h_entry_start, self.h_entry_pos0, group, window, n_kv)
+        row_tiles = choose_row_tiles(self.h_entry_start, group, n_kv)
+        items, citems, n_parts = plan_attention_items(self.h_entry_start, self.h_entry_pos0, group, window, n_kv,
+                                                      rt=row_tiles)
         rt = self.rt
         tag = f"attnplan.{group}.{window}.{n_kv}.{head_dim}"
         flat = np.concatenate([items.reshape(-1), citems.reshape(-1)])
@@ -153,9 +179,9 @@ class StepContext:
         d_citems = dev[items.size:items.size + citems.size] if citems.size else None
         part_o = part_ml = None
         if n_parts:
-            part_o = rt.buffer("attn.part_o", (n_parts * n_kv * 16 * head_dim,), torch.float32)
-            part_ml = rt.buffer("attn.part_ml", (n_parts * n_kv * 16 * 2,), torch.float32)
-        return AttentionPlan(d_items, items.shape[0], d_citems, citems.shape[0], part_o, part_ml, n_parts)
+            part_o = rt.buffer("attn.part_o", (n_parts * row_tiles * n_kv * 16 * head_dim,), torch.float32)
+            part_ml = rt.buffer("attn.part_ml", (n_parts * row_tiles * n_kv * 16 * 2,), torch.float32)
+        return AttentionPlan(d_items, items.shape[0], d_citems, citems.shape[0], part_o, part_ml, n_parts, row_tiles)
 
 
 def decode_chunk(kv_lens: np.ndarray, p_max: int, target_items: int = 1024, min_chunk: int = 64) -> int:

@@ -226,14 +226,17 @@ ATTN_CITEM_INTS = 6
 def attention_bf16(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
                    items: torch.Tensor, n_items: int, citems: Optional[torch.Tensor], n_citems: int, out: torch.Tensor,
                    part_o: Optional[torch.Tensor], part_ml: Optional[torch.Tensor], n_heads: int, n_kv: int,
-                   head_dim: int, window: int, scale: float, max_part: int = 0) -> torch.Tensor:
-    """`items` [>=n_items, 8] int32: entry, q_tok0, q_len, pos0, q_row0, key_lo, key_hi, part (-1 = final).
-    `citems` [>=n_citems, 6] int32: q_tok0, q_len, q_row0, part0, n_parts, 0.  The planner (engine) makes them;
-    `max_part` is the number of partial slots it used, checked against the workspace here."""
+                   head_dim: int, window: int, scale: float, max_part: int = 0, rt: int = 1) -> torch.Tensor:
+    """`items` [>=n_items, 8] int32: entry, q_tok0, q_len, pos0, first row, key_lo, key_hi, partial index (-1 = final);
+    an item covers 16 * rt rows.  `citems` [>=n_citems, 6] int32: q_tok0, q_len, first row of a 16-row tile, first
+    partial index, number of items, tile index within the item.  The planner (engine) makes them; `max_part` is the
+    number of partial indices it used, checked against the workspace here."""
     n = q.shape[0]
     num_pages, kvh, page_size, d = k_pages.shape
     if head_dim % 16 or not 16 <= head_dim <= 256:
         raise KernelError(f"attention_bf16: head size {head_dim} is not a multiple of 16 in 16..256")
+    if rt not in (1, 2, 4):
+        raise KernelError(f"attention_bf16: {rt} row tiles per item (1, 2 or 4)")
     _chk(q, "attention_bf16.q", torch.bfloat16, (n, n_heads * head_dim))
     _chk(k_pages, "attention_bf16.k_pages", torch.bfloat16, (num_pages, n_kv, page_size, head_dim))
     _chk(v_pages, "attention_bf16.v_pages", torch.bfloat16, (num_pages, n_kv, head_dim, page_size))
@@ -248,10 +251,10 @@ def attention_bf16(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor
         _chk(part_ml, "attention_bf16.part_ml", torch.float32)
         if citems.numel() < n_citems * ATTN_CITEM_INTS:
             raise KernelError("attention_bf16: combine list shorter than n_citems")
-        if part_o.numel() < max_part * n_kv * 16 * head_dim or part_ml.numel() < max_part * n_kv * 16 * 2:
+        if part_o.numel() < max_part * rt * n_kv * 16 * head_dim or part_ml.numel() < max_part * rt * n_kv * 16 * 2:
             raise KernelError("attention_bf16: workspace for split keys is too small")
     lib = load_lib("vt_attn_bf16", head_dim)
-    _run(lib, "vt_attn_bf16", _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(block_table), _ptr(items), _i(n_items),
+    _run(lib, "vt_attn_bf16", _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(block_table), _ptr(items), _i(n_items), _i(rt),
          _ptr(citems), _i(n_citems), _ptr(out), _ptr(part_o), _ptr(part_ml), _i(n_heads), _i(n_kv), _i(page_size),
          _i(block_table.shape[1]), _i(num_pages), _i(window), _f(scale), _stream())
     return out

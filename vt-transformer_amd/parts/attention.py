@@ -124,5 +124,5 @@ class PagedAttention(Part):
             plan = ctx.attention_plan(nh // nkv, self.window, nkv, d)
             ops.attention_bf16(q, cache.k, cache.v, cache.block_table, plan.items, plan.n_items, plan.citems,
                                plan.n_citems, out, plan.part_o, plan.part_ml, nh, nkv, d, self.window, self.scale,
-                               max_part=plan.n_parts)
+                               max_part=plan.n_parts, rt=plan.rt)
         return linear(rt, out, self.w_o, self.b_o, "attn.o")
