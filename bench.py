@@ -38,6 +38,7 @@ def main() -> int:
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--no-graphs", action="store_true")
+    ap.add_argument("--no-prefill", action="store_true", help="skip the prefill measurement (profiling runs)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this engine runs on one GPU; N > 1 is not measured")
@@ -117,7 +118,7 @@ def main() -> int:
     achieved = step_bytes / (ms * 1e-3) / 1e9
 
     T = args.prefill_tokens
-    p_dt = prefill_run(T)
+    p_dt = prefill_run(T) if not args.no_prefill else float("nan")
     mm_flops = 2.0 * T * L * (qkv * H + cfg.num_attention_heads * cfg.head_dim * H + 3 * I * H) + 2.0 * V * H
     attn_flops = L * 4.0 * cfg.num_attention_heads * cfg.head_dim * (T * (T + 1) / 2)   # causal: QK^T and PV
     p_flops = mm_flops + attn_flops

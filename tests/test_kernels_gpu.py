@@ -247,20 +247,30 @@ def attention_case(dtype, nh, kvh, d, page_size, window, entries, seed, spike=Fa
         from vt_transformer_amd.engine.step import plan_attention_items
         start = np.cumsum([0] + [n for _, n in entries]).astype(np.int32)
         pos0 = np.array([c for c, _ in entries], dtype=np.int32)
+        from vt_transformer_amd.engine.step import plan_tile_items
         first = None
-        for target, rt in ((0, 1), (10 ** 9, 1), (0, 2), (10 ** 9, 4), (0, 4)):   # keys unsplit and split; 1, 2, 4 row tiles
+        kpd, vpd, btd = kp.to(DEV), vp.to(DEV), bt.to(DEV)
+        # 16-row items with keys unsplit and split, one and two row tiles; then the LDS-tiled kernel on all entries
+        for target, rt in ((0, 1), (10 ** 9, 1), (0, 2), (10 ** 9, 2)):
             items, citems, n_parts = plan_attention_items(start, pos0, nh // kvh, window, kvh, target_waves=target,
                                                           min_chunk=16, rt=rt)
             part_o = torch.full((max(1, n_parts) * rt * kvh * 16 * d,), float("nan"), device=DEV)
             part_ml = torch.full((max(1, n_parts) * rt * kvh * 32,), float("nan"), device=DEV)
             out.fill_(float("nan"))
-            o.attention_bf16(q, kp.to(DEV), vp.to(DEV), bt.to(DEV), torch.from_numpy(items).to(DEV).reshape(-1),
+            o.attention_bf16(q, kpd, vpd, btd, torch.from_numpy(items).to(DEV).reshape(-1),
                              items.shape[0], torch.from_numpy(citems).to(DEV).reshape(-1) if len(citems) else None,
                              len(citems), out, part_o, part_ml, nh, kvh, d, window, scale, max_part=n_parts, rt=rt)
             if first is None:
                 first = out.clone()
             assert bool(torch.isfinite(out).all()), (target, rt)
             assert rel_err(out, first) < 1e-2, (target, rt)  # every way of cutting the work agrees to rounding
+        for rt in (1, 2):
+            items, _ = plan_tile_items(start, pos0, nh // kvh, window, kvh, np.arange(len(entries)), rt=rt)
+            out.fill_(float("nan"))
+            o.attention_bf16_tiles(q, kpd, vpd, btd, torch.from_numpy(items).to(DEV).reshape(-1), items.shape[0], out,
+                                   nh, kvh, d, window, scale, rt=rt)
+            assert bool(torch.isfinite(out).all()), ("tiles", rt)
+            assert rel_err(out, first) < 1e-2, ("tiles", rt)
     ref = torch.cat([ref_attention(qs[e][i], ks[e], vs[e], c + i, window, scale).reshape(1, -1)
                      for e, (c, n) in enumerate(entries) for i in range(n)])
     return out, ref
@@ -293,6 +303,15 @@ def test_attention_window_edge(dtype, window):
     entries = [(0, 70), (130, 1), (window, 1), (window - 1, 1) if window > 1 else (0, 1), (20, 30)]
     got, ref = attention_case(dtype, 4, 2, 32, 16, window, entries, seed=window, spike=True)
     assert rel_err(got, ref) < ATT_TOL[dtype]
+
+
+def test_attention_long_portion_bf16():
+    """A portion of 700 tokens after 4,500 cached ones: more pages than the tiled kernel keeps ids for at a time."""
+    entries = [(4500, 700), (0, 300)]
+    got, ref = attention_case(torch.bfloat16, 4, 2, 32, 16, 0, entries, seed=5)
+    assert rel_err(got, ref) < ATT_TOL[torch.bfloat16]
+    got, ref = attention_case(torch.bfloat16, 2, 1, 64, 16, 600, [(3000, 400)], seed=6, spike=True)
+    assert rel_err(got, ref) < ATT_TOL[torch.bfloat16]
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

@@ -2,13 +2,13 @@
 import numpy as np
 import pytest
 
-from vt_transformer_amd.engine.step import decode_chunk, plan_attention_items
+from vt_transformer_amd.engine.step import decode_chunk, plan_attention_items, plan_tile_items, split_entries
 from vt_transformer_amd.sampling import SamplingParams, request_seed, uniform
 
 
 @pytest.mark.parametrize("group,window", [(1, 0), (7, 0), (2, 5), (5, 40), (3, 16)])
 @pytest.mark.parametrize("target", [0, 2048, 10 ** 9])
-@pytest.mark.parametrize("rt", [1, 2, 4])
+@pytest.mark.parametrize("rt", [1, 2])
 def test_every_row_gets_every_key_it_may_see_exactly_once(group, window, target, rt):
     lens = np.array([1, 37, 1, 2, 19, 130])
     pos0 = np.array([300, 0, 0, 16, 45, 7])
@@ -47,11 +47,36 @@ def test_every_row_gets_every_key_it_may_see_exactly_once(group, window, target,
         assert len(citems) == 0
 
 
+@pytest.mark.parametrize("group,window", [(1, 0), (7, 0), (5, 40)])
+@pytest.mark.parametrize("rt", [1, 2])
+def test_tile_items_cover_the_long_entries(group, window, rt):
+    lens = np.array([1, 300, 40, 2048, 260])
+    pos0 = np.array([300, 0, 10, 77, 5000])
+    start = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    short, long = split_entries(start, group)
+    assert sorted(list(short) + list(long)) == list(range(5))
+    assert all(lens[e] * group >= 256 for e in long) and all(lens[e] * group < 256 for e in short)
+    items, got_rt = plan_tile_items(start, pos0.astype(np.int32), group, window, 4, long, rt=rt)
+    assert got_rt == rt
+    spans = [it[6] - it[5] for it in items.tolist()]
+    assert spans == sorted(spans, reverse=True)                       # the longest first
+    seen = set()
+    for entry, q_tok0, q_len, p0, row0, lo, hi, part in items.tolist():
+        assert part == -1 and lo % 16 == 0 and q_tok0 == start[entry]
+        for r_ in range(row0, min(row0 + 64 * rt, q_len * group)):
+            p = p0 + r_ // group
+            first = max(0, p - window + 1) if window else 0
+            assert lo <= first and p < hi                               # all the keys the row may see are inside
+            assert (entry, r_) not in seen
+            seen.add((entry, r_))
+    assert seen == {(e, r_) for e in long for r_ in range(lens[e] * group)}
+
+
 def test_decode_chunk():
-    assert decode_chunk(np.array([1]), 64) == 64
+    assert decode_chunk(np.array([1]), 64) == 32
     assert decode_chunk(np.array([8192]), 64) % 16 == 0 and decode_chunk(np.array([8192]), 64) * 64 >= 8192
     c = decode_chunk(np.full(64, 1024), 64)
-    assert c % 16 == 0 and 64 <= c <= 128
+    assert c % 16 == 0 and 32 <= c <= 128
 
 
 def test_uniform_numbers_depend_only_on_seed_and_counter():

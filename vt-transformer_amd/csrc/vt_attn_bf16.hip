@@ -78,10 +78,10 @@ struct KVBlock {
     bool ok;
 };
 
-__device__ __forceinline__ void load_block(KVBlock& b, const AttnArgs& a, const int* bt, int j0, int kvh, int r, int g) {
+// `pg` is the page of the block (read from the block table ahead of time, so that the loads below do not wait for it)
+__device__ __forceinline__ void load_block(KVBlock& b, const AttnArgs& a, int pg, int j0, int kvh, int r, int g) {
     const int ps = a.page_size;
     const int blk = j0 / ps;
-    const int pg = bt[blk];
     b.ok = pg >= 0 && pg < a.num_pages;   // a page the window has passed: its keys are masked for every row
     if (!b.ok) return;
     const int off = j0 - blk * ps;
@@ -162,13 +162,27 @@ __global__ __launch_bounds__(256) void attn_bf16_kernel(AttnArgs a) {
         l[rt] = 0.f;
     }
 
+    // Page ids of up to 64 pages at a time, one per lane: reading the table is then off the path of every block's
+    // loads.  (The lane index of a read is the same for the whole wave.)
     const int* bt = a.block_table + (size_t)entry * a.max_blocks;
+    const int ps = a.page_size;
+    const int last_page = (key_hi - 1) / ps;
+    int cache_base = key_lo / ps;
+    int pg_lane = (cache_base + lane <= last_page) ? bt[cache_base + lane] : -1;
+    auto page_of = [&](int j) {
+        int blk = j / ps;
+        if (blk >= cache_base + 64) {
+            cache_base = blk;
+            pg_lane = (cache_base + lane <= last_page) ? bt[cache_base + lane] : -1;
+        }
+        return __builtin_amdgcn_readlane(pg_lane, __builtin_amdgcn_readfirstlane(blk - cache_base));
+    };
     KVBlock cur, nxt;
     nxt.ok = false;
-    load_block(cur, a, bt, key_lo, kvh, r, g);
+    load_block(cur, a, page_of(key_lo), key_lo, kvh, r, g);
     for (int j0 = key_lo; j0 < key_hi; j0 += 16) {
         // the next block's loads are in flight while this one is computed
-        if (j0 + 16 < key_hi) load_block(nxt, a, bt, j0 + 16, kvh, r, g);
+        if (j0 + 16 < key_hi) load_block(nxt, a, page_of(j0 + 16), j0 + 16, kvh, r, g);
         if (cur.ok) {
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
@@ -254,6 +268,243 @@ __global__ __launch_bounds__(256) void attn_bf16_kernel(AttnArgs a) {
     }
 }
 
+// ---------------------------------------------------------------------------
+// Long portions of prompts: a block of 4 waves takes 64 * RT consecutive rows of one (entry, kv head) and walks
+// their keys KB at a time.  Every key/value block is fetched from the pages once per block of waves, by all 256
+// threads together with 16-byte loads, and parked in LDS (two buffers: the next block is on its way from memory
+// while this one is multiplied); the four waves read their matrix operands from there.  Rows of an item that lie
+// wholly above a key block skip it (the upper triangle of a causal portion costs nothing).
+// ---------------------------------------------------------------------------
+constexpr int KB = (D > 128) ? 16 : 32;        // keys per block
+constexpr int KT = KB / 16;                    // score tiles per block
+constexpr int KROW = D + 8;                    // padded rows: operand reads from LDS without bank conflicts
+constexpr int VROW = KB + 8;
+constexpr int KPIECES = KB * (D / 8);          // 16-byte pieces of a key block
+constexpr int VPIECES = D * (KB / 8);
+constexpr int KPT = (KPIECES + 255) / 256;     // pieces per thread
+constexpr int VPT = (VPIECES + 255) / 256;
+constexpr int PAGE_WINDOW = 256;               // page ids kept in LDS at a time
+
+template <int RT>
+__global__ __launch_bounds__(256) void attn_bf16_tile_kernel(AttnArgs a) {
+    __shared__ __attribute__((aligned(16))) bf16_t k_lds[2][KB][KROW];
+    __shared__ __attribute__((aligned(16))) bf16_t v_lds[2][D][VROW];
+    __shared__ int s_pages[PAGE_WINDOW];
+    const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63;
+    const int* it = a.items + (size_t)blockIdx.x * ITEM_INTS;
+    const int entry = it[0], q_tok0 = it[1], q_len = it[2], pos0 = it[3], q_row0 = it[4];
+    const int key_lo = it[5], key_hi = it[6];
+    if (entry < 0) return;
+    const int kvh = blockIdx.y;
+    const int G = a.n_heads / a.n_kv;
+    const int r = lane & 15, g = lane >> 4;
+    const int n_rows = q_len * G;
+    const int ps = a.page_size;
+
+    bool row_ok[RT];
+    int ti[RT], head[RT], p[RT], p_lo[RT], tile_hi[RT], tile_lo[RT];
+    bf16x8_t q8[RT][WIDE ? QSTEPS : 1];
+    bf16x4_t q4[RT][WIDE ? 1 : QSTEPS];
+    f32x4_t o[RT][DT];
+    float m[RT], l[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        const int row0 = q_row0 + (wv * RT + rt) * 16;
+        const int row = row0 + r;
+        row_ok[rt] = row < n_rows;
+        const int rowc = row_ok[rt] ? row : n_rows - 1;
+        ti[rt] = rowc / G;
+        head[rt] = kvh * G + (rowc - ti[rt] * G);
+        p[rt] = pos0 + ti[rt];
+        p_lo[rt] = a.window > 0 ? p[rt] - a.window + 1 : 0;
+        const int last_row = min(n_rows - 1, row0 + 15), first_row = min(n_rows - 1, row0);
+        tile_hi[rt] = (row0 < n_rows) ? pos0 + last_row / G : -1;
+        tile_lo[rt] = a.window > 0 ? pos0 + first_row / G - a.window + 1 : 0;
+        const bf16_t* qrow = a.q + ((size_t)(q_tok0 + ti[rt]) * a.n_heads + head[rt]) * D;
+        if constexpr (WIDE) {
+#pragma unroll
+            for (int s = 0; s < QSTEPS; ++s) { U16 t; t.u = *(const uint4*)(qrow + s * 32 + g * 8); q8[rt][s] = t.v; }
+        } else {
+#pragma unroll
+            for (int s = 0; s < QSTEPS; ++s) { U8 t; t.u = *(const uint2*)(qrow + s * 16 + g * 4); q4[rt][s] = t.v; }
+        }
+#pragma unroll
+        for (int t = 0; t < DT; ++t) o[rt][t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+        m[rt] = -INFINITY;
+        l[rt] = 0.f;
+    }
+
+    const int* bt = a.block_table + (size_t)entry * a.max_blocks;
+    const int last_page = (key_hi - 1) / ps;
+    int page_base = key_lo / ps;
+    auto fill_pages = [&]() {   // all threads; callers put barriers around it
+        const int pgi = page_base + tid;
+        if (tid < PAGE_WINDOW) s_pages[tid] = (pgi <= last_page) ? bt[pgi] : -1;
+    };
+    uint4 kreg[KPT], vreg[VPT];
+    auto fetch = [&](int j0) {   // this thread's pieces of keys [j0, j0 + KB) from the pages into registers
+#pragma unroll
+        for (int i = 0; i < KPT; ++i) {
+            const int idx = tid + 256 * i;
+            kreg[i] = make_uint4(0, 0, 0, 0);
+            if (idx < KPIECES) {
+                const int key = idx / (D / 8), c = idx - key * (D / 8);
+                const int j = j0 + key;
+                const int blk = j / ps;
+                const int pg = (j < key_hi) ? s_pages[blk - page_base] : -1;
+                if (pg >= 0 && pg < a.num_pages)
+                    kreg[i] = *(const uint4*)(a.k_pages + (((size_t)pg * a.n_kv + kvh) * ps + (j - blk * ps)) * D + c * 8);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < VPT; ++i) {
+            const int idx = tid + 256 * i;
+            vreg[i] = make_uint4(0, 0, 0, 0);
+            if (idx < VPIECES) {
+                const int d = idx / (KB / 8), kg = idx - d * (KB / 8);
+                const int j = j0 + kg * 8;
+                const int blk = j / ps;
+                const int pg = (j < key_hi) ? s_pages[blk - page_base] : -1;
+                if (pg >= 0 && pg < a.num_pages)
+                    vreg[i] = *(const uint4*)(a.v_pages + (((size_t)pg * a.n_kv + kvh) * D + d) * ps + (j - blk * ps));
+            }
+        }
+    };
+    auto park = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < KPT; ++i) {
+            const int idx = tid + 256 * i;
+            if (idx < KPIECES) {
+                const int key = idx / (D / 8), c = idx - key * (D / 8);
+                *(uint4*)&k_lds[buf][key][c * 8] = kreg[i];
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < VPT; ++i) {
+            const int idx = tid + 256 * i;
+            if (idx < VPIECES) {
+                const int d = idx / (KB / 8), kg = idx - d * (KB / 8);
+                *(uint4*)&v_lds[buf][d][kg * 8] = vreg[i];
+            }
+        }
+    };
+
+    fill_pages();
+    __syncthreads();
+    fetch(key_lo);
+    park(0);
+    __syncthreads();
+    int buf = 0;
+    for (int j0 = key_lo; j0 < key_hi; j0 += KB) {
+        const int jn = j0 + KB;
+        const bool more = jn < key_hi;
+        if (more) {
+            if ((jn + KB - 1) / ps >= page_base + PAGE_WINDOW) {   // the same decision in every thread
+                __syncthreads();
+                page_base = jn / ps;
+                fill_pages();
+                __syncthreads();
+            }
+            fetch(jn);   // in flight while this block is multiplied
+        }
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+            if (j0 > tile_hi[rt] || j0 + KB - 1 < tile_lo[rt]) continue;   // every key masked for every row of the tile
+            f32x4_t s[KT];
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt) {
+                s[kt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+                const bf16_t* kr = &k_lds[buf][kt * 16 + r][0];
+                if constexpr (WIDE) {
+#pragma unroll
+                    for (int st = 0; st < QSTEPS; ++st) {
+                        U16 t; t.u = *(const uint4*)(kr + st * 32 + g * 8);
+                        s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(t.v, q8[rt][st], s[kt], 0, 0, 0);
+                    }
+                } else {
+#pragma unroll
+                    for (int st = 0; st < QSTEPS; ++st) {
+                        U8 t; t.u = *(const uint2*)(kr + st * 16 + g * 4);
+                        s[kt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(t.v, q4[rt][st], s[kt], 0, 0, 0);
+                    }
+                }
+            }
+            // s[kt][i] is key j0 + 16 kt + 4 g + i against row r of the tile
+            float sv[KT][4];
+            bool ok[KT][4];
+            float mb = -INFINITY;
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int j = j0 + 16 * kt + 4 * g + i;
+                    ok[kt][i] = (j <= p[rt]) && (j >= p_lo[rt]);
+                    sv[kt][i] = s[kt][i] * a.scale_log2;
+                    if (ok[kt][i]) mb = fmaxf(mb, sv[kt][i]);
+                }
+            mb = fmaxf(mb, __shfl_xor(mb, 16, 64));
+            mb = fmaxf(mb, __shfl_xor(mb, 32, 64));
+            const float m_new = fmaxf(m[rt], mb);
+            const float alpha = (m[rt] == -INFINITY) ? 0.f : exp2f(m[rt] - m_new);
+            float pv[KT][4], psum = 0.f;
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    pv[kt][i] = ok[kt][i] ? exp2f(sv[kt][i] - m_new) : 0.f;
+                    psum += pv[kt][i];
+                }
+            l[rt] = l[rt] * alpha + psum;
+            m[rt] = m_new;
+            if constexpr (KT == 2) {
+                // one 16x16x32 instruction per 16 dims: its 8 k slots of lane group g are keys 4g..4g+3 of the
+                // first score tile and of the second
+                U16 pf;
+                pf.u.x = pack2(pv[0][0], pv[0][1]); pf.u.y = pack2(pv[0][2], pv[0][3]);
+                pf.u.z = pack2(pv[1][0], pv[1][1]); pf.u.w = pack2(pv[1][2], pv[1][3]);
+#pragma unroll
+                for (int t = 0; t < DT; ++t) {
+                    const bf16_t* vr = &v_lds[buf][t * 16 + r][4 * g];
+                    U16 vf;
+                    uint2 lo = *(const uint2*)vr, hi = *(const uint2*)(vr + 16);
+                    vf.u = make_uint4(lo.x, lo.y, hi.x, hi.y);
+                    o[rt][t] *= alpha;
+                    o[rt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf.v, o[rt][t], 0, 0, 0);
+                }
+            } else {
+                U8 pf;
+                pf.u.x = pack2(pv[0][0], pv[0][1]); pf.u.y = pack2(pv[0][2], pv[0][3]);
+#pragma unroll
+                for (int t = 0; t < DT; ++t) {
+                    U8 vf; vf.u = *(const uint2*)&v_lds[buf][t * 16 + r][4 * g];
+                    o[rt][t] *= alpha;
+                    o[rt][t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf.v, pf.v, o[rt][t], 0, 0, 0);
+                }
+            }
+        }
+        if (more) park(buf ^ 1);
+        __syncthreads();
+        buf ^= 1;
+    }
+
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        float lt = l[rt];
+        lt += __shfl_xor(lt, 16, 64);
+        lt += __shfl_xor(lt, 32, 64);
+        if (!row_ok[rt]) continue;
+        const float inv = lt > 0.f ? 1.f / lt : 0.f;
+        bf16_t* orow = a.out + ((size_t)(q_tok0 + ti[rt]) * a.n_heads + head[rt]) * D;
+#pragma unroll
+        for (int t = 0; t < DT; ++t) {
+            uint2 w;
+            w.x = pack2(o[rt][t][0] * inv, o[rt][t][1] * inv);
+            w.y = pack2(o[rt][t][2] * inv, o[rt][t][3] * inv);
+            *(uint2*)(orow + t * 16 + 4 * g) = w;
+        }
+    }
+}
+
 // Merge the partial results of a tile of 16 rows whose keys were split over several items.
 // citems: [n][6] = q_tok0, q_len, first row of the tile, first item's partial index, number of items, tile index
 // within its items (each item holds `rt_per_item` tiles).  One block per (tile, kv head).
@@ -330,13 +581,13 @@ static int check_common(const char* who, int n_heads, int n_kv, int page_size, i
 }
 
 // items: [n_items][8] = entry, q_tok0, q_len, pos0, first row, key_lo, key_hi, partial index (-1: writes the output).
-// Each item covers 16 * rt rows (rt = 1, 2 or 4).  The partial workspace holds (partial indices) * rt * n_kv * 16 rows.
+// Each item covers 16 * rt rows (rt = 1 or 2).  The partial workspace holds (partial indices) * rt * n_kv * 16 rows.
 extern "C" int vt_attn_bf16(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
                             const int* items, int n_items, int rt, const int* citems, int n_citems, void* out,
                             float* part_o, float* part_ml, int n_heads, int n_kv, int page_size, int max_blocks,
                             int num_pages, int window, float scale, hipStream_t stream) {
     if (check_common("vt_attn_bf16", n_heads, n_kv, page_size, max_blocks, num_pages)) return -1;
-    VT_REQUIRE(rt == 1 || rt == 2 || rt == 4, "vt_attn_bf16: %d row tiles per item (1, 2 or 4)", rt);
+    VT_REQUIRE(rt == 1 || rt == 2, "vt_attn_bf16: %d row tiles per item (1 or 2)", rt);
     VT_REQUIRE(n_citems == 0 || (part_o && part_ml), "vt_attn_bf16: split keys but no workspace");
     if (n_items <= 0) return 0;
     AttnArgs a;
@@ -347,14 +598,34 @@ extern "C" int vt_attn_bf16(const void* q, const void* k_pages, const void* v_pa
     a.entry_pos0 = nullptr; a.dec_params = nullptr; a.p_max = 0;
     dim3 grid((n_items + 3) / 4, n_kv);
     if (rt == 1) attn_bf16_kernel<false, 1><<<grid, 256, 0, stream>>>(a);
-    else if (rt == 2) attn_bf16_kernel<false, 2><<<grid, 256, 0, stream>>>(a);
-    else attn_bf16_kernel<false, 4><<<grid, 256, 0, stream>>>(a);
+    else attn_bf16_kernel<false, 2><<<grid, 256, 0, stream>>>(a);
     VT_CHECK_LAUNCH("vt_attn_bf16");
     if (n_citems > 0) {
         attn_combine_kernel<false><<<dim3(n_citems, n_kv), 256, 0, stream>>>(citems, part_o, part_ml, (bf16_t*)out,
                                                                             n_heads, n_kv, nullptr, nullptr, 0, window, rt);
         VT_CHECK_LAUNCH("vt_attn_bf16(combine)");
     }
+    return 0;
+}
+
+// Long portions: items [n][8] as above, each 64 * rt rows (rt = 1 or 2) of one entry with all the keys they may
+// see (no split, the partial index is not used); one block of 4 waves per (item, kv head).
+extern "C" int vt_attn_bf16_tiles(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
+                                  const int* items, int n_items, int rt, void* out, int n_heads, int n_kv, int page_size,
+                                  int max_blocks, int num_pages, int window, float scale, hipStream_t stream) {
+    if (check_common("vt_attn_bf16_tiles", n_heads, n_kv, page_size, max_blocks, num_pages)) return -1;
+    VT_REQUIRE(rt == 1 || rt == 2, "vt_attn_bf16_tiles: %d row tiles per wave (1 or 2)", rt);
+    if (n_items <= 0) return 0;
+    AttnArgs a;
+    a.q = (const bf16_t*)q; a.k_pages = (const bf16_t*)k_pages; a.v_pages = (const bf16_t*)v_pages;
+    a.block_table = block_table; a.items = items; a.out = (bf16_t*)out; a.part_o = nullptr; a.part_ml = nullptr;
+    a.n_items = n_items; a.n_heads = n_heads; a.n_kv = n_kv; a.page_size = page_size; a.max_blocks = max_blocks;
+    a.num_pages = num_pages; a.window = window; a.scale_log2 = scale * 1.4426950408889634f;
+    a.entry_pos0 = nullptr; a.dec_params = nullptr; a.p_max = 0;
+    dim3 grid(n_items, n_kv);
+    if (rt == 1) attn_bf16_tile_kernel<1><<<grid, 256, 0, stream>>>(a);
+    else attn_bf16_tile_kernel<2><<<grid, 256, 0, stream>>>(a);
+    VT_CHECK_LAUNCH("vt_attn_bf16_tiles");
     return 0;
 }
 

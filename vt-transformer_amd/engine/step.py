@@ -50,25 +50,64 @@ class AttentionPlan:
     part_ml: Optional[torch.Tensor]
     n_parts: int
     rt: int = 1
+    tile_items: Optional[torch.Tensor] = None     # long entries: items of the LDS-tiled kernel
+    n_tile_items: int = 0
+    tile_rt: int = 1
 
 
 MAX_PARTS = 128     # the merge kernel holds the weights of at most this many items per row tile
 
 
-def choose_row_tiles(entry_start: np.ndarray, group: int, n_kv: int, min_items: int = 768) -> int:
-    """Row tiles (of 16 rows) per attention item: as many as still leave enough items to fill the GPU.  More tiles
-    per item means every key/value block read serves more rows."""
-    rows = int(((entry_start[1:] - entry_start[:-1]).astype(np.int64) * group).sum())
-    for rt in (4, 2):
-        q_len = (entry_start[1:] - entry_start[:-1]).astype(np.int64)
-        items = int(((q_len * group + 16 * rt - 1) // (16 * rt)).sum()) * n_kv
-        if items >= min_items:
-            return rt
-    return 1
+LONG_ENTRY_ROWS = 256   # entries with at least this many (token, head-of-group) rows go to the LDS-tiled kernel
+
+
+def split_entries(entry_start: np.ndarray, group: int) -> Tuple[np.ndarray, np.ndarray]:
+    """(short, long) entry indices: long portions of prompts have rows enough to fill blocks of 64 and more; the
+    rest (decoded tokens, short portions) is cut into 16-row items whose keys may be split."""
+    rows = (entry_start[1:] - entry_start[:-1]).astype(np.int64) * group
+    idx = np.arange(len(rows))
+    return idx[rows < LONG_ENTRY_ROWS], idx[rows >= LONG_ENTRY_ROWS]
+
+
+def plan_tile_items(entry_start: np.ndarray, entry_pos0: np.ndarray, group: int, window: int, n_kv: int,
+                    entries: np.ndarray, rt: Optional[int] = None) -> Tuple[np.ndarray, int]:
+    """Items of the LDS-tiled kernel: 64 * rt rows of one entry and every key they may see, longest first so that
+    the blocks that finish last start first.  Returns (items [n, 8], rt)."""
+    q_len = (entry_start[1:] - entry_start[:-1]).astype(np.int64)[entries]
+    rows = q_len * group
+    if rt is None:
+        rt = 2 if int(((rows + 127) // 128).sum()) * n_kv >= 512 else 1
+    rpi = 64 * rt
+    n_tiles = (rows + rpi - 1) // rpi
+    total = int(n_tiles.sum())
+    if total == 0:
+        return np.zeros((0, ATTN_ITEM_INTS), np.int32), rt
+    which = np.repeat(np.arange(len(entries)), n_tiles)
+    first = np.cumsum(n_tiles) - n_tiles
+    row0 = (np.arange(total) - np.repeat(first, n_tiles)) * rpi
+    ent = entries[which]
+    e_rows, e_len = rows[which], q_len[which]
+    e_pos0, e_start = entry_pos0[ent].astype(np.int64), entry_start[:-1][ent].astype(np.int64)
+    min_p = e_pos0 + row0 // group
+    max_p = e_pos0 + np.minimum(e_rows - 1, row0 + rpi - 1) // group
+    lo = np.maximum(0, min_p - window + 1) if window > 0 else np.zeros_like(min_p)
+    key_lo, key_hi = (lo // 16) * 16, max_p + 1
+    items = np.stack([ent, e_start, e_len, e_pos0, row0, key_lo, key_hi, np.full(total, -1)], axis=1)
+    order = np.argsort(-(key_hi - key_lo), kind="stable")
+    return items[order].astype(np.int32), rt
+
+
+def choose_row_tiles(entry_start: np.ndarray, group: int, n_kv: int, entries: np.ndarray, min_items: int = 768) -> int:
+    """Row tiles (of 16 rows) per item of the per-wave kernel: two if that still leaves enough items to fill the
+    GPU (every key/value block read then serves twice the rows)."""
+    q_len = (entry_start[1:] - entry_start[:-1]).astype(np.int64)[entries]
+    items = int(((q_len * group + 31) // 32).sum()) * n_kv
+    return 2 if items >= min_items else 1
 
 
 def plan_attention_items(entry_start: np.ndarray, entry_pos0: np.ndarray, group: int, window: int, n_kv: int,
-                         target_waves: int = 2048, min_chunk: int = 64, rt: int = 1) -> Tuple[np.ndarray, np.ndarray, int]:
+                         target_waves: int = 2048, min_chunk: int = 32, rt: int = 1,
+                         entries: Optional[np.ndarray] = None) -> Tuple[np.ndarray, np.ndarray, int]:
     """Work items of the bf16 attention kernel for one step.
 
     Rows of an entry are (token, query head of a kv group) pairs, token-major.  An item is 16 * rt rows (rt row
@@ -76,19 +115,22 @@ def plan_attention_items(entry_start: np.ndarray, entry_pos0: np.ndarray, group:
     GPU, an item's keys are cut at absolute multiples of a chunk length into several items whose partial results
     a second kernel merges, tile by tile.
     Returns (items [n, 8], combine items [m, 6], number of partial indices)."""
-    n_entries = len(entry_pos0)
+    if entries is None:
+        entries = np.arange(len(entry_pos0))
     rpi = 16 * rt
-    q_len = (entry_start[1:] - entry_start[:-1]).astype(np.int64)
+    q_len = (entry_start[1:] - entry_start[:-1]).astype(np.int64)[entries]
     rows = q_len * group
     n_tiles = (rows + rpi - 1) // rpi
     total = int(n_tiles.sum())
     if total == 0:
         return np.zeros((0, ATTN_ITEM_INTS), np.int32), np.zeros((0, ATTN_CITEM_INTS), np.int32), 0
-    ent = np.repeat(np.arange(n_entries), n_tiles)
+    which = np.repeat(np.arange(len(entries)), n_tiles)
     first = np.cumsum(n_tiles) - n_tiles
     tile_in_entry = np.arange(total) - np.repeat(first, n_tiles)
     row0 = tile_in_entry * rpi
-    e_rows, e_len, e_pos0, e_start = rows[ent], q_len[ent], entry_pos0[ent].astype(np.int64), entry_start[:-1][ent].astype(np.int64)
+    ent = entries[which]
+    e_rows, e_len = rows[which], q_len[which]
+    e_pos0, e_start = entry_pos0[ent].astype(np.int64), entry_start[:-1][ent].astype(np.int64)
     t_first = row0 // group
     t_last = np.minimum(e_rows - 1, row0 + rpi - 1) // group
     min_p, max_p = e_pos0 + t_first, e_pos0 + t_last
@@ -166,25 +208,29 @@ class StepContext:
 
     def _make_plan(self, key) -> AttentionPlan:
         group, window, n_kv, head_dim = key
-        row_tiles = choose_row_tiles(self.h_entry_start, group, n_kv)
+        short, long = split_entries(self.h_entry_start, group)
+        row_tiles = choose_row_tiles(self.h_entry_start, group, n_kv, short) if len(short) else 1
         items, citems, n_parts = plan_attention_items(self.h_entry_start, self.h_entry_pos0, group, window, n_kv,
-                                                      rt=row_tiles)
+                                                      rt=row_tiles, entries=short)
+        t_items, tile_rt = plan_tile_items(self.h_entry_start, self.h_entry_pos0, group, window, n_kv, long)
         rt = self.rt
         tag = f"attnplan.{group}.{window}.{n_kv}.{head_dim}"
-        flat = np.concatenate([items.reshape(-1), citems.reshape(-1)])
+        flat = np.concatenate([items.reshape(-1), citems.reshape(-1), t_items.reshape(-1)])
         dev = rt.buffer(tag, (max(flat.size, 1),), torch.int32)
         if flat.size:
             dev[:flat.size].copy_(torch.from_numpy(flat))
         d_items = dev[:items.size]
         d_citems = dev[items.size:items.size + citems.size] if citems.size else None
+        d_tiles = dev[items.size + citems.size:flat.size] if t_items.size else None
         part_o = part_ml = None
         if n_parts:
             part_o = rt.buffer("attn.part_o", (n_parts * row_tiles * n_kv * 16 * head_dim,), torch.float32)
             part_ml = rt.buffer("attn.part_ml", (n_parts * row_tiles * n_kv * 16 * 2,), torch.float32)
-        return AttentionPlan(d_items, items.shape[0], d_citems, citems.shape[0], part_o, part_ml, n_parts, row_tiles)
+        return AttentionPlan(d_items, items.shape[0], d_citems, citems.shape[0], part_o, part_ml, n_parts, row_tiles,
+                             d_tiles, t_items.shape[0], tile_rt)
 
 
-def decode_chunk(kv_lens: np.ndarray, p_max: int, target_items: int = 1024, min_chunk: int = 64) -> int:
+def decode_chunk(kv_lens: np.ndarray, p_max: int, target_items: int = 2048, min_chunk: int = 32) -> int:
     """Keys per attention item of a decoding step: small enough to fill the GPU, large enough that the longest
     entry needs at most p_max items; a multiple of 16."""
     total = int(kv_lens.sum())

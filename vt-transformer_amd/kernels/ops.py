@@ -235,8 +235,8 @@ def attention_bf16(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor
     num_pages, kvh, page_size, d = k_pages.shape
     if head_dim % 16 or not 16 <= head_dim <= 256:
         raise KernelError(f"attention_bf16: head size {head_dim} is not a multiple of 16 in 16..256")
-    if rt not in (1, 2, 4):
-        raise KernelError(f"attention_bf16: {rt} row tiles per item (1, 2 or 4)")
+    if rt not in (1, 2):
+        raise KernelError(f"attention_bf16: {rt} row tiles per item (1 or 2)")
     _chk(q, "attention_bf16.q", torch.bfloat16, (n, n_heads * head_dim))
     _chk(k_pages, "attention_bf16.k_pages", torch.bfloat16, (num_pages, n_kv, page_size, head_dim))
     _chk(v_pages, "attention_bf16.v_pages", torch.bfloat16, (num_pages, n_kv, head_dim, page_size))
@@ -257,6 +257,31 @@ def attention_bf16(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor
     _run(lib, "vt_attn_bf16", _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(block_table), _ptr(items), _i(n_items), _i(rt),
          _ptr(citems), _i(n_citems), _ptr(out), _ptr(part_o), _ptr(part_ml), _i(n_heads), _i(n_kv), _i(page_size),
          _i(block_table.shape[1]), _i(num_pages), _i(window), _f(scale), _stream())
+    return out
+
+
+def attention_bf16_tiles(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
+                         items: torch.Tensor, n_items: int, out: torch.Tensor, n_heads: int, n_kv: int, head_dim: int,
+                         window: int, scale: float, rt: int = 1) -> torch.Tensor:
+    """Long portions: `items` as for attention_bf16, each 64 * rt rows of one entry against all the keys they may
+    see; key and value blocks go through LDS once per block of four waves."""
+    n = q.shape[0]
+    num_pages, kvh, page_size, d = k_pages.shape
+    if head_dim % 16 or not 16 <= head_dim <= 256:
+        raise KernelError(f"attention_bf16_tiles: head size {head_dim} is not a multiple of 16 in 16..256")
+    if rt not in (1, 2):
+        raise KernelError(f"attention_bf16_tiles: {rt} row tiles per wave (1 or 2)")
+    _chk(q, "attention_bf16_tiles.q", torch.bfloat16, (n, n_heads * head_dim))
+    _chk(k_pages, "attention_bf16_tiles.k_pages", torch.bfloat16, (num_pages, n_kv, page_size, head_dim))
+    _chk(v_pages, "attention_bf16_tiles.v_pages", torch.bfloat16, (num_pages, n_kv, head_dim, page_size))
+    _chk(block_table, "attention_bf16_tiles.block_table", torch.int32)
+    _chk(items, "attention_bf16_tiles.items", torch.int32)
+    _chk(out, "attention_bf16_tiles.out", torch.bfloat16, (n, n_heads * head_dim))
+    if items.numel() < n_items * ATTN_ITEM_INTS:
+        raise KernelError("attention_bf16_tiles: item list shorter than n_items")
+    _run(load_lib("vt_attn_bf16", head_dim), "vt_attn_bf16_tiles", _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
+         _ptr(items), _i(n_items), _i(rt), _ptr(out), _i(n_heads), _i(n_kv), _i(page_size), _i(block_table.shape[1]),
+         _i(num_pages), _i(window), _f(scale), _stream())
     return out
 
 

@@ -122,7 +122,11 @@ class PagedAttention(Part):
                                       ctx.decode_p_max, out, part_o, part_ml, nh, nkv, d, self.window, self.scale)
         else:
             plan = ctx.attention_plan(nh // nkv, self.window, nkv, d)
-            ops.attention_bf16(q, cache.k, cache.v, cache.block_table, plan.items, plan.n_items, plan.citems,
-                               plan.n_citems, out, plan.part_o, plan.part_ml, nh, nkv, d, self.window, self.scale,
-                               max_part=plan.n_parts, rt=plan.rt)
+            if plan.n_items:        # decoded tokens and short portions: 16-row items, keys split where that helps
+                ops.attention_bf16(q, cache.k, cache.v, cache.block_table, plan.items, plan.n_items, plan.citems,
+                                   plan.n_citems, out, plan.part_o, plan.part_ml, nh, nkv, d, self.window, self.scale,
+                                   max_part=plan.n_parts, rt=plan.rt)
+            if plan.n_tile_items:   # long portions: key/value blocks through LDS, shared by four waves
+                ops.attention_bf16_tiles(q, cache.k, cache.v, cache.block_table, plan.tile_items, plan.n_tile_items,
+                                         out, nh, nkv, d, self.window, self.scale, rt=plan.tile_rt)
         return linear(rt, out, self.w_o, self.b_o, "attn.o")
