@@ -456,7 +456,7 @@ def test_sample_top_k_and_top_p():
 
 @pytest.mark.parametrize("nh,kvh,d", [(28, 4, 128), (4, 2, 16), (16, 1, 48)])
 @pytest.mark.parametrize("window", [0, 37])
-@pytest.mark.parametrize("chunk", [16, 64, 256])
+@pytest.mark.parametrize("chunk", [64, 128, 1024])
 def test_attention_decode_kernel(nh, kvh, d, window, chunk):
     """One token per entry, the keys cut into items on the device from the positions in memory."""
     o = ops()
@@ -469,7 +469,7 @@ def test_attention_decode_kernel(nh, kvh, d, window, chunk):
     kp, vp, bt = make_pages(ks, vs, lens, 16, torch.bfloat16, 9)
     n = len(lens)
     q = torch.cat(qs).reshape(n, nh * d).to(torch.bfloat16).to(DEV)
-    p_max = 64
+    p_max = 16
     if -(-max(lens) // chunk) > p_max:
         pytest.skip("the host never chooses a chunk that needs more items than p_max")
     part_o = torch.full((n * p_max * kvh * 16 * d,), float("nan"), device=DEV)

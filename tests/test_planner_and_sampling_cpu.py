@@ -73,10 +73,16 @@ def test_tile_items_cover_the_long_entries(group, window, rt):
 
 
 def test_decode_chunk():
-    assert decode_chunk(np.array([1]), 64) == 32
-    assert decode_chunk(np.array([8192]), 64) % 16 == 0 and decode_chunk(np.array([8192]), 64) * 64 >= 8192
-    c = decode_chunk(np.full(64, 1024), 64)
-    assert c % 16 == 0 and 32 <= c <= 128
+    from vt_transformer_amd.engine.step import decode_bucket
+    from vt_transformer_amd.parts.attention import decode_bucket as part_bucket
+    assert decode_chunk(np.array([1]), 16) == 64
+    c = decode_chunk(np.array([8192]), 16, n_kv=4)             # one entry: cut into as many items as allowed
+    assert c % 64 == 0 and -(-8192 // c) <= 16
+    assert decode_chunk(np.full(256, 1024), 16, n_kv=4) == 1024  # many entries: one item each
+    c = decode_chunk(np.full(8, 1040), 16, n_kv=4)
+    assert c % 64 == 0 and -(-1040 // c) * 8 * 4 >= 64
+    assert [decode_bucket(n) for n in (1, 2, 3, 4, 7, 8, 64, 1000)] == [0, 1, 1, 2, 2, 3, 6, 7]
+    assert all(decode_bucket(n) == part_bucket(n) for n in range(1, 300))
 
 
 def test_uniform_numbers_depend_only_on_seed_and_counter():

@@ -57,14 +57,71 @@ struct AttnArgs {
     const int* dec_params;  // [0] = chunk: keys per item (a multiple of 16), read from memory so that a
                             //       captured launch can be replayed with another value
     int p_max;              // items per entry
+    int ps_shift;           // log2(page_size) if it is a power of two, else -1
 };
+
+__device__ __forceinline__ int page_index(const AttnArgs& a, int j) {
+    return a.ps_shift >= 0 ? (j >> a.ps_shift) : (j / a.page_size);
+}
 
 union U8 { uint2 u; bf16x4_t v; };
 union U16 { uint4 u; bf16x8_t v; };
 
+typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+
+// two floats to two bf16 (round to nearest even) in one instruction
 __device__ __forceinline__ unsigned pack2(float a, float b) {
-    return (unsigned)f32_to_bf16(a) | ((unsigned)f32_to_bf16(b) << 16);
+    f32x2_t v = {a, b};
+    return __builtin_bit_cast(unsigned, __builtin_convertvector(v, bf16x2_t));
 }
+
+// One step of the running softmax of a row over NK*4 scores held by this lane (s[kt][i] = raw dot product of key
+// j0 + 16 kt + 4 g + i), shared with the three other lanes of the row.  `full`: every key of the block is visible
+// to every row of the tile, so no score is tested.  Leaves the probabilities as bf16 pairs in pk, the factor for
+// what was accumulated before in alpha.  Maxima are kept in the exp2 domain (scores times scale*log2 e).
+template <int NK>
+__device__ __forceinline__ void softmax_step(const f32x4_t (&s)[NK], int j0, int g, int p, int p_lo, bool full,
+                                             float scale_log2, float& m, float& l, float& alpha, unsigned (&pk)[NK * 2]) {
+    float mb = -INFINITY;
+    if (full) {
+#pragma unroll
+        for (int kt = 0; kt < NK; ++kt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) mb = fmaxf(mb, s[kt][i]);
+    } else {
+#pragma unroll
+        for (int kt = 0; kt < NK; ++kt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int j = j0 + 16 * kt + 4 * g + i;
+                if (j <= p && j >= p_lo) mb = fmaxf(mb, s[kt][i]);
+            }
+    }
+    mb *= scale_log2;
+    mb = fmaxf(mb, __shfl_xor(mb, 16, 64));
+    mb = fmaxf(mb, __shfl_xor(mb, 32, 64));
+    const float m_new = fmaxf(m, mb);
+    alpha = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m - m_new);
+    float pv[NK][4], psum = 0.f;
+#pragma unroll
+    for (int kt = 0; kt < NK; ++kt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int j = j0 + 16 * kt + 4 * g + i;
+            const bool ok = full || (j <= p && j >= p_lo);   // a visible key makes m_new finite
+            pv[kt][i] = ok ? __builtin_amdgcn_exp2f(fmaf(s[kt][i], scale_log2, -m_new)) : 0.f;
+            psum += pv[kt][i];
+        }
+    l = l * alpha + psum;
+    m = m_new;
+#pragma unroll
+    for (int kt = 0; kt < NK; ++kt) {
+        pk[2 * kt] = pack2(pv[kt][0], pv[kt][1]);
+        pk[2 * kt + 1] = pack2(pv[kt][2], pv[kt][3]);
+    }
+}
+
 
 constexpr bool WIDE = (D % 32 == 0);           // 16x16x32 instruction for the scores when the head size allows
 constexpr int QSTEPS = WIDE ? D / 32 : D / 16;
@@ -81,7 +138,7 @@ struct KVBlock {
 // `pg` is the page of the block (read from the block table ahead of time, so that the loads below do not wait for it)
 __device__ __forceinline__ void load_block(KVBlock& b, const AttnArgs& a, int pg, int j0, int kvh, int r, int g) {
     const int ps = a.page_size;
-    const int blk = j0 / ps;
+    const int blk = page_index(a, j0);
     b.ok = pg >= 0 && pg < a.num_pages;   // a page the window has passed: its keys are masked for every row
     if (!b.ok) return;
     const int off = j0 - blk * ps;
@@ -102,22 +159,26 @@ __device__ __forceinline__ void load_block(KVBlock& b, const AttnArgs& a, int pg
 template <bool DECODE, int RT>
 __global__ __launch_bounds__(256) void attn_bf16_kernel(AttnArgs a) {
     const int wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int item = blockIdx.x * 4 + wv;
+    // decoding: the four waves of a block share one item and take its key blocks in turn; otherwise one item per wave
+    const int item = DECODE ? (int)blockIdx.x : (int)blockIdx.x * 4 + wv;
     if (item >= a.n_items) return;
     int entry, q_tok0, q_len, pos0, q_row0, key_lo, key_hi, part;
     if (DECODE) {
         // item = (entry, part p): keys [p*chunk, (p+1)*chunk) of the entry's one token
         const int chunk = a.dec_params[0];
-        entry = item / a.p_max;
-        const int pi = item - entry * a.p_max;
+        // Entries vary fastest: consecutive blocks go to different XCDs, and when every entry has one item the
+        // blocks that have work are consecutive (with parts fastest they would all land on one XCD in eight).
+        const int n_entries = a.n_items / a.p_max;
+        const int pi = item / n_entries;
+        entry = item - pi * n_entries;
         q_tok0 = entry; q_len = 1; q_row0 = 0;
         pos0 = a.entry_pos0[entry];
         const int lo = a.window > 0 ? max(0, pos0 - a.window + 1) : 0;
         const int p_first = ((lo >> 4) << 4) / chunk, p_last = pos0 / chunk;
-        if (pi < p_first || pi > p_last) return;
+        if (pi < p_first || pi > p_last) return;      // the whole block leaves together
         key_lo = max((lo >> 4) << 4, pi * chunk);
         key_hi = min(pos0 + 1, (pi + 1) * chunk);
-        part = (p_first == p_last) ? -1 : item;
+        part = (p_first == p_last) ? -1 : entry * a.p_max + pi;
     } else {
         const int* it = a.items + (size_t)item * ITEM_INTS;
         entry = it[0]; q_tok0 = it[1]; q_len = it[2]; pos0 = it[3]; q_row0 = it[4];
@@ -130,7 +191,7 @@ __global__ __launch_bounds__(256) void attn_bf16_kernel(AttnArgs a) {
     const int n_rows = q_len * G;
 
     bool row_ok[RT];
-    int ti[RT], head[RT], p[RT], p_lo[RT], tile_hi[RT], tile_lo[RT];
+    int ti[RT], head[RT], p[RT], p_lo[RT], tile_hi[RT], tile_lo[RT], tile_first_p[RT], tile_last_lo[RT];
     bf16x8_t q8[RT][WIDE ? QSTEPS : 1];
     bf16x4_t q4[RT][WIDE ? 1 : QSTEPS];
     f32x4_t o[RT][DT];
@@ -148,6 +209,9 @@ __global__ __launch_bounds__(256) void attn_bf16_kernel(AttnArgs a) {
         const int last_row = min(n_rows - 1, q_row0 + rt * 16 + 15), first_row = min(n_rows - 1, q_row0 + rt * 16);
         tile_hi[rt] = (q_row0 + rt * 16 < n_rows) ? pos0 + last_row / G : -1;
         tile_lo[rt] = a.window > 0 ? pos0 + first_row / G - a.window + 1 : 0;
+        // a block whose keys lie between these two is visible to every row of the tile
+        tile_first_p[rt] = pos0 + first_row / G;
+        tile_last_lo[rt] = a.window > 0 ? pos0 + last_row / G - a.window + 1 : 0;
         const bf16_t* qrow = a.q + ((size_t)(q_tok0 + ti[rt]) * a.n_heads + head[rt]) * D;
         if constexpr (WIDE) {
 #pragma unroll
@@ -170,72 +234,103 @@ __global__ __launch_bounds__(256) void attn_bf16_kernel(AttnArgs a) {
     int cache_base = key_lo / ps;
     int pg_lane = (cache_base + lane <= last_page) ? bt[cache_base + lane] : -1;
     auto page_of = [&](int j) {
-        int blk = j / ps;
+        int blk = page_index(a, j);
         if (blk >= cache_base + 64) {
             cache_base = blk;
             pg_lane = (cache_base + lane <= last_page) ? bt[cache_base + lane] : -1;
         }
         return __builtin_amdgcn_readlane(pg_lane, __builtin_amdgcn_readfirstlane(blk - cache_base));
     };
-    KVBlock cur, nxt;
-    nxt.ok = false;
-    load_block(cur, a, page_of(key_lo), key_lo, kvh, r, g);
-    for (int j0 = key_lo; j0 < key_hi; j0 += 16) {
-        // the next block's loads are in flight while this one is computed
-        if (j0 + 16 < key_hi) load_block(nxt, a, page_of(j0 + 16), j0 + 16, kvh, r, g);
-        if (cur.ok) {
+    // one block of 16 keys against the RT row tiles of this wave
+    auto multiply = [&](const KVBlock& cur, int j0) {
+        if (!cur.ok) return;
 #pragma unroll
-            for (int rt = 0; rt < RT; ++rt) {
-                if (j0 > tile_hi[rt] || j0 + 15 < tile_lo[rt]) continue;   // every key masked for every row of the tile
-                f32x4_t s = (f32x4_t){0.f, 0.f, 0.f, 0.f};
-                if constexpr (WIDE) {
+        for (int rt = 0; rt < RT; ++rt) {
+            if (j0 > tile_hi[rt] || j0 + 15 < tile_lo[rt]) continue;   // every key masked for every row of the tile
+            f32x4_t s = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+            if constexpr (WIDE) {
 #pragma unroll
-                    for (int st = 0; st < QSTEPS; ++st) {
-                        U16 t; t.u = cur.k8[st];
-                        s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(t.v, q8[rt][st], s, 0, 0, 0);
-                    }
+                for (int st = 0; st < QSTEPS; ++st) {
+                    U16 t; t.u = cur.k8[st];
+                    s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(t.v, q8[rt][st], s, 0, 0, 0);
+                }
+            } else {
+#pragma unroll
+                for (int st = 0; st < QSTEPS; ++st) {
+                    U8 t; t.u = cur.k4[st];
+                    s = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(t.v, q4[rt][st], s, 0, 0, 0);
+                }
+            }
+            // s[i] is key j0 + 4 g + i against row r of the tile
+            const f32x4_t sc[1] = {s};
+            const bool full = (j0 + 15 <= tile_first_p[rt]) && (j0 >= tile_last_lo[rt]);
+            float alpha;
+            unsigned pk[2];
+            softmax_step<1>(sc, j0, g, p[rt], p_lo[rt], full, a.scale_log2, m[rt], l[rt], alpha, pk);
+            U8 pf;
+            pf.u.x = pk[0];
+            pf.u.y = pk[1];
+            const bool rescale = __any(alpha != 1.f);      // the maximum of some row moved
+#pragma unroll
+            for (int t = 0; t < DT; ++t) {
+                U8 vf; vf.u = cur.v[t];
+                if (rescale) o[rt][t] *= alpha;
+                o[rt][t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf.v, pf.v, o[rt][t], 0, 0, 0);
+            }
+        }
+    };
+    // Two register buffers in turn: while one block is multiplied the other one is on its way from memory.
+    KVBlock ba, bb;
+    ba.ok = bb.ok = false;
+    const int j_first = key_lo + (DECODE ? 16 * wv : 0), j_step = DECODE ? 64 : 16;
+    if (j_first < key_hi) load_block(ba, a, page_of(j_first), j_first, kvh, r, g);
+    for (int j0 = j_first; j0 < key_hi; j0 += 2 * j_step) {
+        const int j1 = j0 + j_step, j2 = j0 + 2 * j_step;
+        if (j1 < key_hi) load_block(bb, a, page_of(j1), j1, kvh, r, g);
+        multiply(ba, j0);
+        if (j2 < key_hi) load_block(ba, a, page_of(j2), j2, kvh, r, g);
+        if (j1 < key_hi) multiply(bb, j1);
+    }
+
+    if constexpr (DECODE) {
+        // The four waves hold partial results over disjoint keys of the same rows: merge them through LDS, half
+        // of a large head at a time, and let all 256 threads write the result.
+        constexpr int DH = (D > 128) ? D / 2 : D;
+        __shared__ __attribute__((aligned(16))) float so[4][16][DH + 4];
+        __shared__ float sm[4][16], sl[4][16];
+        float lt = l[0];
+        lt += __shfl_xor(lt, 16, 64);
+        lt += __shfl_xor(lt, 32, 64);
+        if (g == 0) { sm[wv][r] = m[0]; sl[wv][r] = lt; }
+        const int n_valid = min(16, n_rows);
+#pragma unroll
+        for (int half = 0; half < D / DH; ++half) {
+            if (half) __syncthreads();
+#pragma unroll
+            for (int t = 0; t < DH / 16; ++t) *(f32x4_t*)&so[wv][r][t * 16 + 4 * g] = o[0][half * (DH / 16) + t];
+            __syncthreads();
+            for (int idx = threadIdx.x; idx < n_valid * DH; idx += 256) {
+                const int rr = idx / DH, dd = idx - rr * DH;
+                const float mx = fmaxf(fmaxf(sm[0][rr], sm[1][rr]), fmaxf(sm[2][rr], sm[3][rr]));
+                float num = 0.f, den = 0.f;
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    const float wt = (sm[w][rr] == -INFINITY) ? 0.f : exp2f(sm[w][rr] - mx);
+                    num += wt * so[w][rr][dd];
+                    den += wt * sl[w][rr];
+                }
+                const int d = half * DH + dd;
+                if (part < 0) {
+                    const int head_r = kvh * G + rr;      // one token per entry: row = head of the group
+                    a.out[((size_t)q_tok0 * a.n_heads + head_r) * D + d] = f32_to_bf16(den > 0.f ? num / den : 0.f);
                 } else {
-#pragma unroll
-                    for (int st = 0; st < QSTEPS; ++st) {
-                        U8 t; t.u = cur.k4[st];
-                        s = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(t.v, q4[rt][st], s, 0, 0, 0);
-                    }
-                }
-                // s[i] is key j0 + 4 g + i against row r of the tile
-                float sv[4];
-                bool ok[4];
-                float mb = -INFINITY;
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int j = j0 + 4 * g + i;
-                    ok[i] = (j <= p[rt]) && (j >= p_lo[rt]);
-                    sv[i] = s[i] * a.scale_log2;
-                    if (ok[i]) mb = fmaxf(mb, sv[i]);
-                }
-                mb = fmaxf(mb, __shfl_xor(mb, 16, 64));
-                mb = fmaxf(mb, __shfl_xor(mb, 32, 64));
-                const float m_new = fmaxf(m[rt], mb);
-                const float alpha = (m[rt] == -INFINITY) ? 0.f : exp2f(m[rt] - m_new);
-                float pv[4], psum = 0.f;
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    pv[i] = ok[i] ? exp2f(sv[i] - m_new) : 0.f;
-                    psum += pv[i];
-                }
-                l[rt] = l[rt] * alpha + psum;
-                m[rt] = m_new;
-                U8 pf;
-                pf.u.x = pack2(pv[0], pv[1]);
-                pf.u.y = pack2(pv[2], pv[3]);
-#pragma unroll
-                for (int t = 0; t < DT; ++t) {
-                    U8 vf; vf.u = cur.v[t];
-                    o[rt][t] *= alpha;
-                    o[rt][t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf.v, pf.v, o[rt][t], 0, 0, 0);
+                    const size_t slot = ((size_t)part * a.n_kv + kvh) * 16 + rr;
+                    a.part_o[slot * D + d] = num;
+                    if (d == 0) { a.part_ml[slot * 2] = mx; a.part_ml[slot * 2 + 1] = den; }
                 }
             }
         }
-        cur = nxt;
+        return;
     }
 
 #pragma unroll
@@ -302,7 +397,7 @@ __global__ __launch_bounds__(256) void attn_bf16_tile_kernel(AttnArgs a) {
     const int ps = a.page_size;
 
     bool row_ok[RT];
-    int ti[RT], head[RT], p[RT], p_lo[RT], tile_hi[RT], tile_lo[RT];
+    int ti[RT], head[RT], p[RT], p_lo[RT], tile_hi[RT], tile_lo[RT], tile_first_p[RT], tile_last_lo[RT];
     bf16x8_t q8[RT][WIDE ? QSTEPS : 1];
     bf16x4_t q4[RT][WIDE ? 1 : QSTEPS];
     f32x4_t o[RT][DT];
@@ -320,6 +415,8 @@ __global__ __launch_bounds__(256) void attn_bf16_tile_kernel(AttnArgs a) {
         const int last_row = min(n_rows - 1, row0 + 15), first_row = min(n_rows - 1, row0);
         tile_hi[rt] = (row0 < n_rows) ? pos0 + last_row / G : -1;
         tile_lo[rt] = a.window > 0 ? pos0 + first_row / G - a.window + 1 : 0;
+        tile_first_p[rt] = pos0 + first_row / G;
+        tile_last_lo[rt] = a.window > 0 ? pos0 + last_row / G - a.window + 1 : 0;
         const bf16_t* qrow = a.q + ((size_t)(q_tok0 + ti[rt]) * a.n_heads + head[rt]) * D;
         if constexpr (WIDE) {
 #pragma unroll
@@ -341,42 +438,42 @@ __global__ __launch_bounds__(256) void attn_bf16_tile_kernel(AttnArgs a) {
         const int pgi = page_base + tid;
         if (tid < PAGE_WINDOW) s_pages[tid] = (pgi <= last_page) ? bt[pgi] : -1;
     };
-    uint4 kreg[KPT], vreg[VPT];
-    auto fetch = [&](int j0) {   // this thread's pieces of keys [j0, j0 + KB) from the pages into registers
+    struct Stage { uint4 k[KPT]; uint4 v[VPT]; };
+    auto fetch = [&](Stage& st_, int j0) {   // this thread's pieces of keys [j0, j0 + KB) from the pages into registers
 #pragma unroll
         for (int i = 0; i < KPT; ++i) {
             const int idx = tid + 256 * i;
-            kreg[i] = make_uint4(0, 0, 0, 0);
+            st_.k[i] = make_uint4(0, 0, 0, 0);
             if (idx < KPIECES) {
                 const int key = idx / (D / 8), c = idx - key * (D / 8);
                 const int j = j0 + key;
-                const int blk = j / ps;
+                const int blk = page_index(a, j);
                 const int pg = (j < key_hi) ? s_pages[blk - page_base] : -1;
                 if (pg >= 0 && pg < a.num_pages)
-                    kreg[i] = *(const uint4*)(a.k_pages + (((size_t)pg * a.n_kv + kvh) * ps + (j - blk * ps)) * D + c * 8);
+                    st_.k[i] = *(const uint4*)(a.k_pages + (((size_t)pg * a.n_kv + kvh) * ps + (j - blk * ps)) * D + c * 8);
             }
         }
 #pragma unroll
         for (int i = 0; i < VPT; ++i) {
             const int idx = tid + 256 * i;
-            vreg[i] = make_uint4(0, 0, 0, 0);
+            st_.v[i] = make_uint4(0, 0, 0, 0);
             if (idx < VPIECES) {
                 const int d = idx / (KB / 8), kg = idx - d * (KB / 8);
                 const int j = j0 + kg * 8;
-                const int blk = j / ps;
+                const int blk = page_index(a, j);
                 const int pg = (j < key_hi) ? s_pages[blk - page_base] : -1;
                 if (pg >= 0 && pg < a.num_pages)
-                    vreg[i] = *(const uint4*)(a.v_pages + (((size_t)pg * a.n_kv + kvh) * D + d) * ps + (j - blk * ps));
+                    st_.v[i] = *(const uint4*)(a.v_pages + (((size_t)pg * a.n_kv + kvh) * D + d) * ps + (j - blk * ps));
             }
         }
     };
-    auto park = [&](int buf) {
+    auto park = [&](const Stage& st_, int buf) {
 #pragma unroll
         for (int i = 0; i < KPT; ++i) {
             const int idx = tid + 256 * i;
             if (idx < KPIECES) {
                 const int key = idx / (D / 8), c = idx - key * (D / 8);
-                *(uint4*)&k_lds[buf][key][c * 8] = kreg[i];
+                *(uint4*)&k_lds[buf][key][c * 8] = st_.k[i];
             }
         }
 #pragma unroll
@@ -384,29 +481,13 @@ __global__ __launch_bounds__(256) void attn_bf16_tile_kernel(AttnArgs a) {
             const int idx = tid + 256 * i;
             if (idx < VPIECES) {
                 const int d = idx / (KB / 8), kg = idx - d * (KB / 8);
-                *(uint4*)&v_lds[buf][d][kg * 8] = vreg[i];
+                *(uint4*)&v_lds[buf][d][kg * 8] = st_.v[i];
             }
         }
     };
 
-    fill_pages();
-    __syncthreads();
-    fetch(key_lo);
-    park(0);
-    __syncthreads();
-    int buf = 0;
-    for (int j0 = key_lo; j0 < key_hi; j0 += KB) {
-        const int jn = j0 + KB;
-        const bool more = jn < key_hi;
-        if (more) {
-            if ((jn + KB - 1) / ps >= page_base + PAGE_WINDOW) {   // the same decision in every thread
-                __syncthreads();
-                page_base = jn / ps;
-                fill_pages();
-                __syncthreads();
-            }
-            fetch(jn);   // in flight while this block is multiplied
-        }
+    // one key block (in LDS buffer `buf`, keys from j0) against the RT row tiles of this wave
+    auto multiply = [&](int buf, int j0) {
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
             if (j0 > tile_hi[rt] || j0 + KB - 1 < tile_lo[rt]) continue;   // every key masked for every row of the tile
@@ -430,61 +511,66 @@ __global__ __launch_bounds__(256) void attn_bf16_tile_kernel(AttnArgs a) {
                 }
             }
             // s[kt][i] is key j0 + 16 kt + 4 g + i against row r of the tile
-            float sv[KT][4];
-            bool ok[KT][4];
-            float mb = -INFINITY;
-#pragma unroll
-            for (int kt = 0; kt < KT; ++kt)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int j = j0 + 16 * kt + 4 * g + i;
-                    ok[kt][i] = (j <= p[rt]) && (j >= p_lo[rt]);
-                    sv[kt][i] = s[kt][i] * a.scale_log2;
-                    if (ok[kt][i]) mb = fmaxf(mb, sv[kt][i]);
-                }
-            mb = fmaxf(mb, __shfl_xor(mb, 16, 64));
-            mb = fmaxf(mb, __shfl_xor(mb, 32, 64));
-            const float m_new = fmaxf(m[rt], mb);
-            const float alpha = (m[rt] == -INFINITY) ? 0.f : exp2f(m[rt] - m_new);
-            float pv[KT][4], psum = 0.f;
-#pragma unroll
-            for (int kt = 0; kt < KT; ++kt)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    pv[kt][i] = ok[kt][i] ? exp2f(sv[kt][i] - m_new) : 0.f;
-                    psum += pv[kt][i];
-                }
-            l[rt] = l[rt] * alpha + psum;
-            m[rt] = m_new;
+            const bool full = (j0 + KB - 1 <= tile_first_p[rt]) && (j0 >= tile_last_lo[rt]);
+            float alpha;
+            unsigned pk[KT * 2];
+            softmax_step<KT>(s, j0, g, p[rt], p_lo[rt], full, a.scale_log2, m[rt], l[rt], alpha, pk);
+            const bool rescale = __any(alpha != 1.f);      // the maximum of some row moved
             if constexpr (KT == 2) {
                 // one 16x16x32 instruction per 16 dims: its 8 k slots of lane group g are keys 4g..4g+3 of the
                 // first score tile and of the second
                 U16 pf;
-                pf.u.x = pack2(pv[0][0], pv[0][1]); pf.u.y = pack2(pv[0][2], pv[0][3]);
-                pf.u.z = pack2(pv[1][0], pv[1][1]); pf.u.w = pack2(pv[1][2], pv[1][3]);
+                pf.u = make_uint4(pk[0], pk[1], pk[2], pk[3]);
 #pragma unroll
                 for (int t = 0; t < DT; ++t) {
                     const bf16_t* vr = &v_lds[buf][t * 16 + r][4 * g];
                     U16 vf;
                     uint2 lo = *(const uint2*)vr, hi = *(const uint2*)(vr + 16);
                     vf.u = make_uint4(lo.x, lo.y, hi.x, hi.y);
-                    o[rt][t] *= alpha;
+                    if (rescale) o[rt][t] *= alpha;
                     o[rt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf.v, o[rt][t], 0, 0, 0);
                 }
             } else {
                 U8 pf;
-                pf.u.x = pack2(pv[0][0], pv[0][1]); pf.u.y = pack2(pv[0][2], pv[0][3]);
+                pf.u.x = pk[0]; pf.u.y = pk[1];
 #pragma unroll
                 for (int t = 0; t < DT; ++t) {
                     U8 vf; vf.u = *(const uint2*)&v_lds[buf][t * 16 + r][4 * g];
-                    o[rt][t] *= alpha;
+                    if (rescale) o[rt][t] *= alpha;
                     o[rt][t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf.v, pf.v, o[rt][t], 0, 0, 0);
                 }
             }
         }
-        if (more) park(buf ^ 1);
+    };
+    auto window_for = [&](int j) {   // make sure the page ids of block j are in LDS (the same decision in every thread)
+        if (page_index(a, j + KB - 1) >= page_base + PAGE_WINDOW) {
+            __syncthreads();
+            page_base = page_index(a, j);
+            fill_pages();
+            __syncthreads();
+        }
+    };
+
+    // Two sets of staging registers and two LDS buffers: a block is fetched two steps before it is multiplied, so
+    // its loads have two multiplications' time to arrive.
+    Stage sa, sb;
+    fill_pages();
+    __syncthreads();
+    fetch(sa, key_lo);
+    if (key_lo + KB < key_hi) { window_for(key_lo + KB); fetch(sb, key_lo + KB); }
+    park(sa, 0);
+    __syncthreads();
+    for (int j0 = key_lo; j0 < key_hi; j0 += 2 * KB) {
+        const int j1 = j0 + KB, j2 = j0 + 2 * KB, j3 = j0 + 3 * KB;
+        if (j2 < key_hi) { window_for(j2); fetch(sa, j2); }
+        multiply(0, j0);
+        if (j1 < key_hi) park(sb, 1);
         __syncthreads();
-        buf ^= 1;
+        if (j1 >= key_hi) break;
+        if (j3 < key_hi) { window_for(j3); fetch(sb, j3); }
+        multiply(1, j1);
+        if (j2 < key_hi) park(sa, 0);
+        __syncthreads();
     }
 
 #pragma unroll
@@ -572,6 +658,12 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const int* __restrict
 
 extern "C" int vt_attn_bf16_head_dim() { return D; }
 
+static int shift_of(int v) {
+    for (int sft = 0; sft < 31; ++sft)
+        if ((1 << sft) == v) return sft;
+    return -1;
+}
+
 static int check_common(const char* who, int n_heads, int n_kv, int page_size, int max_blocks, int num_pages) {
     VT_REQUIRE(n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "%s: bad heads %d/%d", who, n_heads, n_kv);
     VT_REQUIRE(page_size > 0 && page_size % 16 == 0, "%s: page size %d is not a multiple of 16", who, page_size);
@@ -595,7 +687,7 @@ extern "C" int vt_attn_bf16(const void* q, const void* k_pages, const void* v_pa
     a.block_table = block_table; a.items = items; a.out = (bf16_t*)out; a.part_o = part_o; a.part_ml = part_ml;
     a.n_items = n_items; a.n_heads = n_heads; a.n_kv = n_kv; a.page_size = page_size; a.max_blocks = max_blocks;
     a.num_pages = num_pages; a.window = window; a.scale_log2 = scale * 1.4426950408889634f;
-    a.entry_pos0 = nullptr; a.dec_params = nullptr; a.p_max = 0;
+    a.entry_pos0 = nullptr; a.dec_params = nullptr; a.p_max = 0; a.ps_shift = shift_of(page_size);
     dim3 grid((n_items + 3) / 4, n_kv);
     if (rt == 1) attn_bf16_kernel<false, 1><<<grid, 256, 0, stream>>>(a);
     else attn_bf16_kernel<false, 2><<<grid, 256, 0, stream>>>(a);
@@ -621,7 +713,7 @@ extern "C" int vt_attn_bf16_tiles(const void* q, const void* k_pages, const void
     a.block_table = block_table; a.items = items; a.out = (bf16_t*)out; a.part_o = nullptr; a.part_ml = nullptr;
     a.n_items = n_items; a.n_heads = n_heads; a.n_kv = n_kv; a.page_size = page_size; a.max_blocks = max_blocks;
     a.num_pages = num_pages; a.window = window; a.scale_log2 = scale * 1.4426950408889634f;
-    a.entry_pos0 = nullptr; a.dec_params = nullptr; a.p_max = 0;
+    a.entry_pos0 = nullptr; a.dec_params = nullptr; a.p_max = 0; a.ps_shift = shift_of(page_size);
     dim3 grid(n_items, n_kv);
     if (rt == 1) attn_bf16_tile_kernel<1><<<grid, 256, 0, stream>>>(a);
     else attn_bf16_tile_kernel<2><<<grid, 256, 0, stream>>>(a);
@@ -648,8 +740,8 @@ extern "C" int vt_attn_bf16_decode(const void* q, const void* k_pages, const voi
     a.block_table = block_table; a.items = nullptr; a.out = (bf16_t*)out; a.part_o = part_o; a.part_ml = part_ml;
     a.n_items = n_entries * p_max; a.n_heads = n_heads; a.n_kv = n_kv; a.page_size = page_size; a.max_blocks = max_blocks;
     a.num_pages = num_pages; a.window = window; a.scale_log2 = scale * 1.4426950408889634f;
-    a.entry_pos0 = entry_pos0; a.dec_params = dec_params; a.p_max = p_max;
-    attn_bf16_kernel<true, 1><<<dim3((a.n_items + 3) / 4, n_kv), 256, 0, stream>>>(a);
+    a.entry_pos0 = entry_pos0; a.dec_params = dec_params; a.p_max = p_max; a.ps_shift = shift_of(page_size);
+    attn_bf16_kernel<true, 1><<<dim3(a.n_items, n_kv), 256, 0, stream>>>(a);
     VT_CHECK_LAUNCH("vt_attn_bf16_decode");
     attn_combine_kernel<true><<<dim3(n_entries, n_kv), 256, 0, stream>>>(nullptr, part_o, part_ml, (bf16_t*)out, n_heads,
                                                                         n_kv, entry_pos0, dec_params, p_max, window, 1);

@@ -209,24 +209,52 @@ __global__ void silu_mul_kernel(const TI* __restrict__ gu, TO* __restrict__ out,
     store_f32<TO>(out + (size_t)t * inter, i, g / (1.f + expf(-g)) * u);
 }
 
-// four values per thread with 8- or 16-byte accesses, for widths that are a multiple of 4
+// Four values per access, four accesses of gate and of up in flight per thread before any is used: the kernel
+// moves 3 values per result and lives on bytes in flight.  For widths that are a multiple of 4.
 template <typename TI, typename TO>
-__global__ void silu_mul_vec_kernel(const TI* __restrict__ gu, TO* __restrict__ out, int inter) {
-    int t = blockIdx.y;
-    int i = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
-    if (i >= inter) return;
-    const TI* row = gu + (size_t)t * 2 * inter;
-    float4 g = load4(row + i), u = load4(row + inter + i);
-    store4(out + (size_t)t * inter + i, make_float4(g.x / (1.f + expf(-g.x)) * u.x, g.y / (1.f + expf(-g.y)) * u.y,
-                                                   g.z / (1.f + expf(-g.z)) * u.z, g.w / (1.f + expf(-g.w)) * u.w));
+__global__ __launch_bounds__(256) void silu_mul_vec_kernel(const TI* __restrict__ gu, TO* __restrict__ out, int inter,
+                                                          int n) {
+    const int qpr = inter >> 2;                                   // quads per row
+    const long long total = (long long)qpr * n;
+    const long long stride = (long long)gridDim.x * 256;
+    for (long long base = (long long)blockIdx.x * 256 + threadIdx.x; base < total; base += 4 * stride) {
+        float4 g[4], u[4];
+        long long idx[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            idx[k] = base + k * stride;
+            if (idx[k] < total) {
+                const long long t = idx[k] / qpr;
+                const int i = (int)(idx[k] - t * qpr) * 4;
+                const TI* row = gu + (size_t)t * 2 * inter;
+                g[k] = load4(row + i);
+                u[k] = load4(row + inter + i);
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            if (idx[k] < total) {
+                const long long t = idx[k] / qpr;
+                const int i = (int)(idx[k] - t * qpr) * 4;
+                store4(out + (size_t)t * inter + i,
+                       make_float4(g[k].x / (1.f + __expf(-g[k].x)) * u[k].x, g[k].y / (1.f + __expf(-g[k].y)) * u[k].y,
+                                   g[k].z / (1.f + __expf(-g[k].z)) * u[k].z, g[k].w / (1.f + __expf(-g[k].w)) * u[k].w));
+            }
+        }
+    }
 }
 
 template <typename TI, typename TO>
 static void launch_silu_mul(const void* gu, void* out, int n, int inter, hipStream_t stream) {
-    if (inter % 4 == 0 && !((uintptr_t)gu & 15) && !((uintptr_t)out & 15))
-        silu_mul_vec_kernel<TI, TO><<<dim3((inter / 4 + 255) / 256, n), 256, 0, stream>>>((const TI*)gu, (TO*)out, inter);
-    else
+    if (inter % 4 == 0 && !((uintptr_t)gu & 15) && !((uintptr_t)out & 15)) {
+        const long long total = (long long)(inter / 4) * n;
+        long long blocks = (total + 1023) / 1024;
+        if (blocks > 8192) blocks = 8192;
+        if (blocks < 1) blocks = 1;
+        silu_mul_vec_kernel<TI, TO><<<(unsigned)blocks, 256, 0, stream>>>((const TI*)gu, (TO*)out, inter, n);
+    } else {
         silu_mul_kernel<TI, TO><<<dim3((inter + 255) / 256, n), 256, 0, stream>>>((const TI*)gu, (TO*)out, inter);
+    }
 }
 
 extern "C" int vt_silu_mul(const void* gu, int in_dtype, void* out, int out_dtype, int n, int inter, hipStream_t stream) {

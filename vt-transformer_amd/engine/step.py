@@ -76,7 +76,7 @@ def plan_tile_items(entry_start: np.ndarray, entry_pos0: np.ndarray, group: int,
     q_len = (entry_start[1:] - entry_start[:-1]).astype(np.int64)[entries]
     rows = q_len * group
     if rt is None:
-        rt = 2 if int(((rows + 127) // 128).sum()) * n_kv >= 512 else 1
+        rt = 1      # measured: 128-row items (rt = 2) halve the number of blocks and lose more than their reuse gains
     rpi = 64 * rt
     n_tiles = (rows + rpi - 1) // rpi
     total = int(n_tiles.sum())
@@ -192,8 +192,8 @@ class StepContext:
         self.entry_start = self.entry_pos0 = self.state_slots = self.logit_rows = None
         self.block_tables: List[torch.Tensor] = []
         self.fresh: List[bool] = []           # per entry: the request's first step (its state slot was just cleared)
-        # set when every entry brings exactly one token (decoding): int32 device array whose [0] is the number of
-        # keys per attention item, and the number of items per entry
+        # set when every entry brings exactly one token (decoding): int32 device array of the number of keys per
+        # attention item, by bucket of the number of kv heads (decode_bucket), and the number of items per entry
         self.decode_params: Optional[torch.Tensor] = None
         self.decode_p_max = 0
         self._plans: Dict[Tuple[int, int, int, int], AttentionPlan] = {}
@@ -230,12 +230,22 @@ class StepContext:
                              d_tiles, t_items.shape[0], tile_rt)
 
 
-def decode_chunk(kv_lens: np.ndarray, p_max: int, target_items: int = 2048, min_chunk: int = 32) -> int:
-    """Keys per attention item of a decoding step: small enough to fill the GPU, large enough that the longest
-    entry needs at most p_max items; a multiple of 16."""
-    total = int(kv_lens.sum())
-    chunk = max(min_chunk, -(-total // target_items), -(-int(kv_lens.max()) // p_max))
-    return -(-chunk // 16) * 16
+DECODE_BUCKETS = 8      # chunk lengths for 1, 2-3, 4-7, ... 128+ key/value heads
+
+
+def decode_bucket(n_kv: int) -> int:
+    return min(DECODE_BUCKETS - 1, max(1, int(n_kv)).bit_length() - 1)
+
+
+def decode_chunk(kv_lens: np.ndarray, p_max: int, n_kv: int = 4, want_blocks: int = 512, min_chunk: int = 64) -> int:
+    """Keys per attention item of a decoding step.  A block of four waves takes one item of one (entry, kv head);
+    with enough entries every entry is one item, otherwise the keys are cut so that about `want_blocks` blocks
+    run, never into more than p_max items; a multiple of 64 (the four waves take 16 keys each in turn)."""
+    pairs = max(1, len(kv_lens) * n_kv)
+    splits = min(p_max, max(1, -(-want_blocks // pairs)))
+    longest = int(kv_lens.max())
+    chunk = max(min_chunk, -(-longest // splits))
+    return -(-chunk // 64) * 64
 
 
 class _DecodeGraph:
@@ -264,7 +274,7 @@ class ModelRunner:
         self.vocab_size = model.spec.vocab_size
         self.steps = 0
         self.tokens = 0
-        self.decode_p_max = max(1, min(64, -(-self.max_seq_len // 64)))
+        self.decode_p_max = max(1, min(16, -(-self.max_seq_len // 64)))   # items one entry's keys are cut into at most
         # Decoding steps of a bfloat16 model are captured once per batch size and replayed, unless a mixer keeps
         # state of its own between steps (the warm-up run before a capture would advance it twice).
         self.decode_graphs = False
@@ -334,9 +344,10 @@ class ModelRunner:
         ctx.h_token_ids, ctx.h_positions, ctx.h_tok_entry = h["ids"], h["positions"], h["tok_entry"]
         ctx.h_entry_start, ctx.h_entry_pos0, ctx.h_state_slots = h["start"], h["pos0"], h["slots"]
         ctx.h_logit_rows, ctx.h_block_tables, ctx.fresh = rows, h["tables"], h["fresh"]
-        dec = np.zeros(4, np.int32)
+        dec = np.zeros(DECODE_BUCKETS, np.int32)
         if decode:
-            dec[0] = decode_chunk(h["kv_lens"], self.decode_p_max)
+            for b in range(DECODE_BUCKETS):
+                dec[b] = decode_chunk(h["kv_lens"], self.decode_p_max, n_kv=1 << b)
         parts = [ctx.h_token_ids, ctx.h_positions, ctx.h_tok_entry, ctx.h_entry_start, ctx.h_entry_pos0,
                  ctx.h_state_slots, ctx.h_logit_rows, dec] + [t.reshape(-1) for t in h["tables"]]
         flat = np.concatenate(parts)
@@ -354,7 +365,7 @@ class ModelRunner:
         ctx.block_tables = [v.view(h["n_entries"], h["max_blocks"]) for v in views[8:]]
 
     def _meta_size(self, h: dict, n_rows: int) -> int:
-        return 3 * h["n"] + (h["n_entries"] + 1) + 2 * h["n_entries"] + n_rows + 4 + \
+        return 3 * h["n"] + (h["n_entries"] + 1) + 2 * h["n_entries"] + n_rows + DECODE_BUCKETS + \
             self.storage.n_groups * h["n_entries"] * h["max_blocks"]
 
     def build_context(self, entries: Sequence[StepEntry]) -> StepContext:

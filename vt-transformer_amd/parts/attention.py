@@ -24,6 +24,11 @@ from .base import MIXERS, POSITIONS, CacheNeed, Part, Runtime, StateNeed, Tensor
 from .linear import linear
 
 
+def decode_bucket(n_kv: int) -> int:
+    """Which of the step's decode chunk lengths is meant for this many key/value heads."""
+    return min(7, max(1, int(n_kv)).bit_length() - 1)
+
+
 @MIXERS.register("attention")
 class PagedAttention(Part):
     def __init__(self, *, rt: Runtime, width: int, prefix: str, num_heads: int, num_kv_heads: int, head_dim: int,
@@ -118,7 +123,8 @@ class PagedAttention(Part):
             # one token per entry: the kernel cuts the keys itself from the positions on the device
             part_o = rt.buffer("attn.dec_part_o", (n * ctx.decode_p_max * nkv * 16 * d,), torch.float32)
             part_ml = rt.buffer("attn.dec_part_ml", (n * ctx.decode_p_max * nkv * 32,), torch.float32)
-            ops.attention_bf16_decode(q, cache.k, cache.v, cache.block_table, ctx.entry_pos0, ctx.decode_params,
+            b = decode_bucket(nkv)
+            ops.attention_bf16_decode(q, cache.k, cache.v, cache.block_table, ctx.entry_pos0, ctx.decode_params[b:b + 1],
                                       ctx.decode_p_max, out, part_o, part_ml, nh, nkv, d, self.window, self.scale)
         else:
             plan = ctx.attention_plan(nh // nkv, self.window, nkv, d)
