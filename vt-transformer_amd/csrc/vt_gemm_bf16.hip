@@ -141,6 +141,152 @@ __global__ __launch_bounds__(WPB * 64) void gemm_skinny_kernel(const bf16_t* __r
     }
 }
 
+// ---------------------------------------------------------------------------
+// 17 to 128 rows (a large decoding batch, a short portion): a block of 4 waves takes 64*R rows of W and 64
+// tokens.  The tokens' values pass through LDS once per block (coalesced loads, two buffers), so they cost a
+// fraction of W's traffic instead of a multiple; each wave streams its own 16*R rows of W from memory into
+// registers one stage ahead.  For matrices with few rows the k range is split over blockIdx.z and the partial
+// sums (fp32, [split][N][M]) are added by vt_sum_partials in split order.
+// ---------------------------------------------------------------------------
+#define MID_BK 64
+#define MID_XROW (MID_BK + 8)
+
+template <int R, bool SWIGLU, typename TO>
+__global__ __launch_bounds__(256) void gemm_mid_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                                                      const float* __restrict__ bias, TO* __restrict__ y,
+                                                      float* __restrict__ partial, int N, int Mout, int K,
+                                                      int k_per_split) {
+    constexpr int NW = SWIGLU ? 2 : 1;
+    constexpr int RW = R * NW;
+    __shared__ __attribute__((aligned(16))) bf16_t xs[2][64][MID_XROW];
+    const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63;
+    const int r = lane & 15, g = lane >> 4;
+    const int m0 = blockIdx.x * (64 * R) + wv * (16 * R), n0 = blockIdx.y * 64;
+    const int k_begin = blockIdx.z * k_per_split, k_end = min(K, k_begin + k_per_split);
+
+    const bf16_t* wrow[RW];
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+        const int mc = min(m0 + 16 * j + r, Mout - 1);
+        wrow[j] = w + (size_t)mc * K;
+        if (SWIGLU) wrow[R + j] = w + ((size_t)Mout + mc) * K;
+    }
+    // this thread's two 16-byte pieces of a stage of x: token p/8, k offset 8*(p%8)
+    const bf16_t* xsrc[2];
+    int xtok[2], xcol[2];
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+        const int pidx = tid + 256 * q;
+        xtok[q] = pidx >> 3;
+        xcol[q] = (pidx & 7) * 8;
+        xsrc[q] = x + (size_t)min(n0 + xtok[q], N - 1) * K + xcol[q];
+    }
+    f32x4_t acc[RW][4];
+#pragma unroll
+    for (int a = 0; a < RW; ++a)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[a][i] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+
+    uint4 xreg[2];
+    bf16x8_t wcur[RW][2], wnxt[RW][2];
+    auto fetch_x = [&](int k0) {
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            Frag f;
+            f.v = load_frag(xsrc[q] + k0, k0 + xcol[q] < k_end);
+            xreg[q] = f.u;
+        }
+    };
+    auto park_x = [&](int buf) {
+#pragma unroll
+        for (int q = 0; q < 2; ++q) *(uint4*)&xs[buf][xtok[q]][xcol[q]] = xreg[q];
+    };
+    auto fetch_w = [&](bf16x8_t (&dst)[RW][2], int k0) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int k = k0 + g * 16 + u * 8;
+#pragma unroll
+            for (int a = 0; a < RW; ++a) dst[a][u] = load_frag(wrow[a] + k, k < k_end);
+        }
+    };
+    auto multiply = [&](const bf16x8_t (&wf)[RW][2], int buf) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                Frag xf;
+                xf.u = *(const uint4*)&xs[buf][i * 16 + r][g * 16 + u * 8];
+#pragma unroll
+                for (int a = 0; a < RW; ++a)
+                    acc[a][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[a][u], xf.v, acc[a][i], 0, 0, 0);
+            }
+    };
+
+    if (k_begin < k_end) {
+        fetch_x(k_begin);
+        fetch_w(wcur, k_begin);
+        park_x(0);
+        __syncthreads();
+        // two stages per turn so that the register buffers alternate without copies
+        for (int k0 = k_begin; k0 < k_end; k0 += 2 * MID_BK) {
+            const int k1 = k0 + MID_BK, k2 = k0 + 2 * MID_BK;
+            if (k1 < k_end) { fetch_x(k1); fetch_w(wnxt, k1); }
+            multiply(wcur, 0);
+            if (k1 < k_end) park_x(1);
+            __syncthreads();
+            if (k1 >= k_end) break;
+            if (k2 < k_end) { fetch_x(k2); fetch_w(wcur, k2); }
+            multiply(wnxt, 1);
+            if (k2 < k_end) park_x(0);
+            __syncthreads();
+        }
+    }
+
+    // acc[a][i][e] is feature m0 + 16 j + 4 g + e (j = a mod R) of token n0 + 16 i + r
+    const bool split = gridDim.z > 1;
+#pragma unroll
+    for (int j = 0; j < R; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int n = n0 + i * 16 + r;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int m = m0 + 16 * j + 4 * g + e;
+                if (m >= Mout || n >= N) continue;
+                float v = acc[j][i][e];
+                if (SWIGLU) {
+                    const float u = acc[R + j][i][e];
+                    v = v / (1.f + expf(-v)) * u;
+                } else if (bias && blockIdx.z == 0) {
+                    v += bias[m];
+                }
+                if (split) partial[((size_t)blockIdx.z * N + n) * Mout + m] = v;
+                else store_f32<TO>(y, (size_t)n * Mout + m, v);
+            }
+        }
+}
+
+// y[i] = sum over splits of partial[s][i], added in split order
+template <typename TO>
+__global__ void sum_partials_kernel(const float* __restrict__ partial, TO* __restrict__ y, size_t n, int splits) {
+    const size_t i = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+    if (i >= n) return;
+    if (i + 4 <= n) {
+        float4 a = *(const float4*)(partial + i);
+        for (int s = 1; s < splits; ++s) {
+            float4 b = *(const float4*)(partial + (size_t)s * n + i);
+            a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+        }
+        store_f32<TO>(y, i, a.x); store_f32<TO>(y, i + 1, a.y); store_f32<TO>(y, i + 2, a.z); store_f32<TO>(y, i + 3, a.w);
+    } else {
+        for (size_t j = i; j < n; ++j) {
+            float a = partial[j];
+            for (int s = 1; s < splits; ++s) a += partial[(size_t)s * n + j];
+            store_f32<TO>(y, j, a);
+        }
+    }
+}
+
 // Any shape (k not a multiple of 8): one thread per output, plain loop.
 template <bool SWIGLU, typename TO>
 __global__ void gemm_plain_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
@@ -181,9 +327,27 @@ static int launch_skinny(int wpb, dim3 grid, const bf16_t* x, const bf16_t* w, c
     return launch_one<NT, R, 16, SWIGLU, TO>(grid, x, w, bias, y, N, Mout, K, stream);
 }
 
+// Number of k ranges for the 64-token kernel: from the shape of W only (so the order of additions does not depend
+// on the batch), enough blocks to fill the GPU, every range a multiple of the stage length.
+static int mid_splits(int Mout, int K, int rows_per_block) {
+    const int row_blocks = (Mout + rows_per_block - 1) / rows_per_block;
+    const int stages = (K + MID_BK - 1) / MID_BK;
+    int splits = (512 + row_blocks - 1) / row_blocks;
+    if (splits > 16) splits = 16;
+    if (splits > stages / 4) splits = stages / 4 > 0 ? stages / 4 : 1;
+    return splits < 1 ? 1 : splits;
+}
+
+extern "C" long long vt_linear_bf16_workspace(int N, int M, int K, int gated) {
+    // floats of workspace that vt_linear_bf16 / vt_gated_linear_bf16 need for this shape (0: none)
+    if (N <= 16 || K % 8 != 0 || gated) return 0;
+    const int splits = mid_splits(M, K, 128);
+    return splits > 1 ? (long long)splits * N * M : 0;
+}
+
 template <bool SWIGLU, typename TO>
-static int linear_bf16(const bf16_t* x, const bf16_t* w, const float* bias, TO* y, int N, int Mout, int K,
-                       hipStream_t stream) {
+static int linear_bf16(const bf16_t* x, const bf16_t* w, const float* bias, TO* y, float* workspace, int N, int Mout,
+                       int K, hipStream_t stream) {
     if (N == 0) return 0;
     if (K % 8 != 0 || ((uintptr_t)x & 15) || ((uintptr_t)w & 15)) {
         VT_REQUIRE(N <= 65535, "vt_linear_bf16: too many rows (%d) for the any-shape kernel", N);
@@ -191,39 +355,41 @@ static int linear_bf16(const bf16_t* x, const bf16_t* w, const float* bias, TO* 
         VT_CHECK_LAUNCH("vt_linear_bf16(plain)");
         return 0;
     }
+    if (N > 16) {
+        // 64 tokens per block through LDS; two row tiles per wave (one for the gated product, which has two
+        // matrices' rows per wave already)
+        constexpr int RR = SWIGLU ? 1 : 2;
+        const int splits = SWIGLU ? 1 : mid_splits(Mout, K, 64 * RR);
+        VT_REQUIRE(splits == 1 || workspace, "vt_linear_bf16: this shape needs a workspace (vt_linear_bf16_workspace)");
+        int kps = ((K + splits - 1) / splits + MID_BK - 1) / MID_BK * MID_BK;
+        dim3 grid((Mout + 64 * RR - 1) / (64 * RR), (N + 63) / 64, splits);
+        VT_REQUIRE(grid.y <= 65535, "vt_linear_bf16: too many rows (%d)", N);
+        gemm_mid_kernel<RR, SWIGLU, TO><<<grid, 256, 0, stream>>>(x, w, bias, y, workspace, N, Mout, K, kps);
+        VT_CHECK_LAUNCH("vt_linear_bf16(64 tokens)");
+        if (splits > 1) {
+            const size_t n = (size_t)N * Mout;
+            sum_partials_kernel<TO><<<(unsigned)((n / 4 + 255) / 256 + 1), 256, 0, stream>>>(workspace, y, n, splits);
+            VT_CHECK_LAUNCH("vt_linear_bf16(sum)");
+        }
+        return 0;
+    }
     // How k is split over the waves of a block depends on the shape of W only, so that a token's sums are added
-    // in the same order whatever the number of rows; the number of row tiles per wave does not change that order.
+    // in the same order whatever the number of rows.
     const int tiles16 = (Mout + 15) / 16;
     const int wpb = tiles16 >= 1024 ? 4 : (tiles16 >= 512 ? 8 : 16);
-    const int nt = N <= 16 ? 1 : (N <= 32 ? 2 : 4);
-    // row tiles per wave: as many as token tiles (x is then read no more often than W), two even for one token
-    // tile when W has rows to spare; bounded by the LDS that the sum over the waves needs
-    const int want = nt == 1 ? (tiles16 >= 2048 ? 2 : 1) : nt;
-    const int cap = 32 / (wpb * (SWIGLU ? 2 : 1));
-    const int rr = want <= cap ? want : (cap >= 2 ? 2 : 1);
-    dim3 grid((Mout + 16 * rr - 1) / (16 * rr), (N + 16 * nt - 1) / (16 * nt));
-    VT_REQUIRE(grid.y <= 65535, "vt_linear_bf16: too many rows (%d)", N);
-    int rc;
-#define VT_GO(NT_, R_) rc = launch_skinny<NT_, R_, SWIGLU, TO>(wpb, grid, x, w, bias, y, N, Mout, K, stream)
-    if (nt == 1 && rr == 1) VT_GO(1, 1);
-    else if (nt == 1) VT_GO(1, 2);
-    else if (nt == 2 && rr == 1) VT_GO(2, 1);
-    else if (nt == 2) VT_GO(2, 2);
-    else if (rr == 1) VT_GO(4, 1);
-    else if (rr == 2) VT_GO(4, 2);
-    else VT_GO(4, 4);
-#undef VT_GO
+    dim3 grid(tiles16, 1);
+    int rc = launch_skinny<1, 1, SWIGLU, TO>(wpb, grid, x, w, bias, y, N, Mout, K, stream);
     if (rc) return rc;
     VT_CHECK_LAUNCH("vt_linear_bf16");
     return 0;
 }
 
 // y[N, M] = x[N, K] . W[M, K]^T + bias
-extern "C" int vt_linear_bf16(const void* x, const void* w, const float* bias, void* y, int out_dtype, int N, int M,
-                              int K, hipStream_t stream) {
+extern "C" int vt_linear_bf16(const void* x, const void* w, const float* bias, void* y, int out_dtype, float* workspace,
+                              int N, int M, int K, hipStream_t stream) {
     VT_REQUIRE(N >= 0 && M > 0 && K > 0, "vt_linear_bf16: bad sizes N=%d M=%d K=%d", N, M, K);
-    if (out_dtype == VT_F32) return linear_bf16<false, float>((const bf16_t*)x, (const bf16_t*)w, bias, (float*)y, N, M, K, stream);
-    if (out_dtype == VT_BF16) return linear_bf16<false, bf16_t>((const bf16_t*)x, (const bf16_t*)w, bias, (bf16_t*)y, N, M, K, stream);
+    if (out_dtype == VT_F32) return linear_bf16<false, float>((const bf16_t*)x, (const bf16_t*)w, bias, (float*)y, workspace, N, M, K, stream);
+    if (out_dtype == VT_BF16) return linear_bf16<false, bf16_t>((const bf16_t*)x, (const bf16_t*)w, bias, (bf16_t*)y, workspace, N, M, K, stream);
     return vt_fail("vt_linear_bf16: unknown out dtype %d", out_dtype);
 }
 
@@ -231,7 +397,7 @@ extern "C" int vt_linear_bf16(const void* x, const void* w, const float* bias, v
 extern "C" int vt_gated_linear_bf16(const void* x, const void* w, void* y, int out_dtype, int N, int I, int K,
                                     hipStream_t stream) {
     VT_REQUIRE(N >= 0 && I > 0 && K > 0, "vt_gated_linear_bf16: bad sizes N=%d I=%d K=%d", N, I, K);
-    if (out_dtype == VT_F32) return linear_bf16<true, float>((const bf16_t*)x, (const bf16_t*)w, nullptr, (float*)y, N, I, K, stream);
-    if (out_dtype == VT_BF16) return linear_bf16<true, bf16_t>((const bf16_t*)x, (const bf16_t*)w, nullptr, (bf16_t*)y, N, I, K, stream);
+    if (out_dtype == VT_F32) return linear_bf16<true, float>((const bf16_t*)x, (const bf16_t*)w, nullptr, (float*)y, nullptr, N, I, K, stream);
+    if (out_dtype == VT_BF16) return linear_bf16<true, bf16_t>((const bf16_t*)x, (const bf16_t*)w, nullptr, (bf16_t*)y, nullptr, N, I, K, stream);
     return vt_fail("vt_gated_linear_bf16: unknown out dtype %d", out_dtype);
 }

@@ -175,8 +175,17 @@ def linear_f32(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], o
     return out
 
 
-def linear_bf16(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor) -> torch.Tensor:
-    """Few rows (decoding, short portions): W is read once per 64 rows."""
+def linear_bf16_workspace(n: int, m: int, k: int) -> int:
+    """Floats of scratch memory that linear_bf16 needs for x [n, k], W [m, k] (0: none)."""
+    lib = load_lib("vt_gemm_bf16")
+    lib.vt_linear_bf16_workspace.restype = ctypes.c_longlong
+    return int(lib.vt_linear_bf16_workspace(_i(n), _i(m), _i(k), _i(0)))
+
+
+def linear_bf16(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
+                workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Few rows (decoding, short portions): W is read once per 64 rows.  Shapes whose k range is split over blocks
+    need `workspace` (float32, at least linear_bf16_workspace(n, m, k) elements)."""
     n, k = x.shape
     m = w.shape[0]
     _chk(x, "linear_bf16.x", torch.bfloat16)
@@ -184,8 +193,15 @@ def linear_bf16(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], 
     _chk(out, "linear_bf16.out", None, (n, m))
     if bias is not None:
         _chk(bias, "linear_bf16.bias", torch.float32, (m,))
-    _run(load_lib("vt_gemm_bf16"), "vt_linear_bf16", _ptr(x), _ptr(w), _ptr(bias), _ptr(out), _i(_code(out)), _i(n), _i(m),
-         _i(k), _stream())
+    need = linear_bf16_workspace(n, m, k) if n > 16 else 0
+    if need:
+        if workspace is None:
+            raise KernelError(f"linear_bf16: x [{n}, {k}] with W [{m}, {k}] needs a workspace of {need} floats")
+        _chk(workspace, "linear_bf16.workspace", torch.float32)
+        if workspace.numel() < need:
+            raise KernelError(f"linear_bf16: workspace of {workspace.numel()} floats, need {need}")
+    _run(load_lib("vt_gemm_bf16"), "vt_linear_bf16", _ptr(x), _ptr(w), _ptr(bias), _ptr(out), _i(_code(out)),
+         _ptr(workspace if need else None), _i(n), _i(m), _i(k), _stream())
     return out
 
 

@@ -62,5 +62,7 @@ class LinearHead(Part):
             return ops.linear_f32(x, self.weight, None, out)
         for r0 in range(0, r, SKINNY_MAX_ROWS):
             r1 = min(r, r0 + SKINNY_MAX_ROWS)
-            ops.linear_bf16(x[r0:r1], self.weight, None, out[r0:r1])
+            need = ops.linear_bf16_workspace(r1 - r0, self.vocab, self.width) if r1 - r0 > 16 else 0
+            work = self.rt.buffer("linear.partials", (need,), torch.float32) if need else None
+            ops.linear_bf16(x[r0:r1], self.weight, None, out[r0:r1], work)
         return out

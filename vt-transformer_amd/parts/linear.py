@@ -32,7 +32,9 @@ def linear(rt: Runtime, x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.T
         return ops.linear_f32(x, w, bias, out)
     if n <= SKINNY_MAX_ROWS:
         out = rt.buffer(name, (n, m), out_dtype or torch.float32)
-        return ops.linear_bf16(x, w, bias, out)
+        need = ops.linear_bf16_workspace(n, m, k) if n > 16 else 0
+        work = rt.buffer("linear.partials", (need,), torch.float32) if need else None
+        return ops.linear_bf16(x, w, bias, out, work)
     out = rt.buffer(name + ".lib", (n, m), torch.bfloat16)
     if bias is not None:
         if bias_lowp is None:
