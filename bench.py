@@ -39,6 +39,7 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--no-graphs", action="store_true")
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill measurement (profiling runs)")
+    ap.add_argument("--no-tune", action="store_true", help="do not let the GEMM library search its algorithms at start-up")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this engine runs on one GPU; N > 1 is not measured")
@@ -63,6 +64,9 @@ def main() -> int:
                  decode_graphs=not args.no_graphs)
     torch.cuda.synchronize()
     print(f"[bench] model ready in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
+    if not args.no_tune and not args.no_prefill:
+        print(f"[bench] GEMM library algorithm search at {args.prefill_tokens} rows: "
+              f"{eng.tune_library_products(args.prefill_tokens):.1f} s", file=sys.stderr, flush=True)
     rs = np.random.RandomState(0)
 
     def decode_run(batch: int, steps: int, warmup: int):
@@ -138,7 +142,7 @@ def main() -> int:
                    "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
                    "intermediate": I, "vocab": V, "global_batch": args.batch, "seq_len": args.prompt_len,
                    "prompt_len": args.prompt_len, "context_len": ctx_len, "kv_block": 16, "rope_theta": cfg.rope_theta,
-                   "parallelism": "1 GPU", "decode_graphs": not args.no_graphs},
+                   "parallelism": "1 GPU", "decode_graphs": not args.no_graphs, "gemm_tuning": not args.no_tune},
         "prefill": {"value": round(T / p_dt, 1), "tokens": T, "ms": round(p_dt * 1e3, 3),
                     "frac": round(p_flops / p_dt / PEAK_FLOPS["bf16"], 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBPS, "unit": "GB/s",

@@ -274,3 +274,17 @@ def test_decode_graph_replays_match_eager(model_folders):
     b = graph.step(e3).clone()
     assert torch.equal(a, b)
     assert len(graph._graphs) >= 1
+
+
+def test_library_algorithm_search_keeps_results(model_folders):
+    """With the GEMM library's algorithm search on, a long portion gives the same logits to rounding."""
+    from vt_transformer_amd.engine import Engine, StepEntry
+    toks = random_requests(TINY["B"]["vocab_size"], [150], seed=30)["r0"]
+    logits = []
+    for tune in (False, True):
+        eng = Engine(model_folders["B"], dtype="bfloat16", num_pages=32, max_running_reqs=2, max_seq_len=256,
+                     chunk_size=128, tune_gemm=tune)
+        eng.runner.admit("x")
+        logits.append(eng.runner.step([StepEntry("x", toks, [149])]).float().cpu())
+        assert sum(eng.runner.cache.held_pages()) == 10
+    assert float((logits[0] - logits[1]).abs().max() / logits[0].abs().max()) < 2e-2

@@ -148,8 +148,12 @@ __global__ __launch_bounds__(WPB * 64) void gemm_skinny_kernel(const bf16_t* __r
 // registers one stage ahead.  For matrices with few rows the k range is split over blockIdx.z and the partial
 // sums (fp32, [split][N][M]) are added by vt_sum_partials in split order.
 // ---------------------------------------------------------------------------
-#define MID_BK 64
+#ifndef MID_BK
+#define MID_BK 128                 // k values per stage (a multiple of 64)
+#endif
 #define MID_XROW (MID_BK + 8)
+#define MID_KU (MID_BK / 32)       // matrix instructions along k per stage
+#define MID_XP (MID_BK / 32)       // 16-byte pieces of x per thread and stage (64 tokens * MID_BK / 8 / 256)
 
 template <int R, bool SWIGLU, typename TO>
 __global__ __launch_bounds__(256) void gemm_mid_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
@@ -171,14 +175,14 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const bf16_t* __restrict_
         wrow[j] = w + (size_t)mc * K;
         if (SWIGLU) wrow[R + j] = w + ((size_t)Mout + mc) * K;
     }
-    // this thread's two 16-byte pieces of a stage of x: token p/8, k offset 8*(p%8)
-    const bf16_t* xsrc[2];
-    int xtok[2], xcol[2];
+    // this thread's 16-byte pieces of a stage of x: a token's MID_BK values are MID_BK/8 consecutive pieces
+    const bf16_t* xsrc[MID_XP];
+    int xtok[MID_XP], xcol[MID_XP];
 #pragma unroll
-    for (int q = 0; q < 2; ++q) {
+    for (int q = 0; q < MID_XP; ++q) {
         const int pidx = tid + 256 * q;
-        xtok[q] = pidx >> 3;
-        xcol[q] = (pidx & 7) * 8;
+        xtok[q] = pidx / (MID_BK / 8);
+        xcol[q] = (pidx % (MID_BK / 8)) * 8;
         xsrc[q] = x + (size_t)min(n0 + xtok[q], N - 1) * K + xcol[q];
     }
     f32x4_t acc[RW][4];
@@ -187,11 +191,11 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const bf16_t* __restrict_
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc[a][i] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 
-    uint4 xreg[2];
-    bf16x8_t wcur[RW][2], wnxt[RW][2];
+    uint4 xreg[MID_XP];
+    bf16x8_t wcur[RW][MID_KU], wnxt[RW][MID_KU];
     auto fetch_x = [&](int k0) {
 #pragma unroll
-        for (int q = 0; q < 2; ++q) {
+        for (int q = 0; q < MID_XP; ++q) {
             Frag f;
             f.v = load_frag(xsrc[q] + k0, k0 + xcol[q] < k_end);
             xreg[q] = f.u;
@@ -199,23 +203,24 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const bf16_t* __restrict_
     };
     auto park_x = [&](int buf) {
 #pragma unroll
-        for (int q = 0; q < 2; ++q) *(uint4*)&xs[buf][xtok[q]][xcol[q]] = xreg[q];
+        for (int q = 0; q < MID_XP; ++q) *(uint4*)&xs[buf][xtok[q]][xcol[q]] = xreg[q];
     };
-    auto fetch_w = [&](bf16x8_t (&dst)[RW][2], int k0) {
+    // fragment u of a stage: k = k0 + 64 (u/2) + 16 g + 8 (u%2), so a lane reads 32 contiguous bytes per 64 k
+    auto fetch_w = [&](bf16x8_t (&dst)[RW][MID_KU], int k0) {
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
-            const int k = k0 + g * 16 + u * 8;
+        for (int u = 0; u < MID_KU; ++u) {
+            const int k = k0 + (u >> 1) * 64 + g * 16 + (u & 1) * 8;
 #pragma unroll
             for (int a = 0; a < RW; ++a) dst[a][u] = load_frag(wrow[a] + k, k < k_end);
         }
     };
-    auto multiply = [&](const bf16x8_t (&wf)[RW][2], int buf) {
+    auto multiply = [&](const bf16x8_t (&wf)[RW][MID_KU], int buf) {
 #pragma unroll
-        for (int u = 0; u < 2; ++u)
+        for (int u = 0; u < MID_KU; ++u)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 Frag xf;
-                xf.u = *(const uint4*)&xs[buf][i * 16 + r][g * 16 + u * 8];
+                xf.u = *(const uint4*)&xs[buf][i * 16 + r][(u >> 1) * 64 + g * 16 + (u & 1) * 8];
 #pragma unroll
                 for (int a = 0; a < RW; ++a)
                     acc[a][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[a][u], xf.v, acc[a][i], 0, 0, 0);

@@ -9,6 +9,7 @@ sglfront tokenises and the engine sees ids only.
 """
 from __future__ import annotations
 
+import os
 import time
 from typing import Dict, Hashable, Iterable, List, Optional, Sequence, Union
 
@@ -24,10 +25,13 @@ from .step import ModelRunner, StepEntry
 class Engine:
     def __init__(self, model: Optional[str] = None, *, config: Optional[ModelConfig] = None,
                  random_weights_seed: Optional[int] = None, dtype: str = "bfloat16", seed: int = 0,
-                 scheduler_config: Optional[SchedulerConfig] = None, decode_graphs: bool = True, **options):
+                 scheduler_config: Optional[SchedulerConfig] = None, decode_graphs: bool = True,
+                 tune_gemm: bool = False, **options):
         """model: a folder with config.json and model.safetensors.  Or `config` with `random_weights_seed`
         for random weights drawn on the device.  `options` override fields of SchedulerConfig
-        (max_running_reqs, num_pages, max_seq_len, page_size, max_extend_tokens, default_max_output, chunk_size)."""
+        (max_running_reqs, num_pages, max_seq_len, page_size, max_extend_tokens, default_max_output, chunk_size).
+        tune_gemm: let the GEMM library try its algorithms on this model's products at chunk_size rows once, at
+        start-up (some seconds), and use the fastest from then on."""
         sc = scheduler_config or SchedulerConfig()
         for k, v in options.items():
             if not hasattr(sc, k):
@@ -51,6 +55,36 @@ class Engine:
         self.seed = int(seed)
         self._next_uid = 0
         self.requests: Dict[Hashable, Request] = {}
+        if tune_gemm:
+            self.tune_library_products()
+
+    def tune_library_products(self, rows: Optional[int] = None) -> float:
+        """Long portions multiply through the GEMM library (parts/linear.py).  This runs one portion of `rows`
+        tokens (default: chunk_size) with the library's algorithm search switched on, so that every product of
+        the model is tried at that size; afterwards the search is off again and other sizes take the library's
+        default.  What it finds is kept in a file beside the compiled kernels, so a later start is quick.
+        Returns the seconds it took."""
+        import torch.cuda.tunable as tunable
+        sc = self.config
+        n = rows or sc.chunk_size
+        n = max(65, min(n, sc.max_seq_len - 1, self.runner.cache.available_tokens()))
+        t0 = time.time()
+        tunable.enable(True)
+        # the library reads earlier results from this file and rewrites it when the process ends
+        from ..kernels.build import _build_dir
+        tunable.set_filename(os.path.join(_build_dir(), "gemm_algorithms.csv"))
+        tunable.tuning_enable(True)
+        try:
+            rid = ("tune", id(self))
+            self.runner.admit(rid)
+            try:
+                self.runner.step([StepEntry(rid, [0] * n, [n - 1])])
+                torch.cuda.synchronize()
+            finally:
+                self.runner.release(rid)
+        finally:
+            tunable.tuning_enable(False)
+        return time.time() - t0
 
     # -- requests ------------------------------------------------------------
     def add_request(self, prompt: Sequence[int], params: Optional[SamplingParams] = None,
