@@ -76,6 +76,20 @@ __device__ __forceinline__ unsigned pack2(float a, float b) {
     return __builtin_bit_cast(unsigned, __builtin_convertvector(v, bf16x2_t));
 }
 
+// Maximum over the four lanes that share a row (lane % 16): two register swaps between rows of 16 and halves of 32
+// lanes, which stay in the vector unit (a shuffle would go through the LDS crossbar).
+typedef __attribute__((ext_vector_type(2))) unsigned u32x2_t;
+typedef __attribute__((ext_vector_type(4))) unsigned u32x4_t;
+__device__ __forceinline__ float row_max4(float v) {
+    const unsigned u = __float_as_uint(v);
+    const u32x2_t a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    const unsigned a0 = a.x, a1 = a.y;     // copies: a bit cast of a vector element reads the wrong one
+    const unsigned x = __float_as_uint(fmaxf(__uint_as_float(a0), __uint_as_float(a1)));
+    const u32x2_t b = __builtin_amdgcn_permlane32_swap(x, x, false, false);
+    const unsigned b0 = b.x, b1 = b.y;
+    return fmaxf(__uint_as_float(b0), __uint_as_float(b1));
+}
+
 // One step of the running softmax of a row over NK*4 scores held by this lane (s[kt][i] = raw dot product of key
 // j0 + 16 kt + 4 g + i), shared with the three other lanes of the row.  `full`: every key of the block is visible
 // to every row of the tile, so no score is tested.  Leaves the probabilities as bf16 pairs in pk, the factor for
@@ -98,9 +112,7 @@ __device__ __forceinline__ void softmax_step(const f32x4_t (&s)[NK], int j0, int
                 if (j <= p && j >= p_lo) mb = fmaxf(mb, s[kt][i]);
             }
     }
-    mb *= scale_log2;
-    mb = fmaxf(mb, __shfl_xor(mb, 16, 64));
-    mb = fmaxf(mb, __shfl_xor(mb, 32, 64));
+    mb = row_max4(mb * scale_log2);
     const float m_new = fmaxf(m, mb);
     alpha = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m - m_new);
     float pv[NK][4], psum = 0.f;
@@ -157,7 +169,7 @@ __device__ __forceinline__ void load_block(KVBlock& b, const AttnArgs& a, int pg
 
 // RT row tiles of 16 rows per wave share every key/value block they read.
 template <bool DECODE, int RT>
-__global__ __launch_bounds__(256) void attn_bf16_kernel(AttnArgs a) {
+__global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_kernel(AttnArgs a) {
     const int wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
     // decoding: the four waves of a block share one item and take its key blocks in turn; otherwise one item per wave
     const int item = DECODE ? (int)blockIdx.x : (int)blockIdx.x * 4 + wv;
@@ -366,26 +378,96 @@ __global__ __launch_bounds__(256) void attn_bf16_kernel(AttnArgs a) {
 // ---------------------------------------------------------------------------
 // Long portions of prompts: a block of 4 waves takes 64 * RT consecutive rows of one (entry, kv head) and walks
 // their keys KB at a time.  Every key/value block is fetched from the pages once per block of waves, by all 256
-// threads together with 16-byte loads, and parked in LDS (two buffers: the next block is on its way from memory
-// while this one is multiplied); the four waves read their matrix operands from there.  Rows of an item that lie
-// wholly above a key block skip it (the upper triangle of a causal portion costs nothing).
+// threads together with 16-byte loads, and parked in LDS (two buffers: the next block comes from memory into
+// registers while this one is multiplied, and is parked in the other buffer afterwards); the four waves read their
+// matrix operands from there, each operand once for all RT row tiles of the wave.  Rows of an item that lie wholly
+// above a key block skip it (the upper triangle of a causal portion costs nothing).
+//
+// A block of keys is KH halves of 32.  The 32 LDS rows of a half hold its key 8q + 4t + i at row 16t + 4q + i
+// (t = 0, 1: the half's two score tiles), so that the eight scores a lane holds after the first product (four
+// each from the two tiles) are eight consecutive keys 8g..8g+7: exactly the k slots of its B operand in the
+// 16x16x32 product with the values, whose A operand is then one 16-byte read of the value rows in their natural
+// key order.  The row sums of the probabilities come out of the matrix cores too: one more product per half
+// against a tile of ones, which leaves every lane with the sum of its row.
 // ---------------------------------------------------------------------------
-constexpr int KB = (D > 128) ? 16 : 32;        // keys per block
+constexpr int KB = (D > 128) ? 32 : 64;        // keys per block
+constexpr int KH = KB / 32;                    // halves of 32 keys
 constexpr int KT = KB / 16;                    // score tiles per block
 constexpr int KROW = D + 8;                    // padded rows: operand reads from LDS without bank conflicts
 constexpr int VROW = KB + 8;
-constexpr int KPIECES = KB * (D / 8);          // 16-byte pieces of a key block
-constexpr int VPIECES = D * (KB / 8);
-constexpr int KPT = (KPIECES + 255) / 256;     // pieces per thread
-constexpr int VPT = (VPIECES + 255) / 256;
-constexpr int PAGE_WINDOW = 256;               // page ids kept in LDS at a time
+constexpr int GP = 2 * D;                      // 16-byte pieces of 16 keys (and of their values)
+constexpr int NP = (GP + 255) / 256;           // pieces per thread and group of 16 keys
+constexpr int TILE_LDS_BYTES = 2 * (KB * KROW + D * VROW) * (int)sizeof(bf16_t);
+
+// key (relative to the block's first) of score tile kt, lane group g, register i
+__device__ __forceinline__ int tile_key(int kt, int g, int i) { return 32 * (kt >> 1) + 8 * g + 4 * (kt & 1) + i; }
+
+// Maximum of three floats in one instruction.  (fmaxf first makes each operand canonical, an instruction per
+// operand, because a signalling NaN must become quiet; there is none here.)
+__device__ __forceinline__ float max3(float x, float y, float z) {
+    float d;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(d) : "v"(x), "v"(y), "v"(z));
+    return d;
+}
+__device__ __forceinline__ float max2(float x, float y) {
+    float d;
+    asm("v_max_f32 %0, %1, %2" : "=v"(d) : "v"(x), "v"(y));
+    return d;
+}
+__device__ __forceinline__ float row_max4_lean(float v) {
+    const unsigned u = __float_as_uint(v);
+    const u32x2_t a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    const unsigned a0 = a.x, a1 = a.y;
+    const unsigned x = __float_as_uint(max2(__uint_as_float(a0), __uint_as_float(a1)));
+    const u32x2_t b = __builtin_amdgcn_permlane32_swap(x, x, false, false);
+    const unsigned b0 = b.x, b1 = b.y;
+    return max2(__uint_as_float(b0), __uint_as_float(b1));
+}
+
+// softmax_step for the tiled kernel: the same arithmetic, the key order above, no row sum (the matrix cores add
+// it).  FULL: every key of the block is visible to every row of the tile, nothing is tested.
+template <bool FULL>
+__device__ __forceinline__ void tile_softmax(const f32x4_t (&s)[KT], int j0, int g, int p, int p_lo,
+                                             float scale_log2, float& m, float& alpha, unsigned (&pk)[KT * 2]) {
+    bool ok[KT][4];
+    float v[KT][4];
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int j = j0 + tile_key(kt, g, i);
+            ok[kt][i] = FULL || (j <= p && j >= p_lo);
+            v[kt][i] = ok[kt][i] ? s[kt][i] : -INFINITY;
+        }
+    float mb = max2(max3(v[0][0], v[0][1], v[0][2]), v[0][3]);
+#pragma unroll
+    for (int kt = 1; kt < KT; ++kt) mb = max3(max3(mb, v[kt][0], v[kt][1]), v[kt][2], v[kt][3]);
+    mb = row_max4_lean(mb * scale_log2);
+    const float m_new = max2(m, mb);
+    alpha = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m - m_new);
+    m = m_new;
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) {
+        float pv[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float e = __builtin_amdgcn_exp2f(fmaf(s[kt][i], scale_log2, -m_new));
+            pv[i] = (FULL || ok[kt][i]) ? e : 0.f;      // a visible key makes m_new finite
+        }
+        pk[2 * kt] = pack2(pv[0], pv[1]);
+        pk[2 * kt + 1] = pack2(pv[2], pv[3]);
+    }
+}
 
 template <int RT>
-__global__ __launch_bounds__(256) void attn_bf16_tile_kernel(AttnArgs a) {
-    __shared__ __attribute__((aligned(16))) bf16_t k_lds[2][KB][KROW];
-    __shared__ __attribute__((aligned(16))) bf16_t v_lds[2][D][VROW];
-    __shared__ int s_pages[PAGE_WINDOW];
-    const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63;
+__global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_tile_kernel(AttnArgs a) {
+    extern __shared__ __attribute__((aligned(16))) bf16_t tile_lds[];
+    bf16_t* const k_lds = tile_lds;                       // [2][KB][KROW]
+    bf16_t* const v_lds = tile_lds + 2 * KB * KROW;       // [2][D][VROW]
+    const int tid = threadIdx.x, lane = tid & 63;
+    // the wave's index as a scalar: what depends only on it (which keys the wave's tiles see) then stays in scalar
+    // registers and its tests are scalar branches
+    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int* it = a.items + (size_t)blockIdx.x * ITEM_INTS;
     const int entry = it[0], q_tok0 = it[1], q_len = it[2], pos0 = it[3], q_row0 = it[4];
     const int key_lo = it[5], key_hi = it[6];
@@ -397,11 +479,12 @@ __global__ __launch_bounds__(256) void attn_bf16_tile_kernel(AttnArgs a) {
     const int ps = a.page_size;
 
     bool row_ok[RT];
-    int ti[RT], head[RT], p[RT], p_lo[RT], tile_hi[RT], tile_lo[RT], tile_first_p[RT], tile_last_lo[RT];
+    int ti[RT], head[RT], p[RT], p_lo[RT], tile_first_p[RT], tile_last_lo[RT];
     bf16x8_t q8[RT][WIDE ? QSTEPS : 1];
     bf16x4_t q4[RT][WIDE ? 1 : QSTEPS];
-    f32x4_t o[RT][DT];
-    float m[RT], l[RT];
+    f32x4_t o[RT][DT], ol[RT];     // ol: the row sums, the same value in all four registers
+    float m[RT];
+    int wave_hi = -1, wave_lo = 0x7fffffff;   // keys that any row of the wave may see
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
         const int row0 = q_row0 + (wv * RT + rt) * 16;
@@ -413,10 +496,13 @@ __global__ __launch_bounds__(256) void attn_bf16_tile_kernel(AttnArgs a) {
         p[rt] = pos0 + ti[rt];
         p_lo[rt] = a.window > 0 ? p[rt] - a.window + 1 : 0;
         const int last_row = min(n_rows - 1, row0 + 15), first_row = min(n_rows - 1, row0);
-        tile_hi[rt] = (row0 < n_rows) ? pos0 + last_row / G : -1;
-        tile_lo[rt] = a.window > 0 ? pos0 + first_row / G - a.window + 1 : 0;
+        // a block whose keys lie between these two is visible to every row of the tile
         tile_first_p[rt] = pos0 + first_row / G;
         tile_last_lo[rt] = a.window > 0 ? pos0 + last_row / G - a.window + 1 : 0;
+        if (row0 < n_rows) {
+            wave_hi = max(wave_hi, pos0 + last_row / G);
+            wave_lo = min(wave_lo, a.window > 0 ? pos0 + first_row / G - a.window + 1 : 0);
+        }
         const bf16_t* qrow = a.q + ((size_t)(q_tok0 + ti[rt]) * a.n_heads + head[rt]) * D;
         if constexpr (WIDE) {
 #pragma unroll
@@ -427,158 +513,172 @@ __global__ __launch_bounds__(256) void attn_bf16_tile_kernel(AttnArgs a) {
         }
 #pragma unroll
         for (int t = 0; t < DT; ++t) o[rt][t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+        ol[rt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
         m[rt] = -INFINITY;
-        l[rt] = 0.f;
     }
 
+    // This thread's pieces of a group of 16 keys: piece x of the keys is (key x / (D/8), dims 8 (x % (D/8))..),
+    // piece x of the values is (dim x / 2, keys 8 (x % 2)..).  Byte offsets from the group's first element in the
+    // pages, element offsets in an LDS buffer; fixed for the whole walk.
+    unsigned k_src[NP], v_src[NP];
+    int k_dst[KT][NP], v_dst[NP];
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+        const int x = tid + 256 * i;
+        const int key = x / (D / 8), c = x - key * (D / 8);
+        k_src[i] = 2u * (unsigned)(key * D + c * 8);
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) {
+            const int jb = 16 * (kt & 1) + key;      // key within its half -> its LDS row
+            const int row = 32 * (kt >> 1) + ((jb & 7) >> 2) * 16 + 4 * (jb >> 3) + (jb & 3);
+            k_dst[kt][i] = row * KROW + c * 8;
+        }
+        const int d = x >> 1, h = x & 1;
+        v_src[i] = 2u * (unsigned)(d * ps + 8 * h);
+        v_dst[i] = d * VROW + 8 * h;
+    }
+
+    // The next fetch starts at offset f_off of the entry's page f_blk.  The page ids of that block's groups of 16
+    // keys are read from the block table a step ahead; all of it is the same in every thread and lives in scalar
+    // registers.  A group without a page (beyond the entry's keys, or passed by a window: every row masks its
+    // keys) reads the entry's last page instead, whose contents are as harmless as the unused slots of any page.
     const int* bt = a.block_table + (size_t)entry * a.max_blocks;
     const int last_page = (key_hi - 1) / ps;
-    int page_base = key_lo / ps;
-    auto fill_pages = [&]() {   // all threads; callers put barriers around it
-        const int pgi = page_base + tid;
-        if (tid < PAGE_WINDOW) s_pages[tid] = (pgi <= last_page) ? bt[pgi] : -1;
-    };
-    struct Stage { uint4 k[KPT]; uint4 v[VPT]; };
-    auto fetch = [&](Stage& st_, int j0) {   // this thread's pieces of keys [j0, j0 + KB) from the pages into registers
+    const int pg_spare = min(max(bt[last_page], 0), a.num_pages - 1);
+    int f_blk = key_lo / ps, f_off = key_lo - f_blk * ps;
+    int pgn[KT];
+    auto next_pages = [&]() __attribute__((always_inline)) {
+        int blk = f_blk, off = f_off;
 #pragma unroll
-        for (int i = 0; i < KPT; ++i) {
-            const int idx = tid + 256 * i;
-            st_.k[i] = make_uint4(0, 0, 0, 0);
-            if (idx < KPIECES) {
-                const int key = idx / (D / 8), c = idx - key * (D / 8);
-                const int j = j0 + key;
-                const int blk = page_index(a, j);
-                const int pg = (j < key_hi) ? s_pages[blk - page_base] : -1;
-                if (pg >= 0 && pg < a.num_pages)
-                    st_.k[i] = *(const uint4*)(a.k_pages + (((size_t)pg * a.n_kv + kvh) * ps + (j - blk * ps)) * D + c * 8);
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < VPT; ++i) {
-            const int idx = tid + 256 * i;
-            st_.v[i] = make_uint4(0, 0, 0, 0);
-            if (idx < VPIECES) {
-                const int d = idx / (KB / 8), kg = idx - d * (KB / 8);
-                const int j = j0 + kg * 8;
-                const int blk = page_index(a, j);
-                const int pg = (j < key_hi) ? s_pages[blk - page_base] : -1;
-                if (pg >= 0 && pg < a.num_pages)
-                    st_.v[i] = *(const uint4*)(a.v_pages + (((size_t)pg * a.n_kv + kvh) * D + d) * ps + (j - blk * ps));
-            }
+        for (int kt = 0; kt < KT; ++kt) {
+            pgn[kt] = bt[min(blk, last_page)];
+            off += 16;
+            const bool wrap = off == ps;
+            off = wrap ? 0 : off;
+            blk += wrap ? 1 : 0;
         }
     };
-    auto park = [&](const Stage& st_, int buf) {
+    const unsigned page_bytes = (unsigned)(a.n_kv * ps * D) * 2u;     // bytes per page, keys or values
+    const char* const k_base = (const char*)(a.k_pages + (size_t)kvh * ps * D);
+    const char* const v_base = (const char*)(a.v_pages + (size_t)kvh * ps * D);
+    // (a native vector type: copies of HIP's uint4 struct become memcpy calls that keep the stage in scratch memory)
+    u32x4_t st_k[KT][NP], st_v[KT][NP];
+    auto fetch = [&]() __attribute__((always_inline)) {   // this thread's pieces of the next KB keys, pages -> registers
 #pragma unroll
-        for (int i = 0; i < KPT; ++i) {
-            const int idx = tid + 256 * i;
-            if (idx < KPIECES) {
-                const int key = idx / (D / 8), c = idx - key * (D / 8);
-                *(uint4*)&k_lds[buf][key][c * 8] = st_.k[i];
-            }
-        }
+        for (int kt = 0; kt < KT; ++kt) {
+            const int pg = (pgn[kt] >= 0 && pgn[kt] < a.num_pages) ? pgn[kt] : pg_spare;
+            const size_t pg_off = (size_t)pg * page_bytes;
+            const char* kb = k_base + (pg_off + (unsigned)(f_off * (2 * D)));
+            const char* vb = v_base + (pg_off + (unsigned)(f_off * 2));
 #pragma unroll
-        for (int i = 0; i < VPT; ++i) {
-            const int idx = tid + 256 * i;
-            if (idx < VPIECES) {
-                const int d = idx / (KB / 8), kg = idx - d * (KB / 8);
-                *(uint4*)&v_lds[buf][d][kg * 8] = st_.v[i];
-            }
-        }
-    };
-
-    // one key block (in LDS buffer `buf`, keys from j0) against the RT row tiles of this wave
-    auto multiply = [&](int buf, int j0) {
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt) {
-            if (j0 > tile_hi[rt] || j0 + KB - 1 < tile_lo[rt]) continue;   // every key masked for every row of the tile
-            f32x4_t s[KT];
-#pragma unroll
-            for (int kt = 0; kt < KT; ++kt) {
-                s[kt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
-                const bf16_t* kr = &k_lds[buf][kt * 16 + r][0];
-                if constexpr (WIDE) {
-#pragma unroll
-                    for (int st = 0; st < QSTEPS; ++st) {
-                        U16 t; t.u = *(const uint4*)(kr + st * 32 + g * 8);
-                        s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(t.v, q8[rt][st], s[kt], 0, 0, 0);
-                    }
-                } else {
-#pragma unroll
-                    for (int st = 0; st < QSTEPS; ++st) {
-                        U8 t; t.u = *(const uint2*)(kr + st * 16 + g * 4);
-                        s[kt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(t.v, q4[rt][st], s[kt], 0, 0, 0);
-                    }
+            for (int i = 0; i < NP; ++i) {
+                if (GP % 256 == 0 || tid + 256 * i < GP) {
+                    st_k[kt][i] = *(const u32x4_t*)(kb + k_src[i]);
+                    st_v[kt][i] = *(const u32x4_t*)(vb + v_src[i]);
                 }
             }
-            // s[kt][i] is key j0 + 16 kt + 4 g + i against row r of the tile
-            const bool full = (j0 + KB - 1 <= tile_first_p[rt]) && (j0 >= tile_last_lo[rt]);
-            float alpha;
-            unsigned pk[KT * 2];
-            softmax_step<KT>(s, j0, g, p[rt], p_lo[rt], full, a.scale_log2, m[rt], l[rt], alpha, pk);
-            const bool rescale = __any(alpha != 1.f);      // the maximum of some row moved
-            if constexpr (KT == 2) {
-                // one 16x16x32 instruction per 16 dims: its 8 k slots of lane group g are keys 4g..4g+3 of the
-                // first score tile and of the second
-                U16 pf;
-                pf.u = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+            f_off += 16;
+            const bool wrap = f_off == ps;
+            f_off = wrap ? 0 : f_off;
+            f_blk += wrap ? 1 : 0;
+        }
+        next_pages();
+    };
+    auto park = [&](int buf) __attribute__((always_inline)) {
+        bf16_t* const kd = k_lds + buf * (KB * KROW);
+        bf16_t* const vd = v_lds + buf * (D * VROW);
 #pragma unroll
-                for (int t = 0; t < DT; ++t) {
-                    const bf16_t* vr = &v_lds[buf][t * 16 + r][4 * g];
-                    U16 vf;
-                    uint2 lo = *(const uint2*)vr, hi = *(const uint2*)(vr + 16);
-                    vf.u = make_uint4(lo.x, lo.y, hi.x, hi.y);
-                    if (rescale) o[rt][t] *= alpha;
-                    o[rt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf.v, o[rt][t], 0, 0, 0);
+        for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+            for (int i = 0; i < NP; ++i)
+                if (GP % 256 == 0 || tid + 256 * i < GP) {
+                    *(u32x4_t*)(kd + k_dst[kt][i]) = st_k[kt][i];
+                    *(u32x4_t*)(vd + v_dst[i] + 16 * kt) = st_v[kt][i];
+                }
+    };
+
+    bf16x8_t ones8;
+    { U16 t; t.u = make_uint4(0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u); ones8 = t.v; }
+    // one key block (in LDS buffer `buf`, keys from j0) against the RT row tiles of this wave
+    auto multiply = [&](int buf, int j0) __attribute__((always_inline)) {
+        if (j0 > wave_hi || j0 + KB - 1 < wave_lo) return;   // every key masked for every row of the wave
+        const bf16_t* const kd = k_lds + buf * (KB * KROW);
+        const bf16_t* const vd = v_lds + buf * (D * VROW);
+        f32x4_t s[RT][KT];
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) {
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) s[rt][kt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+            const bf16_t* kr = kd + (kt * 16 + r) * KROW;
+            if constexpr (WIDE) {
+#pragma unroll
+                for (int st = 0; st < QSTEPS; ++st) {
+                    U16 t; t.u = *(const uint4*)(kr + st * 32 + g * 8);
+#pragma unroll
+                    for (int rt = 0; rt < RT; ++rt)
+                        s[rt][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(t.v, q8[rt][st], s[rt][kt], 0, 0, 0);
                 }
             } else {
-                U8 pf;
-                pf.u.x = pk[0]; pf.u.y = pk[1];
 #pragma unroll
-                for (int t = 0; t < DT; ++t) {
-                    U8 vf; vf.u = *(const uint2*)&v_lds[buf][t * 16 + r][4 * g];
-                    if (rescale) o[rt][t] *= alpha;
-                    o[rt][t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf.v, pf.v, o[rt][t], 0, 0, 0);
+                for (int st = 0; st < QSTEPS; ++st) {
+                    U8 t; t.u = *(const uint2*)(kr + st * 16 + g * 4);
+#pragma unroll
+                    for (int rt = 0; rt < RT; ++rt)
+                        s[rt][kt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(t.v, q4[rt][st], s[rt][kt], 0, 0, 0);
                 }
             }
         }
-    };
-    auto window_for = [&](int j) {   // make sure the page ids of block j are in LDS (the same decision in every thread)
-        if (page_index(a, j + KB - 1) >= page_base + PAGE_WINDOW) {
-            __syncthreads();
-            page_base = page_index(a, j);
-            fill_pages();
-            __syncthreads();
+        // s[rt][kt][i] is key j0 + tile_key(kt, g, i) against row r of tile rt.  A tile with no visible key in
+        // this block keeps its state: every probability is 0 and its factor 1.
+        unsigned pk[RT][KT * 2];
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+            const bool full = (j0 + KB - 1 <= tile_first_p[rt]) && (j0 >= tile_last_lo[rt]);
+            float alpha;
+            if (full) tile_softmax<true>(s[rt], j0, g, p[rt], p_lo[rt], a.scale_log2, m[rt], alpha, pk[rt]);
+            else tile_softmax<false>(s[rt], j0, g, p[rt], p_lo[rt], a.scale_log2, m[rt], alpha, pk[rt]);
+            if (__any(alpha != 1.f)) {      // the maximum of some row moved
+#pragma unroll
+                for (int t = 0; t < DT; ++t) o[rt][t] *= alpha;
+                ol[rt] *= alpha;
+            }
+        }
+#pragma unroll
+        for (int h = 0; h < KH; ++h) {
+            U16 pf[RT];
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+                pf[rt].u = make_uint4(pk[rt][4 * h], pk[rt][4 * h + 1], pk[rt][4 * h + 2], pk[rt][4 * h + 3]);
+                ol[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones8, pf[rt].v, ol[rt], 0, 0, 0);
+            }
+#pragma unroll
+            for (int t = 0; t < DT; ++t) {
+                U16 vf; vf.u = *(const uint4*)(vd + (t * 16 + r) * VROW + 32 * h + 8 * g);
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt)
+                    o[rt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[rt].v, o[rt][t], 0, 0, 0);
+            }
         }
     };
 
-    // Two sets of staging registers and two LDS buffers: a block is fetched two steps before it is multiplied, so
-    // its loads have two multiplications' time to arrive.
-    Stage sa, sb;
-    fill_pages();
+    next_pages();
+    fetch();
+    park(0);
     __syncthreads();
-    fetch(sa, key_lo);
-    if (key_lo + KB < key_hi) { window_for(key_lo + KB); fetch(sb, key_lo + KB); }
-    park(sa, 0);
-    __syncthreads();
-    for (int j0 = key_lo; j0 < key_hi; j0 += 2 * KB) {
-        const int j1 = j0 + KB, j2 = j0 + 2 * KB, j3 = j0 + 3 * KB;
-        if (j2 < key_hi) { window_for(j2); fetch(sa, j2); }
-        multiply(0, j0);
-        if (j1 < key_hi) park(sb, 1);
+    int buf = 0;
+    for (int j0 = key_lo; j0 < key_hi; j0 += KB) {
+        const bool more = j0 + KB < key_hi;
+        if (more) fetch();              // the next block is on its way while this one is multiplied
+        multiply(buf, j0);
+        if (more) park(buf ^ 1);
         __syncthreads();
-        if (j1 >= key_hi) break;
-        if (j3 < key_hi) { window_for(j3); fetch(sb, j3); }
-        multiply(1, j1);
-        if (j2 < key_hi) park(sa, 0);
-        __syncthreads();
+        buf ^= 1;
     }
 
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
-        float lt = l[rt];
-        lt += __shfl_xor(lt, 16, 64);
-        lt += __shfl_xor(lt, 32, 64);
         if (!row_ok[rt]) continue;
+        const float lt = ol[rt][0];
         const float inv = lt > 0.f ? 1.f / lt : 0.f;
         bf16_t* orow = a.out + ((size_t)(q_tok0 + ti[rt]) * a.n_heads + head[rt]) * D;
 #pragma unroll
@@ -715,8 +815,17 @@ extern "C" int vt_attn_bf16_tiles(const void* q, const void* k_pages, const void
     a.num_pages = num_pages; a.window = window; a.scale_log2 = scale * 1.4426950408889634f;
     a.entry_pos0 = nullptr; a.dec_params = nullptr; a.p_max = 0; a.ps_shift = shift_of(page_size);
     dim3 grid(n_items, n_kv);
-    if (rt == 1) attn_bf16_tile_kernel<1><<<grid, 256, 0, stream>>>(a);
-    else attn_bf16_tile_kernel<2><<<grid, 256, 0, stream>>>(a);
+    // more LDS than a kernel gets without asking
+    static bool lds_set = false;
+    if (!lds_set) {
+        hipError_t e1 = hipFuncSetAttribute((const void*)attn_bf16_tile_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, TILE_LDS_BYTES);
+        hipError_t e2 = hipFuncSetAttribute((const void*)attn_bf16_tile_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize, TILE_LDS_BYTES);
+        VT_REQUIRE(e1 == hipSuccess && e2 == hipSuccess, "vt_attn_bf16_tiles: cannot get %d bytes of LDS: %s", TILE_LDS_BYTES,
+                   hipGetErrorString(e1 != hipSuccess ? e1 : e2));
+        lds_set = true;
+    }
+    if (rt == 1) attn_bf16_tile_kernel<1><<<grid, 256, TILE_LDS_BYTES, stream>>>(a);
+    else attn_bf16_tile_kernel<2><<<grid, 256, TILE_LDS_BYTES, stream>>>(a);
     VT_CHECK_LAUNCH("vt_attn_bf16_tiles");
     return 0;
 }

@@ -58,6 +58,7 @@ class AttentionPlan:
 MAX_PARTS = 128     # the merge kernel holds the weights of at most this many items per row tile
 
 
+TILE_RT2_MIN_BLOCKS = 384
 LONG_ENTRY_ROWS = 256   # entries with at least this many (token, head-of-group) rows go to the LDS-tiled kernel
 
 
@@ -76,7 +77,10 @@ def plan_tile_items(entry_start: np.ndarray, entry_pos0: np.ndarray, group: int,
     q_len = (entry_start[1:] - entry_start[:-1]).astype(np.int64)[entries]
     rows = q_len * group
     if rt is None:
-        rt = 1      # measured: 128-row items (rt = 2) halve the number of blocks and lose more than their reuse gains
+        # 128-row items (rt = 2) read every operand from LDS half as often, but halve the number of blocks: they
+        # pay once the machine's 256 compute units still get well over one block each (measured on 2,048 and
+        # 1,024-token portions)
+        rt = 2 if int(((rows + 127) // 128).sum()) * n_kv >= TILE_RT2_MIN_BLOCKS else 1
     rpi = 64 * rt
     n_tiles = (rows + rpi - 1) // rpi
     total = int(n_tiles.sum())
