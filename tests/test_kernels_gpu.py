@@ -510,3 +510,47 @@ def test_attention_decode_kernel(nh, kvh, d, window, chunk):
                             nh, kvh, d, window, scale)
     ref = torch.cat([ref_attention(qs[e][0], ks[e], vs[e], cached[e], window, scale).reshape(1, -1) for e in range(n)])
     assert rel_err(out, ref) < ATT_TOL[torch.bfloat16]
+
+
+@pytest.mark.parametrize("nh,kvh,d,rot", [(28, 4, 128, 128), (4, 2, 64, 32), (6, 2, 80, 0), (16, 1, 256, 256), (3, 1, 48, 32)])
+@pytest.mark.parametrize("window", [0, 37])
+@pytest.mark.parametrize("chunk", [64, 1024])
+def test_attention_decode_fused_kernel(nh, kvh, d, rot, window, chunk):
+    """The decode attention that rotates and writes the pages itself against the separate rotation kernel followed
+    by the plain decode attention, at two sets of positions."""
+    o = ops()
+    g = torch.Generator().manual_seed(nh + d + chunk + window)
+    p_max, ps, max_pos = 16, 16, 1100
+    half = rot // 2
+    cos = sin = None
+    if rot:
+        ang = torch.rand(max_pos, half, generator=g, dtype=torch.float64) * 6.28
+        cos, sin = torch.cos(ang).float().to(DEV), torch.sin(ang).float().to(DEV)
+    for cached in ([0, 15, 16, 17, 300, 63, 1000], [31, 1, 999]):
+        n = len(cached)
+        lens = [c + 1 for c in cached]
+        ks = [torch.randn(t, kvh, d, generator=g).to(torch.bfloat16).float() for t in lens]
+        vs = [torch.randn(t, kvh, d, generator=g).to(torch.bfloat16).float() for t in lens]
+        kp, vp, bt = make_pages(ks, vs, lens, ps, torch.bfloat16, 9)
+        kp, vp, bt = kp.to(DEV), vp.to(DEV), bt.to(DEV)
+        # the last key and value of every entry come from the projection's row instead of the pages
+        qkv = torch.randn(n, (nh + 2 * kvh) * d, generator=g).to(DEV)
+        pos = torch.tensor(cached, dtype=torch.int32, device=DEV)
+        tok_entry = torch.arange(n, dtype=torch.int32, device=DEV)
+        kp_ref, vp_ref = kp.clone(), vp.clone()
+        q_ref = torch.empty(n, nh * d, dtype=torch.bfloat16, device=DEV)
+        o.rope_store(qkv, cos, sin, pos, tok_entry, bt, q_ref, kp_ref, vp_ref, nh, kvh, d)
+        part_o = torch.full((n * p_max * kvh * 16 * d,), float("nan"), device=DEV)
+        part_ml = torch.full((n * p_max * kvh * 32,), float("nan"), device=DEV)
+        dec = torch.tensor([chunk, 0, 0, 0], dtype=torch.int32, device=DEV)
+        scale = 1.0 / math.sqrt(d)
+        out_ref = torch.full((n, nh * d), float("nan"), dtype=torch.bfloat16, device=DEV)
+        o.attention_bf16_decode(q_ref, kp_ref, vp_ref, bt, pos, dec, p_max, out_ref, part_o.clone(), part_ml.clone(), nh, kvh,
+                                d, window, scale)
+        out = torch.full((n, nh * d), float("nan"), dtype=torch.bfloat16, device=DEV)
+        o.attention_bf16_decode_fused(qkv, cos, sin, kp, vp, bt, pos, dec, p_max, out, part_o, part_ml, nh, kvh, d, window,
+                                      scale)
+        torch.cuda.synchronize()
+        assert torch.equal(kp, kp_ref) and torch.equal(vp, vp_ref)       # the same bits in the pages
+        assert bool(torch.isfinite(out.float()).all())
+        assert rel_err(out, out_ref.float().cpu()) < 2e-3                 # the same products, merged in the same order

@@ -58,6 +58,13 @@ struct AttnArgs {
                             //       captured launch can be replayed with another value
     int p_max;              // items per entry
     int ps_shift;           // log2(page_size) if it is a power of two, else -1
+    // fused decode: the projections' output comes in unrotated and in fp32; the kernel rotates queries and the new
+    // key itself and writes the new key and value into their page
+    const float* qkv;       // [entries][qkv_stride]: queries of all heads, then keys, then values; or null
+    long long qkv_stride;
+    const float* cos_t;     // [max_pos][rot / 2]
+    const float* sin_t;
+    int rot, max_pos;       // rotated dims of a head (a multiple of 16, or 0)
 };
 
 __device__ __forceinline__ int page_index(const AttnArgs& a, int j) {
@@ -167,6 +174,78 @@ __device__ __forceinline__ void load_block(KVBlock& b, const AttnArgs& a, int pg
     for (int t = 0; t < DT; ++t) b.v[t] = *(const uint2*)(vb + (size_t)t * 16 * ps);
 }
 
+// CH consecutive elements (from c, a multiple of CH) of a head as the projection left them in fp32, rotated: the
+// pairs are (i, i + rot/2) for i < rot/2, elements from rot on pass through; rot is a multiple of 2 CH.  The same
+// arithmetic as the separate rotation kernel (vt_rope_store).
+template <int CH>
+__device__ __forceinline__ void rotated_chunk(float (&x)[CH], const float* row, int c, int rot, const float* cos_t,
+                                              const float* sin_t, int pos, int max_pos) {
+#pragma unroll
+    for (int i = 0; i < CH; i += 4) {
+        const float4 v = *(const float4*)(row + c + i);
+        x[i] = v.x; x[i + 1] = v.y; x[i + 2] = v.z; x[i + 3] = v.w;
+    }
+    if (c < rot) {
+        const int half = rot >> 1;
+        const bool low = c < half;
+        const int tp = pos < max_pos ? (pos < 0 ? 0 : pos) : max_pos - 1;
+        const float* ct = cos_t + (size_t)tp * half + (low ? c : c - half);
+        const float* st = sin_t + (size_t)tp * half + (low ? c : c - half);
+        const float* other = row + (low ? c + half : c - half);
+#pragma unroll
+        for (int i = 0; i < CH; i += 4) {
+            const float4 y = *(const float4*)(other + i), cc = *(const float4*)(ct + i), sn = *(const float4*)(st + i);
+            if (low) {
+                x[i] = cc.x * x[i] - sn.x * y.x; x[i + 1] = cc.y * x[i + 1] - sn.y * y.y;
+                x[i + 2] = cc.z * x[i + 2] - sn.z * y.z; x[i + 3] = cc.w * x[i + 3] - sn.w * y.w;
+            } else {
+                x[i] = cc.x * x[i] + sn.x * y.x; x[i + 1] = cc.y * x[i + 1] + sn.y * y.y;
+                x[i + 2] = cc.z * x[i + 2] + sn.z * y.z; x[i + 3] = cc.w * x[i + 3] + sn.w * y.w;
+            }
+        }
+    }
+}
+
+// Merge the partial results of a tile of 16 rows whose keys were split over n_parts items; all 256 threads of a
+// block.  sm and sl are [MAX_PARTS][16] floats of LDS.  Slot of (part pi, row r) = slot0 + pi * slot_step + r.
+#define MAX_PARTS 128
+__device__ __forceinline__ void merge_parts(float (*sm)[16], float (*sl)[16], const float* part_o, const float* part_ml,
+                                            bf16_t* out, size_t slot0, size_t slot_step, int n_parts, int n_valid,
+                                            int q_tok0, int q_row0, int G, int kvh, int n_heads) {
+    const int tid = threadIdx.x;
+    for (int i = tid; i < n_parts * 16; i += 256) {
+        const int pi = i >> 4, r = i & 15;
+        const size_t sl_ = slot0 + pi * slot_step + r;
+        const bool ok = r < n_valid;
+        sm[pi][r] = ok ? part_ml[sl_ * 2] : -INFINITY;
+        sl[pi][r] = ok ? part_ml[sl_ * 2 + 1] : 0.f;
+    }
+    __syncthreads();
+    if (tid < 16) {
+        float mx = -INFINITY;
+        for (int pi = 0; pi < n_parts; ++pi) mx = fmaxf(mx, sm[pi][tid]);
+        float den = 0.f;
+        for (int pi = 0; pi < n_parts; ++pi) {
+            const float w = (sm[pi][tid] == -INFINITY) ? 0.f : exp2f(sm[pi][tid] - mx);
+            den += w * sl[pi][tid];
+            sm[pi][tid] = w;
+        }
+        const float inv = den > 0.f ? 1.f / den : 0.f;
+        for (int pi = 0; pi < n_parts; ++pi) sm[pi][tid] *= inv;
+    }
+    __syncthreads();
+    for (int idx = tid; idx < n_valid * D; idx += 256) {
+        const int r = idx / D, d = idx - r * D;
+        const float* po = part_o + (slot0 + r) * D + d;
+        float acc = 0.f;
+#pragma unroll 4
+        for (int pi = 0; pi < n_parts; ++pi) acc += sm[pi][r] * po[(size_t)pi * slot_step * D];
+        const int row = q_row0 + r;
+        const int ti = row / G, head = kvh * G + (row - ti * G);
+        out[((size_t)(q_tok0 + ti) * n_heads + head) * D + d] = f32_to_bf16(acc);
+    }
+}
+
 // RT row tiles of 16 rows per wave share every key/value block they read.
 template <bool DECODE, int RT>
 __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_kernel(AttnArgs a) {
@@ -175,6 +254,7 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_kernel(AttnArg
     const int item = DECODE ? (int)blockIdx.x : (int)blockIdx.x * 4 + wv;
     if (item >= a.n_items) return;
     int entry, q_tok0, q_len, pos0, q_row0, key_lo, key_hi, part;
+    bool dec_writes = false;
     if (DECODE) {
         // item = (entry, part p): keys [p*chunk, (p+1)*chunk) of the entry's one token
         const int chunk = a.dec_params[0];
@@ -191,6 +271,7 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_kernel(AttnArg
         key_lo = max((lo >> 4) << 4, pi * chunk);
         key_hi = min(pos0 + 1, (pi + 1) * chunk);
         part = (p_first == p_last) ? -1 : entry * a.p_max + pi;
+        dec_writes = pi == p_last;                    // this item's keys include the token's own
     } else {
         const int* it = a.items + (size_t)item * ITEM_INTS;
         entry = it[0]; q_tok0 = it[1]; q_len = it[2]; pos0 = it[3]; q_row0 = it[4];
@@ -224,18 +305,63 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_kernel(AttnArg
         // a block whose keys lie between these two is visible to every row of the tile
         tile_first_p[rt] = pos0 + first_row / G;
         tile_last_lo[rt] = a.window > 0 ? pos0 + last_row / G - a.window + 1 : 0;
-        const bf16_t* qrow = a.q + ((size_t)(q_tok0 + ti[rt]) * a.n_heads + head[rt]) * D;
-        if constexpr (WIDE) {
+        if (DECODE && a.qkv) {
+            // the query as the projection left it: rotate its pairs (i, i + rot/2) by the angles of its position
+            const float* qrow = a.qkv + (size_t)q_tok0 * a.qkv_stride + (size_t)head[rt] * D;
+            constexpr int CH = WIDE ? 8 : 4, STEP = WIDE ? 32 : 16;
 #pragma unroll
-            for (int s = 0; s < QSTEPS; ++s) { U16 t; t.u = *(const uint4*)(qrow + s * 32 + g * 8); q8[rt][s] = t.v; }
+            for (int s = 0; s < QSTEPS; ++s) {
+                float x[CH];
+                rotated_chunk<CH>(x, qrow, s * STEP + g * CH, a.rot, a.cos_t, a.sin_t, pos0, a.max_pos);
+                if constexpr (WIDE) {
+                    U16 t; t.u = make_uint4(pack2(x[0], x[1]), pack2(x[2], x[3]), pack2(x[4], x[5]), pack2(x[6], x[7]));
+                    q8[rt][s] = t.v;
+                } else {
+                    U8 t; t.u = make_uint2(pack2(x[0], x[1]), pack2(x[2], x[3]));
+                    q4[rt][s] = t.v;
+                }
+            }
         } else {
+            const bf16_t* qrow = a.q + ((size_t)(q_tok0 + ti[rt]) * a.n_heads + head[rt]) * D;
+            if constexpr (WIDE) {
 #pragma unroll
-            for (int s = 0; s < QSTEPS; ++s) { U8 t; t.u = *(const uint2*)(qrow + s * 16 + g * 4); q4[rt][s] = t.v; }
+                for (int s = 0; s < QSTEPS; ++s) { U16 t; t.u = *(const uint4*)(qrow + s * 32 + g * 8); q8[rt][s] = t.v; }
+            } else {
+#pragma unroll
+                for (int s = 0; s < QSTEPS; ++s) { U8 t; t.u = *(const uint2*)(qrow + s * 16 + g * 4); q4[rt][s] = t.v; }
+            }
         }
 #pragma unroll
         for (int t = 0; t < DT; ++t) o[rt][t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
         m[rt] = -INFINITY;
         l[rt] = 0.f;
+    }
+
+    if (DECODE && a.qkv && dec_writes) {
+        // The token's own key (rotated) and value go into their page before this block reads it.  No other block
+        // reads this slot: the other items of the entry end before it, other kv heads have pages of their own.
+        const int ps_ = a.page_size;
+        const int blk = pos0 / ps_, slot = pos0 - blk * ps_;
+        const int pg = a.block_table[(size_t)entry * a.max_blocks + blk];
+        if (pg >= 0 && pg < a.num_pages) {      // the host never leaves the token without a page
+            const int tid = threadIdx.x;
+            if (tid < D / 4) {
+                float x[4];
+                rotated_chunk<4>(x, a.qkv + (size_t)q_tok0 * a.qkv_stride + (size_t)(a.n_heads + kvh) * D, tid * 4, a.rot,
+                                 a.cos_t, a.sin_t, pos0, a.max_pos);
+                bf16_t* kp = (bf16_t*)a.k_pages + (((size_t)pg * a.n_kv + kvh) * ps_ + slot) * D + tid * 4;
+                *(uint2*)kp = make_uint2(pack2(x[0], x[1]), pack2(x[2], x[3]));
+            } else if (tid >= 64 && tid < 64 + D / 4) {
+                const int i = (tid - 64) * 4;
+                const float4 v = *(const float4*)(a.qkv + (size_t)q_tok0 * a.qkv_stride + (size_t)(a.n_heads + a.n_kv + kvh) * D + i);
+                bf16_t* vp = (bf16_t*)a.v_pages + (((size_t)pg * a.n_kv + kvh) * D + i) * ps_ + slot;
+                vp[0] = f32_to_bf16(v.x);
+                vp[(size_t)ps_] = f32_to_bf16(v.y);
+                vp[(size_t)2 * ps_] = f32_to_bf16(v.z);
+                vp[(size_t)3 * ps_] = f32_to_bf16(v.w);
+            }
+        }
+        __syncthreads();
     }
 
     // Page ids of up to 64 pages at a time, one per lane: reading the table is then off the path of every block's
@@ -691,10 +817,8 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_tile_kernel(At
     }
 }
 
-// Merge the partial results of a tile of 16 rows whose keys were split over several items.
 // citems: [n][6] = q_tok0, q_len, first row of the tile, first item's partial index, number of items, tile index
 // within its items (each item holds `rt_per_item` tiles).  One block per (tile, kv head).
-#define MAX_PARTS 128
 template <bool DECODE>
 __global__ __launch_bounds__(256) void attn_combine_kernel(const int* __restrict__ citems, const float* __restrict__ part_o,
                                                           const float* __restrict__ part_ml, bf16_t* __restrict__ out,
@@ -718,42 +842,11 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const int* __restrict
         if (n_parts <= 0) return;
     }
     n_parts = min(n_parts, MAX_PARTS);   // the host never plans more
-    const int kvh = blockIdx.y, G = n_heads / n_kv, tid = threadIdx.x;
+    const int kvh = blockIdx.y, G = n_heads / n_kv;
     const int n_valid = min(16, q_len * G - q_row0);
-    // slot of (part pi, row r) = (((part0 + pi) * rt_per_item + rt) * n_kv + kvh) * 16 + r
     const size_t slot0 = (((size_t)part0 * rt_per_item + rt) * n_kv + kvh) * 16;
     const size_t slot_step = (size_t)rt_per_item * n_kv * 16;
-    for (int i = tid; i < n_parts * 16; i += 256) {
-        const int pi = i >> 4, r = i & 15;
-        const size_t sl_ = slot0 + pi * slot_step + r;
-        const bool ok = r < n_valid;
-        sm[pi][r] = ok ? part_ml[sl_ * 2] : -INFINITY;
-        sl[pi][r] = ok ? part_ml[sl_ * 2 + 1] : 0.f;
-    }
-    __syncthreads();
-    if (tid < 16) {
-        float mx = -INFINITY;
-        for (int pi = 0; pi < n_parts; ++pi) mx = fmaxf(mx, sm[pi][tid]);
-        float den = 0.f;
-        for (int pi = 0; pi < n_parts; ++pi) {
-            const float w = (sm[pi][tid] == -INFINITY) ? 0.f : exp2f(sm[pi][tid] - mx);
-            den += w * sl[pi][tid];
-            sm[pi][tid] = w;
-        }
-        const float inv = den > 0.f ? 1.f / den : 0.f;
-        for (int pi = 0; pi < n_parts; ++pi) sm[pi][tid] *= inv;
-    }
-    __syncthreads();
-    for (int idx = tid; idx < n_valid * D; idx += 256) {
-        const int r = idx / D, d = idx - r * D;
-        const float* po = part_o + (slot0 + r) * D + d;
-        float acc = 0.f;
-#pragma unroll 4
-        for (int pi = 0; pi < n_parts; ++pi) acc += sm[pi][r] * po[(size_t)pi * slot_step * D];
-        const int row = q_row0 + r;
-        const int ti = row / G, head = kvh * G + (row - ti * G);
-        out[((size_t)(q_tok0 + ti) * n_heads + head) * D + d] = f32_to_bf16(acc);
-    }
+    merge_parts(sm, sl, part_o, part_ml, out, slot0, slot_step, n_parts, n_valid, q_tok0, q_row0, G, kvh, n_heads);
 }
 
 extern "C" int vt_attn_bf16_head_dim() { return D; }
@@ -788,6 +881,7 @@ extern "C" int vt_attn_bf16(const void* q, const void* k_pages, const void* v_pa
     a.n_items = n_items; a.n_heads = n_heads; a.n_kv = n_kv; a.page_size = page_size; a.max_blocks = max_blocks;
     a.num_pages = num_pages; a.window = window; a.scale_log2 = scale * 1.4426950408889634f;
     a.entry_pos0 = nullptr; a.dec_params = nullptr; a.p_max = 0; a.ps_shift = shift_of(page_size);
+    a.qkv = nullptr; a.qkv_stride = 0; a.cos_t = a.sin_t = nullptr; a.rot = a.max_pos = 0;
     dim3 grid((n_items + 3) / 4, n_kv);
     if (rt == 1) attn_bf16_kernel<false, 1><<<grid, 256, 0, stream>>>(a);
     else attn_bf16_kernel<false, 2><<<grid, 256, 0, stream>>>(a);
@@ -814,6 +908,7 @@ extern "C" int vt_attn_bf16_tiles(const void* q, const void* k_pages, const void
     a.n_items = n_items; a.n_heads = n_heads; a.n_kv = n_kv; a.page_size = page_size; a.max_blocks = max_blocks;
     a.num_pages = num_pages; a.window = window; a.scale_log2 = scale * 1.4426950408889634f;
     a.entry_pos0 = nullptr; a.dec_params = nullptr; a.p_max = 0; a.ps_shift = shift_of(page_size);
+    a.qkv = nullptr; a.qkv_stride = 0; a.cos_t = a.sin_t = nullptr; a.rot = a.max_pos = 0;
     dim3 grid(n_items, n_kv);
     // more LDS than a kernel gets without asking
     static bool lds_set = false;
@@ -850,10 +945,46 @@ extern "C" int vt_attn_bf16_decode(const void* q, const void* k_pages, const voi
     a.n_items = n_entries * p_max; a.n_heads = n_heads; a.n_kv = n_kv; a.page_size = page_size; a.max_blocks = max_blocks;
     a.num_pages = num_pages; a.window = window; a.scale_log2 = scale * 1.4426950408889634f;
     a.entry_pos0 = entry_pos0; a.dec_params = dec_params; a.p_max = p_max; a.ps_shift = shift_of(page_size);
+    a.qkv = nullptr; a.qkv_stride = 0; a.cos_t = a.sin_t = nullptr; a.rot = a.max_pos = 0;
     attn_bf16_kernel<true, 1><<<dim3(a.n_items, n_kv), 256, 0, stream>>>(a);
     VT_CHECK_LAUNCH("vt_attn_bf16_decode");
     attn_combine_kernel<true><<<dim3(n_entries, n_kv), 256, 0, stream>>>(nullptr, part_o, part_ml, (bf16_t*)out, n_heads,
                                                                         n_kv, entry_pos0, dec_params, p_max, window, 1);
     VT_CHECK_LAUNCH("vt_attn_bf16_decode(combine)");
+    return 0;
+}
+
+// Decoding, fused: as vt_attn_bf16_decode, but from the projections' fp32 output qkv [entries][qkv_stride] (queries
+// of all heads, keys, values).  The attention kernel rotates the queries and the new key by the angles of the
+// token's position (tables [max_pos][rot/2]; rot = 0: no rotation) and writes the new key and value into the
+// token's page itself: two launches instead of three.  (Merging an entry's items in the same launch, by the item
+// that finishes last, was measured too: the device-wide fences it needs cost more than the launch they save.)
+extern "C" int vt_attn_bf16_decode_fused(const float* qkv, long long qkv_stride, const float* cos_t, const float* sin_t,
+                                         int rot, int max_pos, void* k_pages, void* v_pages, const int* block_table,
+                                         const int* entry_pos0, const int* dec_params, int n_entries, int p_max, void* out,
+                                         float* part_o, float* part_ml, int n_heads, int n_kv, int page_size,
+                                         int max_blocks, int num_pages, int window, float scale, hipStream_t stream) {
+    if (check_common("vt_attn_bf16_decode_fused", n_heads, n_kv, page_size, max_blocks, num_pages)) return -1;
+    VT_REQUIRE(n_heads / n_kv <= 16, "vt_attn_bf16_decode_fused: %d query heads per kv head do not fit one tile of 16 rows",
+               n_heads / n_kv);
+    VT_REQUIRE(p_max > 0 && p_max <= MAX_PARTS, "vt_attn_bf16_decode_fused: %d items per entry (1..%d)", p_max, MAX_PARTS);
+    VT_REQUIRE(qkv && part_o && part_ml && entry_pos0 && dec_params, "vt_attn_bf16_decode_fused: missing buffers");
+    VT_REQUIRE(qkv_stride >= (long long)(n_heads + 2 * n_kv) * D && qkv_stride % 4 == 0,
+               "vt_attn_bf16_decode_fused: row stride %lld does not hold %d heads of %d", qkv_stride, n_heads + 2 * n_kv, D);
+    VT_REQUIRE(rot >= 0 && rot <= D && rot % 16 == 0, "vt_attn_bf16_decode_fused: %d rotated dims (a multiple of 16 up to %d)", rot, D);
+    VT_REQUIRE(rot == 0 || (cos_t && sin_t && max_pos > 0), "vt_attn_bf16_decode_fused: no rotary table");
+    if (n_entries <= 0) return 0;
+    AttnArgs a;
+    a.q = nullptr; a.k_pages = (const bf16_t*)k_pages; a.v_pages = (const bf16_t*)v_pages;
+    a.block_table = block_table; a.items = nullptr; a.out = (bf16_t*)out; a.part_o = part_o; a.part_ml = part_ml;
+    a.n_items = n_entries * p_max; a.n_heads = n_heads; a.n_kv = n_kv; a.page_size = page_size; a.max_blocks = max_blocks;
+    a.num_pages = num_pages; a.window = window; a.scale_log2 = scale * 1.4426950408889634f;
+    a.entry_pos0 = entry_pos0; a.dec_params = dec_params; a.p_max = p_max; a.ps_shift = shift_of(page_size);
+    a.qkv = qkv; a.qkv_stride = qkv_stride; a.cos_t = cos_t; a.sin_t = sin_t; a.rot = rot; a.max_pos = max_pos;
+    attn_bf16_kernel<true, 1><<<dim3(a.n_items, n_kv), 256, 0, stream>>>(a);
+    VT_CHECK_LAUNCH("vt_attn_bf16_decode_fused");
+    attn_combine_kernel<true><<<dim3(n_entries, n_kv), 256, 0, stream>>>(nullptr, part_o, part_ml, (bf16_t*)out, n_heads,
+                                                                        n_kv, entry_pos0, dec_params, p_max, window, 1);
+    VT_CHECK_LAUNCH("vt_attn_bf16_decode_fused(combine)");
     return 0;
 }

@@ -330,6 +330,47 @@ def attention_bf16_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch
     return out
 
 
+def attention_bf16_decode_fused(qkv: torch.Tensor, cos: Optional[torch.Tensor], sin: Optional[torch.Tensor],
+                                k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
+                                entry_pos0: torch.Tensor, dec_params: torch.Tensor, p_max: int, out: torch.Tensor,
+                                part_o: torch.Tensor, part_ml: torch.Tensor, n_heads: int, n_kv: int, head_dim: int,
+                                window: int, scale: float) -> torch.Tensor:
+    """attention_bf16_decode from the projections' fp32 output (queries, keys, values of token i = entry i in row i):
+    the attention kernel rotates queries and the new key and writes key and value into the token's page itself."""
+    n = qkv.shape[0]
+    num_pages, kvh, page_size, d = k_pages.shape
+    if head_dim % 16 or not 16 <= head_dim <= 256:
+        raise KernelError(f"attention_bf16_decode_fused: head size {head_dim} is not a multiple of 16 in 16..256")
+    _chk(qkv, "attention_bf16_decode_fused.qkv", torch.float32)
+    if qkv.dim() != 2 or qkv.shape[1] < (n_heads + 2 * n_kv) * head_dim or qkv.stride(1) != 1:
+        raise KernelError(f"attention_bf16_decode_fused.qkv: shape {tuple(qkv.shape)} does not hold {n_heads}+2x{n_kv} heads of {head_dim}")
+    rot = max_pos = 0
+    if cos is not None:
+        _chk(cos, "attention_bf16_decode_fused.cos", torch.float32)
+        _chk(sin, "attention_bf16_decode_fused.sin", torch.float32, cos.shape)
+        max_pos, half = cos.shape
+        rot = 2 * half
+        if rot % 16 or rot > head_dim:
+            raise KernelError(f"attention_bf16_decode_fused: {rot} rotated dims (a multiple of 16 up to {head_dim})")
+    _chk(k_pages, "attention_bf16_decode_fused.k_pages", torch.bfloat16, (num_pages, n_kv, page_size, head_dim))
+    _chk(v_pages, "attention_bf16_decode_fused.v_pages", torch.bfloat16, (num_pages, n_kv, head_dim, page_size))
+    _chk(block_table, "attention_bf16_decode_fused.block_table", torch.int32)
+    if block_table.shape[0] < n:
+        raise KernelError("attention_bf16_decode_fused: fewer block table rows than entries")
+    _chk(entry_pos0, "attention_bf16_decode_fused.entry_pos0", torch.int32, (n,))
+    _chk(dec_params, "attention_bf16_decode_fused.dec_params", torch.int32)
+    _chk(out, "attention_bf16_decode_fused.out", torch.bfloat16, (n, n_heads * head_dim))
+    _chk(part_o, "attention_bf16_decode_fused.part_o", torch.float32)
+    _chk(part_ml, "attention_bf16_decode_fused.part_ml", torch.float32)
+    if part_o.numel() < n * p_max * n_kv * 16 * head_dim or part_ml.numel() < n * p_max * n_kv * 32:
+        raise KernelError("attention_bf16_decode_fused: workspace too small")
+    _run(load_lib("vt_attn_bf16", head_dim), "vt_attn_bf16_decode_fused", _ptr(qkv), ctypes.c_longlong(qkv.stride(0)),
+         _ptr(cos), _ptr(sin), _i(rot), _i(max_pos), _ptr(k_pages), _ptr(v_pages), _ptr(block_table), _ptr(entry_pos0),
+         _ptr(dec_params), _i(n), _i(p_max), _ptr(out), _ptr(part_o), _ptr(part_ml), _i(n_heads), _i(n_kv),
+         _i(page_size), _i(block_table.shape[1]), _i(num_pages), _i(window), _f(scale), _stream())
+    return out
+
+
 # ---------------------------------------------------------------------------
 def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
            uniform: torch.Tensor, work: torch.Tensor, out: torch.Tensor) -> torch.Tensor:

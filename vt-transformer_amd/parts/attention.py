@@ -112,6 +112,18 @@ class PagedAttention(Part):
             if cache.writes:
                 qkv[:, nq:nq + nkv * d] = k2.reshape(n, nkv * d).to(qkv.dtype)
         cos, sin = tables if tables is not None else (None, None)
+        plain_positions = tables is not None or getattr(self.position, "dim", 0) == 0
+        if (rt.dtype == torch.bfloat16 and ctx.decode_params is not None and cache.writes and qkv.dtype == torch.float32
+                and plain_positions and nh // nkv <= 16 and (cos is None or cos.shape[1] % 8 == 0)):
+            # one token per entry, straight from the projection: the attention kernel rotates and writes the pages
+            out = rt.buffer("attn.out", (n, nq), rt.dtype)
+            part_o = rt.buffer("attn.dec_part_o", (n * ctx.decode_p_max * nkv * 16 * d,), torch.float32)
+            part_ml = rt.buffer("attn.dec_part_ml", (n * ctx.decode_p_max * nkv * 32,), torch.float32)
+            b = decode_bucket(nkv)
+            ops.attention_bf16_decode_fused(qkv, cos, sin, cache.k, cache.v, cache.block_table, ctx.entry_pos0,
+                                            ctx.decode_params[b:b + 1], ctx.decode_p_max, out, part_o, part_ml, nh, nkv, d,
+                                            self.window, self.scale)
+            return linear(rt, out, self.w_o, self.b_o, "attn.o")
         q = rt.buffer("attn.q", (n, nq), rt.dtype)
         ops.rope_store(qkv, cos, sin, ctx.positions, ctx.tok_entry, cache.block_table, q, cache.k, cache.v, nh, nkv, d,
                        write_kv=cache.writes)
