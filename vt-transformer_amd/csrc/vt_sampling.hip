@@ -1,4 +1,5 @@
-// Next-token choice from fp32 logits, one block per row.
+// Next-token choice from fp32 logits: the largest logit of every row first, by SLICES blocks per row that
+// each scan a slice; then one block per row.
 //
 // Greedy: the largest logit, the lowest index among equals.  The reference's
 // easy_top1 (v1/tensortype/hip_kernels/sampling.cpp:138-165) leaves the order
@@ -32,38 +33,63 @@ __device__ __forceinline__ int block_sum_int(int v, int* red) {
     return t;
 }
 
+#define SLICES 32
+
+__device__ __forceinline__ void take_larger(float& bv, int& bi, float v, int i) {
+    if (v > bv || (v == bv && i < bi)) { bv = v; bi = i; }
+}
+
+// largest logit (lowest index among equals) of slice blockIdx.x of row blockIdx.y -> pval/pidx[row][slice]
+__global__ __launch_bounds__(256) void argmax_slices_kernel(const float* __restrict__ logits, int V, float* __restrict__ pval,
+                                                           int* __restrict__ pidx) {
+    __shared__ float sval[4];
+    __shared__ int sidx[4];
+    const int row = blockIdx.y, tid = threadIdx.x;
+    const float* lg = logits + (size_t)row * V;
+    // slices of whole groups of four, so that an aligned row is read 16 bytes at a time
+    const int per = ((V + SLICES - 1) / SLICES + 3) & ~3;
+    const int b = blockIdx.x * per, e = min(V, b + per);
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    if ((((size_t)lg) & 15) == 0) {
+        const int e4 = b + ((e - b) & ~3);
+        for (int i = b + tid * 4; i < e4; i += 1024) {
+            const float4 v = *(const float4*)(lg + i);
+            take_larger(bv, bi, v.x, i); take_larger(bv, bi, v.y, i + 1);
+            take_larger(bv, bi, v.z, i + 2); take_larger(bv, bi, v.w, i + 3);
+        }
+        for (int i = e4 + tid; i < e; i += 256) take_larger(bv, bi, lg[i], i);
+    } else {
+        for (int i = b + tid; i < e; i += 256) take_larger(bv, bi, lg[i], i);
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) take_larger(bv, bi, __shfl_xor(bv, o, 64), __shfl_xor(bi, o, 64));
+    if ((tid & 63) == 0) { sval[tid >> 6] = bv; sidx[tid >> 6] = bi; }
+    __syncthreads();
+    if (tid == 0) {
+        for (int w = 1; w < 4; ++w) take_larger(bv, bi, sval[w], sidx[w]);
+        pval[row * SLICES + blockIdx.x] = bv;
+        pidx[row * SLICES + blockIdx.x] = bi;
+    }
+}
+
 __global__ __launch_bounds__(ST) void sample_kernel(const float* __restrict__ logits, int V,
                                                    const float* __restrict__ temperature, const int* __restrict__ top_k,
                                                    const float* __restrict__ top_p, const float* __restrict__ uniform,
+                                                   const float* __restrict__ pval, const int* __restrict__ pidx,
                                                    float* __restrict__ work, int* __restrict__ out) {
     __shared__ float red[16];
     __shared__ int redi[16];
-    __shared__ float sval[ST / 64];
-    __shared__ int sidx[ST / 64];
     __shared__ float seg[ST];
     const int row = blockIdx.x, tid = threadIdx.x;
     const float* lg = logits + (size_t)row * V;
     const float T = temperature[row];
     const int k = top_k[row];
 
-    // ---- largest logit, lowest index among equals ----
+    // ---- largest logit, lowest index among equals: the best of the slices ----
     float bv = -INFINITY;
     int bi = 0x7fffffff;
-    for (int i = tid; i < V; i += ST) {
-        float v = lg[i];
-        if (v > bv || (v == bv && i < bi)) { bv = v; bi = i; }
-    }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        float ov = __shfl_xor(bv, o, 64);
-        int oi = __shfl_xor(bi, o, 64);
-        if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
-    }
-    if ((tid & 63) == 0) { sval[tid >> 6] = bv; sidx[tid >> 6] = bi; }
-    __syncthreads();
-    bv = sval[0]; bi = sidx[0];
-    for (int w = 1; w < ST / 64; ++w)
-        if (sval[w] > bv || (sval[w] == bv && sidx[w] < bi)) { bv = sval[w]; bi = sidx[w]; }
+    for (int w = 0; w < SLICES; ++w) take_larger(bv, bi, pval[row * SLICES + w], pidx[row * SLICES + w]);
     if (!(T > 0.f) || k == 1) {
         if (tid == 0) out[row] = bi;
         return;
@@ -152,11 +178,21 @@ __global__ __launch_bounds__(ST) void sample_kernel(const float* __restrict__ lo
     }
 }
 
+// partials: 2 * vt_sample_slices() floats per row, scratch
+extern "C" int vt_sample_slices() { return SLICES; }
+
 extern "C" int vt_sample(const float* logits, int rows, int V, const float* temperature, const int* top_k,
-                         const float* top_p, const float* uniform, float* work, int* out, hipStream_t stream) {
+                         const float* top_p, const float* uniform, float* work, float* partials, int* out,
+                         hipStream_t stream) {
     VT_REQUIRE(rows >= 0 && V > 0, "vt_sample: bad sizes rows=%d vocab=%d", rows, V);
+    VT_REQUIRE(rows <= 65535, "vt_sample: %d rows (at most 65535)", rows);
+    VT_REQUIRE(partials != nullptr, "vt_sample: no scratch for the slices' maxima");
     if (rows == 0) return 0;
-    sample_kernel<<<rows, ST, 0, stream>>>(logits, V, temperature, top_k, top_p, uniform, work, out);
+    float* pval = partials;
+    int* pidx = (int*)(partials + (size_t)rows * SLICES);
+    argmax_slices_kernel<<<dim3(SLICES, rows), 256, 0, stream>>>(logits, V, pval, pidx);
+    VT_CHECK_LAUNCH("vt_sample(slices)");
+    sample_kernel<<<rows, ST, 0, stream>>>(logits, V, temperature, top_k, top_p, uniform, pval, pidx, work, out);
     VT_CHECK_LAUNCH("vt_sample");
     return 0;
 }

@@ -26,7 +26,7 @@ import torch
 from ..cache.pages import NO_PAGE, CacheError
 from ..cache.storage import CacheStorage
 from ..kernels.ops import ATTN_CITEM_INTS, ATTN_ITEM_INTS
-from ..parts.base import Runtime
+from ..parts.base import HostStaging, Runtime
 
 
 class OutOfPages(RuntimeError):
@@ -278,6 +278,7 @@ class ModelRunner:
         self.vocab_size = model.spec.vocab_size
         self.steps = 0
         self.tokens = 0
+        self._staging = HostStaging(torch.int32)
         self.decode_p_max = max(1, min(16, -(-self.max_seq_len // 64)))   # items one entry's keys are cut into at most
         # Decoding steps of a bfloat16 model are captured once per batch size and replayed, unless a mixer keeps
         # state of its own between steps (the warm-up run before a capture would advance it twice).
@@ -357,7 +358,7 @@ class ModelRunner:
         flat = np.concatenate(parts)
         if dev.numel() != flat.size:
             raise RuntimeError("step metadata does not fit its device buffer")
-        dev.copy_(torch.from_numpy(flat))
+        self._staging.upload(flat, dev)
         views, off = [], 0
         for p in parts:
             views.append(dev[off:off + p.size])

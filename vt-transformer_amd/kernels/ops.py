@@ -373,7 +373,9 @@ def attention_bf16_decode_fused(qkv: torch.Tensor, cos: Optional[torch.Tensor], 
 
 # ---------------------------------------------------------------------------
 def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
-           uniform: torch.Tensor, work: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+           uniform: torch.Tensor, work: torch.Tensor, out: torch.Tensor,
+           partials: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """partials: scratch of sample_partials_size(rows) floats (made here if not given)."""
     rows, vocab = logits.shape
     _chk(logits, "sample.logits", torch.float32)
     _chk(temperature, "sample.temperature", torch.float32, (rows,))
@@ -384,9 +386,18 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
     if work.numel() < rows * vocab:
         raise KernelError("sample: workspace smaller than the logits")
     _chk(out, "sample.out", torch.int32, (rows,))
+    if partials is None:
+        partials = torch.empty(sample_partials_size(rows), dtype=torch.float32, device=logits.device)
+    _chk(partials, "sample.partials", torch.float32)
+    if partials.numel() < sample_partials_size(rows):
+        raise KernelError("sample: scratch for the slices' maxima is too small")
     _run(load_lib("vt_sampling"), "vt_sample", _ptr(logits), _i(rows), _i(vocab), _ptr(temperature), _ptr(top_k),
-         _ptr(top_p), _ptr(uniform), _ptr(work), _ptr(out), _stream())
+         _ptr(top_p), _ptr(uniform), _ptr(work), _ptr(partials), _ptr(out), _stream())
     return out
+
+
+def sample_partials_size(rows: int) -> int:
+    return 2 * max(1, rows) * int(load_lib("vt_sampling").vt_sample_slices())
 
 
 def require_gpu() -> torch.device:

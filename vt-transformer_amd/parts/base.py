@@ -122,6 +122,31 @@ class Runtime:
         return _Scope()
 
 
+class HostStaging:
+    """Pinned host buffers in rotation for copies to the device that do not make the host wait: a buffer is
+    written again only after the copy that last read it has run."""
+
+    def __init__(self, dtype: torch.dtype, depth: int = 4):
+        self.dtype = dtype
+        self._slots = [[None, None] for _ in range(depth)]   # [pinned tensor, event of its last copy]
+        self._next = 0
+
+    def upload(self, host, dev: torch.Tensor) -> None:
+        """host: a numpy array of the buffer's dtype; dev: a device tensor of the same size."""
+        n = int(host.size)
+        slot = self._slots[self._next]
+        self._next = (self._next + 1) % len(self._slots)
+        if slot[1] is not None:
+            slot[1].synchronize()
+        if slot[0] is None or slot[0].numel() < n:
+            slot[0] = torch.empty(max(n, 256), dtype=self.dtype, pin_memory=True)
+        slot[0][:n].numpy()[...] = host.reshape(-1)
+        dev.view(-1).copy_(slot[0][:n], non_blocking=True)
+        if slot[1] is None:
+            slot[1] = torch.cuda.Event()
+        slot[1].record()
+
+
 class Part:
     """Base of all parts."""
 

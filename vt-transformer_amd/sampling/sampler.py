@@ -16,7 +16,7 @@ import numpy as np
 import torch
 
 from ..kernels import ops
-from ..parts.base import Runtime
+from ..parts.base import HostStaging, Runtime
 from .params import SamplingParams
 
 _M64 = (1 << 64) - 1
@@ -45,6 +45,7 @@ def request_seed(engine_seed: int, request_key) -> int:
 class Sampler:
     def __init__(self, rt: Runtime):
         self.rt = rt
+        self._staging = HostStaging(torch.float32)
 
     def sample(self, logits: torch.Tensor, rows: Sequence[Tuple[SamplingParams, int, int]]) -> List[int]:
         """logits [R, V] fp32 on the device; rows[i] = (params, seed, counter) of row i."""
@@ -59,11 +60,12 @@ class Sampler:
             host[2, i] = uniform(seed, counter)
             host[3, i] = np.int32(p.top_k).view(np.float32)
         dev = self.rt.buffer("sample.params", (4, r), torch.float32)
-        dev.copy_(torch.from_numpy(host))
+        self._staging.upload(host, dev)
         out = self.rt.buffer("sample.out", (r,), torch.int32)
         if any(host[0, i] > 0 for i in range(r)):
             work = self.rt.buffer("sample.work", (r * v,), torch.float32)   # probabilities of the stochastic rows
         else:
             work = logits.view(-1)   # greedy rows never touch the workspace
-        ops.sample(logits, dev[0], dev[3].view(torch.int32), dev[1], dev[2], work, out)
+        partials = self.rt.buffer("sample.partials", (ops.sample_partials_size(r),), torch.float32)
+        ops.sample(logits, dev[0], dev[3].view(torch.int32), dev[1], dev[2], work, out, partials)
         return out.cpu().tolist()
