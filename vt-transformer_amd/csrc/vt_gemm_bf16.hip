@@ -1,7 +1,7 @@
 // bfloat16 linear layers on the gfx950 matrix cores, for few rows (decoding
 // and short portions): y[n, m] = sum_k x[n, k] * W[m, k] (+ bias[m]), fp32
 // accumulation, fp32 or bf16 output; and the same with the SiLU gate fused:
-// y[n, i] = silu(x.W[i]) * (x.W[I + i]).
+// y[n, i] = silu(x.Wg[i]) * (x.Wu[i]).
 //
 // The reference calls hipblasGemmEx for each projection, rounds the result
 // to 16 bits and then adds the bias in a second kernel
@@ -10,10 +10,19 @@
 // (v1/models/qwen2-7b/inference_fp16.dag:333-336).  Here the bias and the gate
 // are applied to the fp32 accumulator.
 //
-// With few rows the time goes to reading W once from HBM, so the work is
-// laid out for that: a wave owns 16 rows of W and a slice of k, reads its
-// slice with 32 contiguous bytes per lane and feeds it to
-// v_mfma_f32_16x16x32_bf16 as the A operand; the tokens are the B operand.
+// With few rows the time goes to reading W once from HBM, so the weights are
+// kept in the order in which the matrix instruction wants them.  W [M, K] is
+// cut into tiles of 16 rows x 32 k; a tile is stored as the 64 lanes' operand
+// fragments one after the other (lane 16 g + r holds W[16 mt + r][32 kt + 8 g ..
+// + 8]), 1 KB in all, and the tiles of a row of tiles follow each other along k:
+//     packed[((mt * KT + kt) * 64 + lane) * 8 + j]
+// with M padded to 16 and K to 128 by zeros (vt_pack_matrix_bf16).  A wave's load
+// of a fragment is then 1 KB of consecutive memory, eight cache lines, where the
+// same fragment from a row-major W touches 64 separate 16-byte pieces of 16 rows:
+// the first-level cache handles a line per cycle, and with a piece per cycle the
+// matrix could not be read faster than about 4.4 TB/s; in this order it is read
+// at 5.3 to 5.6 TB/s.
+//
 // The waves of a block split k and add their partial sums through LDS in wave
 // order.  How k is split depends on the shape of W only, never on the number
 // of rows, so a token's result does not change with the batch around it.
@@ -29,151 +38,153 @@ union Frag {
     bf16x8_t v;
 };
 
-__device__ __forceinline__ bf16x8_t load_frag(const bf16_t* p, bool ok) {
+#define PK_TILE 512                 // elements of a packed tile
+#define PK_KPAD 128                 // K is padded to a multiple of this
+
+__host__ __device__ static inline int pk_rows(int M) { return (M + 15) & ~15; }
+__host__ __device__ static inline int pk_cols(int K) { return (K + PK_KPAD - 1) / PK_KPAD * PK_KPAD; }
+
+// ---------------------------------------------------------------------------
+// Packing: one thread per 16-byte piece of the packed matrix.
+// ---------------------------------------------------------------------------
+__global__ void pack_matrix_kernel(const bf16_t* __restrict__ w, bf16_t* __restrict__ wp, int M, int K, int KT, size_t pieces) {
+    const size_t p = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (p >= pieces) return;
+    const int lane = (int)(p & 63);
+    const size_t tile = p >> 6;
+    const int kt = (int)(tile % KT), mt = (int)(tile / KT);
+    const int m = mt * 16 + (lane & 15), k = kt * 32 + (lane >> 4) * 8;
+    uint32_t v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = (m < M && k + j < K) ? w[(size_t)m * K + k + j] : 0u;
+    uint4 o;
+    o.x = v[0] | (v[1] << 16); o.y = v[2] | (v[3] << 16);
+    o.z = v[4] | (v[5] << 16); o.w = v[6] | (v[7] << 16);
+    *(uint4*)(wp + p * 8) = o;
+}
+
+extern "C" long long vt_packed_elems(int M, int K) { return (long long)pk_rows(M) * pk_cols(K); }
+
+// wp must hold vt_packed_elems(M, K) elements
+extern "C" int vt_pack_matrix_bf16(const void* w, void* wp, int M, int K, hipStream_t stream) {
+    VT_REQUIRE(M > 0 && K > 0, "vt_pack_matrix_bf16: bad sizes M=%d K=%d", M, K);
+    VT_REQUIRE((((uintptr_t)wp) & 15) == 0, "vt_pack_matrix_bf16: the packed matrix must be 16-byte aligned");
+    const int KT = pk_cols(K) / 32;
+    const size_t pieces = (size_t)(pk_rows(M) / 16) * KT * 64;
+    pack_matrix_kernel<<<(unsigned)((pieces + 255) / 256), 256, 0, stream>>>((const bf16_t*)w, (bf16_t*)wp, M, K, KT, pieces);
+    VT_CHECK_LAUNCH("vt_pack_matrix_bf16");
+    return 0;
+}
+
+// x[row][k .. k + 8); beyond the end of the row its last eight values are read instead (W is zero there)
+__device__ __forceinline__ bf16x8_t load_x(const bf16_t* row, int k, int K) {
     Frag f;
-    if (ok) f.u = *(const uint4*)p;
-    else f.u = make_uint4(0, 0, 0, 0);
+    f.u = *(const uint4*)(row + min(k, K - 8));
     return f.v;
 }
 
-// One "step" is 64 values of k: lane group g = lane/16 reads k in [64 s + 16 g, 64 s + 16 g + 16),
-// the first 8 for one matrix instruction and the next 8 for a second one.
-//
-// A wave owns R tiles of 16 rows of W (rows m0 + 16 j + r) and NT tiles of 16 tokens: every fragment of x it
-// reads serves R row tiles, so the traffic for x (from L2) stays at NT/R of the traffic for W (from HBM).
-template <int NT, int R, int WPB, bool SWIGLU, typename TO>
-__global__ __launch_bounds__(WPB * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ x,
-                                                              const bf16_t* __restrict__ w,
-                                                              const float* __restrict__ bias, TO* __restrict__ y,
-                                                              int N, int Mout, int K) {
+// ---------------------------------------------------------------------------
+// Up to 16 tokens: a block owns one tile row of W (16 features; two for the gated product) and all of k, which
+// its WPB waves split; the tokens are the B operand, read from x as it lies in memory.  U tiles are in flight
+// per wave and matrix.
+// ---------------------------------------------------------------------------
+template <int WPB, bool SWIGLU, typename TO>
+__global__ __launch_bounds__(WPB * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wp,
+                                                              const float* __restrict__ bias, TO* __restrict__ y, int N,
+                                                              int Mout, int K, int KT, int up_tiles) {
     constexpr int NW = SWIGLU ? 2 : 1;
-    constexpr int RW = R * NW;                      // W fragments per k position
-    constexpr int U = (RW >= 4) ? 2 : 4;            // fragments of 8 k values in flight per row (1 or 2 steps)
-    __shared__ float red[RW][WPB][256];
+    constexpr int U = 4;
+    __shared__ float red[NW][WPB][256];
     const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63;
     const int r = lane & 15, g = lane >> 4;
-    const int m0 = blockIdx.x * (16 * R), n0 = blockIdx.y * (16 * NT);
-
-    const int S = (K + 63) >> 6;
-    const int s_begin = (int)(((long long)wv * S) / WPB), s_end = (int)(((long long)(wv + 1) * S) / WPB);
-
-    const bf16_t* wrow[RW];
+    const int mt = blockIdx.x;
+    const int t_begin = (int)(((long long)wv * KT) / WPB), t_end = (int)(((long long)(wv + 1) * KT) / WPB);
+    const bf16_t* wbase[NW];
+    wbase[0] = wp + ((size_t)mt * KT * 64 + lane) * 8;
+    if (SWIGLU) wbase[1] = wp + ((size_t)(mt + up_tiles) * KT * 64 + lane) * 8;
+    const bf16_t* xrow = x + (size_t)min(r, N - 1) * K;
+    f32x4_t acc[NW];
 #pragma unroll
-    for (int j = 0; j < R; ++j) {
-        const int mc = min(m0 + 16 * j + r, Mout - 1);
-        wrow[j] = w + (size_t)mc * K;
-        if (SWIGLU) wrow[R + j] = w + ((size_t)Mout + mc) * K;
-    }
-    const bf16_t* xrow[NT];
-#pragma unroll
-    for (int i = 0; i < NT; ++i) xrow[i] = x + (size_t)min(n0 + i * 16 + r, N - 1) * K;
-
-    f32x4_t acc[RW][NT];
-#pragma unroll
-    for (int a = 0; a < RW; ++a)
-#pragma unroll
-        for (int i = 0; i < NT; ++i) acc[a][i] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
-
-    // k position of fragment u of the group starting at step s: 64 s + 16 g + 8 u for u = 0, 1 and the same one
-    // step later for u = 2, 3
-    int s = s_begin;
-    constexpr int SPI = U / 2;                      // steps per iteration
-    for (; s + SPI <= s_end; s += SPI) {
-        bf16x8_t wa[RW][U], xa[NT][U];
+    for (int a = 0; a < NW; ++a) acc[a] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+    int t = t_begin;
+    for (; t + U <= t_end; t += U) {
+        Frag wa[NW][U];
+        bf16x8_t xa[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int k = (s + (u >> 1)) * 64 + g * 16 + (u & 1) * 8;
-            const bool ok = k < K;
 #pragma unroll
-            for (int a = 0; a < RW; ++a) wa[a][u] = load_frag(wrow[a] + k, ok);
-#pragma unroll
-            for (int i = 0; i < NT; ++i) xa[i][u] = load_frag(xrow[i] + k, ok);
+            for (int a = 0; a < NW; ++a) wa[a][u].u = *(const uint4*)(wbase[a] + (size_t)(t + u) * PK_TILE);
+            xa[u] = load_x(xrow, (t + u) * 32 + g * 8, K);
         }
 #pragma unroll
         for (int u = 0; u < U; ++u)
 #pragma unroll
-            for (int a = 0; a < RW; ++a)
-#pragma unroll
-                for (int i = 0; i < NT; ++i)
-                    acc[a][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[a][u], xa[i][u], acc[a][i], 0, 0, 0);
+            for (int a = 0; a < NW; ++a)
+                acc[a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[a][u].v, xa[u], acc[a], 0, 0, 0);
     }
-    for (; s < s_end; ++s) {
+    for (; t < t_end; ++t) {
+        const bf16x8_t xa = load_x(xrow, t * 32 + g * 8, K);
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
-            const int k = s * 64 + g * 16 + u * 8;
-            const bool ok = k < K;
-            bf16x8_t wa[RW], xa[NT];
-#pragma unroll
-            for (int a = 0; a < RW; ++a) wa[a] = load_frag(wrow[a] + k, ok);
-#pragma unroll
-            for (int i = 0; i < NT; ++i) xa[i] = load_frag(xrow[i] + k, ok);
-#pragma unroll
-            for (int a = 0; a < RW; ++a)
-#pragma unroll
-                for (int i = 0; i < NT; ++i)
-                    acc[a][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[a], xa[i], acc[a][i], 0, 0, 0);
+        for (int a = 0; a < NW; ++a) {
+            Frag wa;
+            wa.u = *(const uint4*)(wbase[a] + (size_t)t * PK_TILE);
+            acc[a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa.v, xa, acc[a], 0, 0, 0);
         }
     }
-
-    // acc[j][i][e] is feature m0 + 16 j + 4 g + e of token n0 + 16 i + r.  Sum the waves in wave order.
+    // acc[a][e] is feature 16 mt + 4 g + e of token r.  Sum the waves in wave order.
 #pragma unroll
-    for (int i = 0; i < NT; ++i) {
+    for (int a = 0; a < NW; ++a)
 #pragma unroll
-        for (int a = 0; a < RW; ++a)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) red[a][wv][lane * 4 + e] = acc[a][i][e];
-        __syncthreads();
-        for (int idx = tid; idx < R * 256; idx += WPB * 64) {
-            const int j = idx >> 8, c = idx & 255;
-            const int ln = c >> 2, e = c & 3;
-            const int m = m0 + 16 * j + 4 * (ln >> 4) + e, n = n0 + i * 16 + (ln & 15);
-            float v = 0.f, u = 0.f;
-            for (int q = 0; q < WPB; ++q) v += red[j][q][c];
-            if (SWIGLU)
-                for (int q = 0; q < WPB; ++q) u += red[(NW - 1) * R + j][q][c];
-            if (m < Mout && n < N) {
-                if (SWIGLU) v = v / (1.f + expf(-v)) * u;
-                else if (bias) v += bias[m];
-                store_f32<TO>(y, (size_t)n * Mout + m, v);
-            }
+        for (int e = 0; e < 4; ++e) red[a][wv][lane * 4 + e] = acc[a][e];
+    __syncthreads();
+    for (int c = tid; c < 256; c += WPB * 64) {
+        const int ln = c >> 2, e = c & 3;
+        const int m = mt * 16 + 4 * (ln >> 4) + e, n = ln & 15;
+        float v = 0.f, u = 0.f;
+        for (int q = 0; q < WPB; ++q) v += red[0][q][c];
+        if (SWIGLU)
+            for (int q = 0; q < WPB; ++q) u += red[NW - 1][q][c];
+        if (m < Mout && n < N) {
+            if (SWIGLU) v = v / (1.f + expf(-v)) * u;
+            else if (bias) v += bias[m];
+            store_f32<TO>(y, (size_t)n * Mout + m, v);
         }
-        __syncthreads();
     }
 }
 
 // ---------------------------------------------------------------------------
-// 17 to 128 rows (a large decoding batch, a short portion): a block of 4 waves takes 64*R rows of W and 64
-// tokens.  The tokens' values pass through LDS once per block (coalesced loads, two buffers), so they cost a
-// fraction of W's traffic instead of a multiple; each wave streams its own 16*R rows of W from memory into
-// registers one stage ahead.  For matrices with few rows the k range is split over blockIdx.z and the partial
-// sums (fp32, [split][N][M]) are added by vt_sum_partials in split order.
+// 17 to 64 tokens per block (a large decoding batch, a short portion): a block of 4 waves takes 64*R features
+// and 64 tokens.  The tokens' values pass through LDS once per block (coalesced loads, two buffers), so they cost
+// a fraction of W's traffic instead of a multiple; each wave streams the tiles of its own R tile rows of W from
+// memory into registers a stage (128 k, four tiles) ahead.  For matrices with few rows the k range is split over
+// blockIdx.z and the partial sums (fp32, [split][N][M]) are added by sum_partials_kernel in split order.
 // ---------------------------------------------------------------------------
-#ifndef MID_BK
-#define MID_BK 128                 // k values per stage (a multiple of 64)
-#endif
+#define MID_BK 128                 // k values per stage = PK_KPAD: a stage never leaves the packed matrix
 #define MID_XROW (MID_BK + 8)
-#define MID_KU (MID_BK / 32)       // matrix instructions along k per stage
+#define MID_KU (MID_BK / 32)       // tiles along k per stage
 #define MID_XP (MID_BK / 32)       // 16-byte pieces of x per thread and stage (64 tokens * MID_BK / 8 / 256)
 
 template <int R, bool SWIGLU, typename TO>
-__global__ __launch_bounds__(256) void gemm_mid_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+__global__ __launch_bounds__(256) void gemm_mid_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wp,
                                                       const float* __restrict__ bias, TO* __restrict__ y,
-                                                      float* __restrict__ partial, int N, int Mout, int K,
-                                                      int k_per_split) {
+                                                      float* __restrict__ partial, int N, int Mout, int K, int KT,
+                                                      int up_tiles, int k_per_split) {
     constexpr int NW = SWIGLU ? 2 : 1;
     constexpr int RW = R * NW;
     __shared__ __attribute__((aligned(16))) bf16_t xs[2][64][MID_XROW];
     const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63;
     const int r = lane & 15, g = lane >> 4;
-    const int m0 = blockIdx.x * (64 * R) + wv * (16 * R), n0 = blockIdx.y * 64;
-    const int k_begin = blockIdx.z * k_per_split, k_end = min(K, k_begin + k_per_split);
+    const int mt0 = (blockIdx.x * 4 + wv) * R, n0 = blockIdx.y * 64;
+    const int k_begin = blockIdx.z * k_per_split, k_end = min(pk_cols(K), k_begin + k_per_split);
+    const int m_tiles = pk_rows(Mout) >> 4;
 
-    const bf16_t* wrow[RW];
+    // this wave's tile rows; beyond the matrix the last one again (its results are not stored)
+    const bf16_t* wbase[RW];
 #pragma unroll
     for (int j = 0; j < R; ++j) {
-        const int mc = min(m0 + 16 * j + r, Mout - 1);
-        wrow[j] = w + (size_t)mc * K;
-        if (SWIGLU) wrow[R + j] = w + ((size_t)Mout + mc) * K;
+        const int mt = min(mt0 + j, m_tiles - 1);
+        wbase[j] = wp + ((size_t)mt * KT * 64 + lane) * 8;
+        if (SWIGLU) wbase[R + j] = wp + ((size_t)(mt + up_tiles) * KT * 64 + lane) * 8;
     }
     // this thread's 16-byte pieces of a stage of x: a token's MID_BK values are MID_BK/8 consecutive pieces
     const bf16_t* xsrc[MID_XP];
@@ -183,7 +194,7 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const bf16_t* __restrict_
         const int pidx = tid + 256 * q;
         xtok[q] = pidx / (MID_BK / 8);
         xcol[q] = (pidx % (MID_BK / 8)) * 8;
-        xsrc[q] = x + (size_t)min(n0 + xtok[q], N - 1) * K + xcol[q];
+        xsrc[q] = x + (size_t)min(n0 + xtok[q], N - 1) * K;
     }
     f32x4_t acc[RW][4];
 #pragma unroll
@@ -192,42 +203,41 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const bf16_t* __restrict_
         for (int i = 0; i < 4; ++i) acc[a][i] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 
     uint4 xreg[MID_XP];
-    bf16x8_t wcur[RW][MID_KU], wnxt[RW][MID_KU];
-    auto fetch_x = [&](int k0) {
+    Frag wcur[RW][MID_KU], wnxt[RW][MID_KU];
+    auto fetch_x = [&](int k0) __attribute__((always_inline)) {
 #pragma unroll
         for (int q = 0; q < MID_XP; ++q) {
             Frag f;
-            f.v = load_frag(xsrc[q] + k0, k0 + xcol[q] < k_end);
+            f.v = load_x(xsrc[q], k0 + xcol[q], K);
             xreg[q] = f.u;
         }
     };
-    auto park_x = [&](int buf) {
+    auto park_x = [&](int buf) __attribute__((always_inline)) {
 #pragma unroll
         for (int q = 0; q < MID_XP; ++q) *(uint4*)&xs[buf][xtok[q]][xcol[q]] = xreg[q];
     };
-    // fragment u of a stage: k = k0 + 64 (u/2) + 16 g + 8 (u%2), so a lane reads 32 contiguous bytes per 64 k
-    auto fetch_w = [&](bf16x8_t (&dst)[RW][MID_KU], int k0) {
+    auto fetch_w = [&](Frag (&dst)[RW][MID_KU], int k0) __attribute__((always_inline)) {
+        const size_t t0 = (size_t)(k0 >> 5) * PK_TILE;
 #pragma unroll
-        for (int u = 0; u < MID_KU; ++u) {
-            const int k = k0 + (u >> 1) * 64 + g * 16 + (u & 1) * 8;
+        for (int u = 0; u < MID_KU; ++u)
 #pragma unroll
-            for (int a = 0; a < RW; ++a) dst[a][u] = load_frag(wrow[a] + k, k < k_end);
-        }
+            for (int a = 0; a < RW; ++a) dst[a][u].u = *(const uint4*)(wbase[a] + t0 + (size_t)u * PK_TILE);
     };
-    auto multiply = [&](const bf16x8_t (&wf)[RW][MID_KU], int buf) {
+    auto multiply = [&](const Frag (&wf)[RW][MID_KU], int buf) __attribute__((always_inline)) {
 #pragma unroll
         for (int u = 0; u < MID_KU; ++u)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 Frag xf;
-                xf.u = *(const uint4*)&xs[buf][i * 16 + r][(u >> 1) * 64 + g * 16 + (u & 1) * 8];
+                xf.u = *(const uint4*)&xs[buf][i * 16 + r][u * 32 + g * 8];
 #pragma unroll
                 for (int a = 0; a < RW; ++a)
-                    acc[a][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[a][u], xf.v, acc[a][i], 0, 0, 0);
+                    acc[a][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[a][u].v, xf.v, acc[a][i], 0, 0, 0);
             }
     };
 
     if (k_begin < k_end) {
+        // x first: loads finish in the order they were issued, and parking x must not wait for W
         fetch_x(k_begin);
         fetch_w(wcur, k_begin);
         park_x(0);
@@ -247,7 +257,7 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const bf16_t* __restrict_
         }
     }
 
-    // acc[a][i][e] is feature m0 + 16 j + 4 g + e (j = a mod R) of token n0 + 16 i + r
+    // acc[a][i][e] is feature 16 (mt0 + j) + 4 g + e (j = a mod R) of token n0 + 16 i + r
     const bool split = gridDim.z > 1;
 #pragma unroll
     for (int j = 0; j < R; ++j)
@@ -256,7 +266,7 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const bf16_t* __restrict_
             const int n = n0 + i * 16 + r;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                const int m = m0 + 16 * j + 4 * g + e;
+                const int m = (mt0 + j) * 16 + 4 * g + e;
                 if (m >= Mout || n >= N) continue;
                 float v = acc[j][i][e];
                 if (SWIGLU) {
@@ -292,19 +302,21 @@ __global__ void sum_partials_kernel(const float* __restrict__ partial, TO* __res
     }
 }
 
-// Any shape (k not a multiple of 8): one thread per output, plain loop.
+// Any shape (k not a multiple of 8, or x not aligned): one thread per output, plain loop over the packed matrix.
+__device__ __forceinline__ float packed_at(const bf16_t* wp, int KT, int m, int k) {
+    return bf16_to_f32(wp[(((size_t)(m >> 4) * KT + (k >> 5)) * 64 + ((k & 31) >> 3) * 16 + (m & 15)) * 8 + (k & 7)]);
+}
 template <bool SWIGLU, typename TO>
-__global__ void gemm_plain_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
-                                  const float* __restrict__ bias, TO* __restrict__ y, int N, int Mout, int K) {
+__global__ void gemm_plain_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wp,
+                                  const float* __restrict__ bias, TO* __restrict__ y, int N, int Mout, int K, int KT,
+                                  int up_tiles) {
     int m = blockIdx.x * blockDim.x + threadIdx.x, n = blockIdx.y;
     if (m >= Mout) return;
     const bf16_t* xr = x + (size_t)n * K;
-    const bf16_t* wr = w + (size_t)m * K;
     float v = 0.f, u = 0.f;
-    for (int k = 0; k < K; ++k) v = fmaf(bf16_to_f32(xr[k]), bf16_to_f32(wr[k]), v);
+    for (int k = 0; k < K; ++k) v = fmaf(bf16_to_f32(xr[k]), packed_at(wp, KT, m, k), v);
     if (SWIGLU) {
-        const bf16_t* wu = w + ((size_t)Mout + m) * K;
-        for (int k = 0; k < K; ++k) u = fmaf(bf16_to_f32(xr[k]), bf16_to_f32(wu[k]), u);
+        for (int k = 0; k < K; ++k) u = fmaf(bf16_to_f32(xr[k]), packed_at(wp, KT, up_tiles * 16 + m, k), u);
         v = v / (1.f + expf(-v)) * u;
     } else if (bias) {
         v += bias[m];
@@ -312,31 +324,11 @@ __global__ void gemm_plain_kernel(const bf16_t* __restrict__ x, const bf16_t* __
     store_f32<TO>(y, (size_t)n * Mout + m, v);
 }
 
-// the partial sums of a block pass through R * (SWIGLU ? 2 : 1) * WPB KB of LDS: at most 32 KB
-template <int NT, int R, int WPB, bool SWIGLU, typename TO>
-static int launch_one(dim3 grid, const bf16_t* x, const bf16_t* w, const float* bias, TO* y, int N, int Mout, int K,
-                      hipStream_t stream) {
-    if constexpr (R * (SWIGLU ? 2 : 1) * WPB <= 32) {
-        gemm_skinny_kernel<NT, R, WPB, SWIGLU, TO><<<grid, WPB * 64, 0, stream>>>(x, w, bias, y, N, Mout, K);
-        return 0;
-    } else {
-        return vt_fail("vt_linear_bf16: no kernel for %d row tiles with %d waves", R, WPB);
-    }
-}
-
-template <int NT, int R, bool SWIGLU, typename TO>
-static int launch_skinny(int wpb, dim3 grid, const bf16_t* x, const bf16_t* w, const float* bias, TO* y, int N,
-                         int Mout, int K, hipStream_t stream) {
-    if (wpb == 4) return launch_one<NT, R, 4, SWIGLU, TO>(grid, x, w, bias, y, N, Mout, K, stream);
-    if (wpb == 8) return launch_one<NT, R, 8, SWIGLU, TO>(grid, x, w, bias, y, N, Mout, K, stream);
-    return launch_one<NT, R, 16, SWIGLU, TO>(grid, x, w, bias, y, N, Mout, K, stream);
-}
-
 // Number of k ranges for the 64-token kernel: from the shape of W only (so the order of additions does not depend
 // on the batch), enough blocks to fill the GPU, every range a multiple of the stage length.
 static int mid_splits(int Mout, int K, int rows_per_block) {
     const int row_blocks = (Mout + rows_per_block - 1) / rows_per_block;
-    const int stages = (K + MID_BK - 1) / MID_BK;
+    const int stages = pk_cols(K) / MID_BK;
     int splits = (512 + row_blocks - 1) / row_blocks;
     if (splits > 16) splits = 16;
     if (splits > stages / 4) splits = stages / 4 > 0 ? stages / 4 : 1;
@@ -351,25 +343,27 @@ extern "C" long long vt_linear_bf16_workspace(int N, int M, int K, int gated) {
 }
 
 template <bool SWIGLU, typename TO>
-static int linear_bf16(const bf16_t* x, const bf16_t* w, const float* bias, TO* y, float* workspace, int N, int Mout,
+static int linear_bf16(const bf16_t* x, const bf16_t* wp, const float* bias, TO* y, float* workspace, int N, int Mout,
                        int K, hipStream_t stream) {
     if (N == 0) return 0;
-    if (K % 8 != 0 || ((uintptr_t)x & 15) || ((uintptr_t)w & 15)) {
+    const int KT = pk_cols(K) / 32, up_tiles = pk_rows(Mout) / 16;
+    VT_REQUIRE((((uintptr_t)wp) & 15) == 0, "vt_linear_bf16: the packed matrix is not 16-byte aligned");
+    if (K % 8 != 0 || ((uintptr_t)x & 15)) {
         VT_REQUIRE(N <= 65535, "vt_linear_bf16: too many rows (%d) for the any-shape kernel", N);
-        gemm_plain_kernel<SWIGLU, TO><<<dim3((Mout + 255) / 256, N), 256, 0, stream>>>(x, w, bias, y, N, Mout, K);
+        gemm_plain_kernel<SWIGLU, TO><<<dim3((Mout + 255) / 256, N), 256, 0, stream>>>(x, wp, bias, y, N, Mout, K, KT, up_tiles);
         VT_CHECK_LAUNCH("vt_linear_bf16(plain)");
         return 0;
     }
     if (N > 16) {
-        // 64 tokens per block through LDS; two row tiles per wave (one for the gated product, which has two
+        // 64 tokens per block through LDS; two tile rows per wave (one for the gated product, which has two
         // matrices' rows per wave already)
         constexpr int RR = SWIGLU ? 1 : 2;
         const int splits = SWIGLU ? 1 : mid_splits(Mout, K, 64 * RR);
         VT_REQUIRE(splits == 1 || workspace, "vt_linear_bf16: this shape needs a workspace (vt_linear_bf16_workspace)");
-        int kps = ((K + splits - 1) / splits + MID_BK - 1) / MID_BK * MID_BK;
+        int kps = ((pk_cols(K) + splits - 1) / splits + MID_BK - 1) / MID_BK * MID_BK;
         dim3 grid((Mout + 64 * RR - 1) / (64 * RR), (N + 63) / 64, splits);
         VT_REQUIRE(grid.y <= 65535, "vt_linear_bf16: too many rows (%d)", N);
-        gemm_mid_kernel<RR, SWIGLU, TO><<<grid, 256, 0, stream>>>(x, w, bias, y, workspace, N, Mout, K, kps);
+        gemm_mid_kernel<RR, SWIGLU, TO><<<grid, 256, 0, stream>>>(x, wp, bias, y, workspace, N, Mout, K, KT, up_tiles, kps);
         VT_CHECK_LAUNCH("vt_linear_bf16(64 tokens)");
         if (splits > 1) {
             const size_t n = (size_t)N * Mout;
@@ -379,30 +373,29 @@ static int linear_bf16(const bf16_t* x, const bf16_t* w, const float* bias, TO* 
         return 0;
     }
     // How k is split over the waves of a block depends on the shape of W only, so that a token's sums are added
-    // in the same order whatever the number of rows.
+    // in the same order whatever the number of rows: 8 waves where there are tile rows enough to fill the GPU
+    // with them, 16 for the smaller matrices.
     const int tiles16 = (Mout + 15) / 16;
-    const int wpb = tiles16 >= 1024 ? 4 : (tiles16 >= 512 ? 8 : 16);
-    dim3 grid(tiles16, 1);
-    int rc = launch_skinny<1, 1, SWIGLU, TO>(wpb, grid, x, w, bias, y, N, Mout, K, stream);
-    if (rc) return rc;
+    if (tiles16 >= 512) gemm_skinny_kernel<8, SWIGLU, TO><<<tiles16, 8 * 64, 0, stream>>>(x, wp, bias, y, N, Mout, K, KT, up_tiles);
+    else gemm_skinny_kernel<16, SWIGLU, TO><<<tiles16, 16 * 64, 0, stream>>>(x, wp, bias, y, N, Mout, K, KT, up_tiles);
     VT_CHECK_LAUNCH("vt_linear_bf16");
     return 0;
 }
 
-// y[N, M] = x[N, K] . W[M, K]^T + bias
-extern "C" int vt_linear_bf16(const void* x, const void* w, const float* bias, void* y, int out_dtype, float* workspace,
+// y[N, M] = x[N, K] . W[M, K]^T + bias; wp = W packed by vt_pack_matrix_bf16
+extern "C" int vt_linear_bf16(const void* x, const void* wp, const float* bias, void* y, int out_dtype, float* workspace,
                               int N, int M, int K, hipStream_t stream) {
     VT_REQUIRE(N >= 0 && M > 0 && K > 0, "vt_linear_bf16: bad sizes N=%d M=%d K=%d", N, M, K);
-    if (out_dtype == VT_F32) return linear_bf16<false, float>((const bf16_t*)x, (const bf16_t*)w, bias, (float*)y, workspace, N, M, K, stream);
-    if (out_dtype == VT_BF16) return linear_bf16<false, bf16_t>((const bf16_t*)x, (const bf16_t*)w, bias, (bf16_t*)y, workspace, N, M, K, stream);
+    if (out_dtype == VT_F32) return linear_bf16<false, float>((const bf16_t*)x, (const bf16_t*)wp, bias, (float*)y, workspace, N, M, K, stream);
+    if (out_dtype == VT_BF16) return linear_bf16<false, bf16_t>((const bf16_t*)x, (const bf16_t*)wp, bias, (bf16_t*)y, workspace, N, M, K, stream);
     return vt_fail("vt_linear_bf16: unknown out dtype %d", out_dtype);
 }
 
-// y[N, I] = silu(x . Wg^T) * (x . Wu^T),  W = [Wg; Wu] of shape [2 I, K]
-extern "C" int vt_gated_linear_bf16(const void* x, const void* w, void* y, int out_dtype, int N, int I, int K,
+// y[N, I] = silu(x . Wg^T) * (x . Wu^T); wp = Wg [I, K] packed, followed by Wu [I, K] packed
+extern "C" int vt_gated_linear_bf16(const void* x, const void* wp, void* y, int out_dtype, int N, int I, int K,
                                     hipStream_t stream) {
     VT_REQUIRE(N >= 0 && I > 0 && K > 0, "vt_gated_linear_bf16: bad sizes N=%d I=%d K=%d", N, I, K);
-    if (out_dtype == VT_F32) return linear_bf16<true, float>((const bf16_t*)x, (const bf16_t*)w, nullptr, (float*)y, nullptr, N, I, K, stream);
-    if (out_dtype == VT_BF16) return linear_bf16<true, bf16_t>((const bf16_t*)x, (const bf16_t*)w, nullptr, (bf16_t*)y, nullptr, N, I, K, stream);
+    if (out_dtype == VT_F32) return linear_bf16<true, float>((const bf16_t*)x, (const bf16_t*)wp, nullptr, (float*)y, nullptr, N, I, K, stream);
+    if (out_dtype == VT_BF16) return linear_bf16<true, bf16_t>((const bf16_t*)x, (const bf16_t*)wp, nullptr, (bf16_t*)y, nullptr, N, I, K, stream);
     return vt_fail("vt_gated_linear_bf16: unknown out dtype %d", out_dtype);
 }

@@ -175,6 +175,41 @@ def linear_f32(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], o
     return out
 
 
+class PackedMatrix:
+    """W [rows, cols] in bfloat16 in the order the matrix instruction reads it (vt_gemm_bf16.hip): tiles of
+    16 rows x 32 columns, each stored as the 64 lanes' fragments; rows padded to 16 and columns to 128 by zeros.
+    `halves` = 2: two matrices of `rows` rows each, packed one after the other (gate, then up)."""
+
+    __slots__ = ("data", "rows", "cols", "halves")
+
+    def __init__(self, data: torch.Tensor, rows: int, cols: int, halves: int = 1):
+        self.data, self.rows, self.cols, self.halves = data, int(rows), int(cols), int(halves)
+
+    def first_rows(self, n: int) -> "PackedMatrix":
+        """The matrix of the first n rows (a multiple of 16): the packed rows of tiles are contiguous."""
+        if self.halves != 1 or n % 16 or not 0 < n <= self.rows:
+            raise KernelError(f"cannot take the first {n} rows of a packed matrix of {self.rows}")
+        per_tile_row = self.data.numel() // ((self.rows + 15) // 16)
+        return PackedMatrix(self.data[:(n // 16) * per_tile_row], n, self.cols)
+
+
+def pack_matrix_bf16(w: torch.Tensor, halves: int = 1) -> PackedMatrix:
+    """Pack W [rows, cols] (halves = 2: [2 * rows, cols], the two matrices stacked) for linear_bf16 /
+    gated_linear_bf16."""
+    _chk(w, "pack_matrix_bf16.w", torch.bfloat16)
+    if w.dim() != 2 or w.shape[0] % halves:
+        raise KernelError(f"pack_matrix_bf16: shape {tuple(w.shape)} is not {halves} stacked matrices")
+    rows, cols = w.shape[0] // halves, w.shape[1]
+    lib = load_lib("vt_gemm_bf16")
+    lib.vt_packed_elems.restype = ctypes.c_longlong
+    per = int(lib.vt_packed_elems(_i(rows), _i(cols)))
+    data = torch.empty(halves * per, dtype=torch.bfloat16, device=w.device)
+    for h in range(halves):
+        _run(lib, "vt_pack_matrix_bf16", _ptr(w[h * rows:(h + 1) * rows]), _ptr(data[h * per:(h + 1) * per]), _i(rows),
+             _i(cols), _stream())
+    return PackedMatrix(data, rows, cols, halves)
+
+
 def linear_bf16_workspace(n: int, m: int, k: int) -> int:
     """Floats of scratch memory that linear_bf16 needs for x [n, k], W [m, k] (0: none)."""
     lib = load_lib("vt_gemm_bf16")
@@ -182,14 +217,20 @@ def linear_bf16_workspace(n: int, m: int, k: int) -> int:
     return int(lib.vt_linear_bf16_workspace(_i(n), _i(m), _i(k), _i(0)))
 
 
-def linear_bf16(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
+def linear_bf16(x: torch.Tensor, w, bias: Optional[torch.Tensor], out: torch.Tensor,
                 workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Few rows (decoding, short portions): W is read once per 64 rows.  Shapes whose k range is split over blocks
-    need `workspace` (float32, at least linear_bf16_workspace(n, m, k) elements)."""
+    """Few rows (decoding, short portions): W is read once per 64 rows.  w: a PackedMatrix (a plain [m, k] tensor
+    is packed on the spot, which costs more than the product).  Shapes whose k range is split over blocks need
+    `workspace` (float32, at least linear_bf16_workspace(n, m, k) elements)."""
     n, k = x.shape
-    m = w.shape[0]
+    if not isinstance(w, PackedMatrix):
+        _chk(w, "linear_bf16.w", torch.bfloat16, (w.shape[0], k))
+        w = pack_matrix_bf16(w)
+    m = w.rows
+    if w.cols != k or w.halves != 1:
+        raise KernelError(f"linear_bf16: x [{n}, {k}] does not fit a packed matrix [{w.rows}, {w.cols}] x {w.halves}")
     _chk(x, "linear_bf16.x", torch.bfloat16)
-    _chk(w, "linear_bf16.w", torch.bfloat16, (m, k))
+    _chk(w.data, "linear_bf16.w", torch.bfloat16)
     _chk(out, "linear_bf16.out", None, (n, m))
     if bias is not None:
         _chk(bias, "linear_bf16.bias", torch.float32, (m,))
@@ -200,19 +241,26 @@ def linear_bf16(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], 
         _chk(workspace, "linear_bf16.workspace", torch.float32)
         if workspace.numel() < need:
             raise KernelError(f"linear_bf16: workspace of {workspace.numel()} floats, need {need}")
-    _run(load_lib("vt_gemm_bf16"), "vt_linear_bf16", _ptr(x), _ptr(w), _ptr(bias), _ptr(out), _i(_code(out)),
+    _run(load_lib("vt_gemm_bf16"), "vt_linear_bf16", _ptr(x), _ptr(w.data), _ptr(bias), _ptr(out), _i(_code(out)),
          _ptr(workspace if need else None), _i(n), _i(m), _i(k), _stream())
     return out
 
 
-def gated_linear_bf16(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+def gated_linear_bf16(x: torch.Tensor, w_gate_up, out: torch.Tensor) -> torch.Tensor:
+    """out = silu(x Wg^T) * (x Wu^T).  w_gate_up: a PackedMatrix of two halves (pack_matrix_bf16(w, halves=2)), or
+    the stacked [2 I, k] tensor, which is packed on the spot."""
     n, k = x.shape
-    two_i = w_gate_up.shape[0]
+    if not isinstance(w_gate_up, PackedMatrix):
+        _chk(w_gate_up, "gated_linear_bf16.w", torch.bfloat16, (w_gate_up.shape[0], k))
+        w_gate_up = pack_matrix_bf16(w_gate_up, halves=2)
+    w = w_gate_up
+    if w.cols != k or w.halves != 2:
+        raise KernelError(f"gated_linear_bf16: x [{n}, {k}] does not fit a packed matrix [{w.rows}, {w.cols}] x {w.halves}")
     _chk(x, "gated_linear_bf16.x", torch.bfloat16)
-    _chk(w_gate_up, "gated_linear_bf16.w", torch.bfloat16, (two_i, k))
-    _chk(out, "gated_linear_bf16.out", None, (n, two_i // 2))
-    _run(load_lib("vt_gemm_bf16"), "vt_gated_linear_bf16", _ptr(x), _ptr(w_gate_up), _ptr(out), _i(_code(out)), _i(n),
-         _i(two_i // 2), _i(k), _stream())
+    _chk(w.data, "gated_linear_bf16.w", torch.bfloat16)
+    _chk(out, "gated_linear_bf16.out", None, (n, w.rows))
+    _run(load_lib("vt_gemm_bf16"), "vt_gated_linear_bf16", _ptr(x), _ptr(w.data), _ptr(out), _i(_code(out)), _i(n),
+         _i(w.rows), _i(k), _stream())
     return out
 
 

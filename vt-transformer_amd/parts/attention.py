@@ -54,7 +54,7 @@ class PagedAttention(Part):
         if key not in shared:
             shared[key] = POSITIONS.build(pos_spec, rt=rt)
         self.position = shared[key]
-        self.w_qkv = self.b_qkv = self.b_qkv_lowp = self.w_o = self.b_o = None
+        self.w_qkv = self.b_qkv = self.b_qkv_lowp = self.w_o = self.b_o = self.p_qkv = self.p_o = None
 
     # -- what the cache manager must hold for this mixer --------------------
     def cache_need(self) -> Optional[CacheNeed]:
@@ -89,6 +89,7 @@ class PagedAttention(Part):
         self.w_o = rt.place(get(nm["o"] + ".weight"), "matrix")
         if self.out_bias:
             self.b_o = rt.place(get(nm["o"] + ".bias"), "bias")
+        self.p_qkv, self.p_o = rt.pack(self.w_qkv), rt.pack(self.w_o)
 
     # -- one step --------------------------------------------------------------
     def forward(self, x: torch.Tensor, ctx, cache, state=None) -> torch.Tensor:
@@ -96,11 +97,12 @@ class PagedAttention(Part):
         n = x.shape[0]
         nq = nh * d
         if cache.writes:
-            qkv = linear(rt, x, self.w_qkv, self.b_qkv, "attn.qkv", bias_lowp=self.b_qkv_lowp)
+            qkv = linear(rt, x, self.w_qkv, self.b_qkv, "attn.qkv", bias_lowp=self.b_qkv_lowp, packed=self.p_qkv)
         else:  # keys and values of another layer: only queries are made
             bq = self.b_qkv[:nq] if self.b_qkv is not None else None
             bql = self.b_qkv_lowp[:nq] if self.b_qkv_lowp is not None else None
-            qkv = linear(rt, x, self.w_qkv[:nq], bq, "attn.qonly", bias_lowp=bql)
+            qkv = linear(rt, x, self.w_qkv[:nq], bq, "attn.qonly", bias_lowp=bql,
+                         packed=self.p_qkv.first_rows(nq) if self.p_qkv is not None else None)
         tables = self.position.rotary_tables(ctx.n_positions)
         if tables is None and hasattr(self.position, "apply") and self.position.dim != 0:
             # a position encoding that is not a plain rotation: let it rewrite queries and keys, then store unrotated
@@ -123,7 +125,7 @@ class PagedAttention(Part):
             ops.attention_bf16_decode_fused(qkv, cos, sin, cache.k, cache.v, cache.block_table, ctx.entry_pos0,
                                             ctx.decode_params[b:b + 1], ctx.decode_p_max, out, part_o, part_ml, nh, nkv, d,
                                             self.window, self.scale)
-            return linear(rt, out, self.w_o, self.b_o, "attn.o")
+            return linear(rt, out, self.w_o, self.b_o, "attn.o", packed=self.p_o)
         q = rt.buffer("attn.q", (n, nq), rt.dtype)
         ops.rope_store(qkv, cos, sin, ctx.positions, ctx.tok_entry, cache.block_table, q, cache.k, cache.v, nh, nkv, d,
                        write_kv=cache.writes)
@@ -147,4 +149,4 @@ class PagedAttention(Part):
             if plan.n_tile_items:   # long portions: key/value blocks through LDS, shared by four waves
                 ops.attention_bf16_tiles(q, cache.k, cache.v, cache.block_table, plan.tile_items, plan.n_tile_items,
                                          out, nh, nkv, d, self.window, self.scale, rt=plan.tile_rt)
-        return linear(rt, out, self.w_o, self.b_o, "attn.o")
+        return linear(rt, out, self.w_o, self.b_o, "attn.o", packed=self.p_o)

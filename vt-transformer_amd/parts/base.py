@@ -91,6 +91,14 @@ class Runtime:
             return t.to(device=self.device, dtype=torch.int32).contiguous()
         raise ValueError(f"unknown tensor role {role!r}")
 
+    def pack(self, w: torch.Tensor, halves: int = 1):
+        """The bfloat16 matrix once more in the order the few-row matrix kernels read it (None in float32).  The
+        row-major matrix stays for the GEMM library, which long portions go through."""
+        if self.dtype != torch.bfloat16:
+            return None
+        from ..kernels import ops
+        return ops.pack_matrix_bf16(w, halves)
+
     def buffer(self, name: str, shape, dtype: torch.dtype) -> torch.Tensor:
         """A scratch tensor that keeps its address between steps (grown when a step needs more)."""
         n = 1

@@ -39,6 +39,7 @@ class LinearHead(Part):
     def __init__(self, *, rt: Runtime, width: int, vocab_size: int, name: str, tied_to: Optional[str] = None):
         self.rt, self.width, self.vocab, self.name, self.tied_to = rt, int(width), int(vocab_size), name, tied_to
         self.weight: Optional[torch.Tensor] = None
+        self.packed = None
 
     def tensors(self) -> Dict[str, TensorDecl]:
         if self.tied_to:
@@ -53,6 +54,9 @@ class LinearHead(Part):
             self.weight = shared[self.tied_to]
         else:
             self.weight = rt.place(get(self.name), "matrix")
+        self.packed = rt.pack(self.weight)
+        if self.packed is not None and not self.tied_to:
+            self.weight = None      # bfloat16 logits always come from the packed matrix
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         """x [R, H] (normed rows) -> fp32 logits [R, V]."""
@@ -64,5 +68,5 @@ class LinearHead(Part):
             r1 = min(r, r0 + SKINNY_MAX_ROWS)
             need = ops.linear_bf16_workspace(r1 - r0, self.vocab, self.width) if r1 - r0 > 16 else 0
             work = self.rt.buffer("linear.partials", (need,), torch.float32) if need else None
-            ops.linear_bf16(x[r0:r1], self.weight, None, out[r0:r1], work)
+            ops.linear_bf16(x[r0:r1], self.packed, None, out[r0:r1], work)
         return out

@@ -31,7 +31,7 @@ class GatedMLP(Part):
         n = {"gate": "gate_proj", "up": "up_proj", "down": "down_proj"}
         n.update(names or {})
         self.names = {k: prefix + v for k, v in n.items()}
-        self.w_gu = self.w_down = None
+        self.w_gu = self.w_down = self.p_gu = self.p_down = None
 
     def tensors(self) -> Dict[str, TensorDecl]:
         nm = self.names
@@ -46,14 +46,15 @@ class GatedMLP(Part):
         self.w_gu = torch.cat([rt.place(get(nm["gate"] + ".weight"), "matrix"),
                                rt.place(get(nm["up"] + ".weight"), "matrix")], dim=0).contiguous()
         self.w_down = rt.place(get(nm["down"] + ".weight"), "matrix")
+        self.p_gu, self.p_down = rt.pack(self.w_gu, halves=2), rt.pack(self.w_down)
 
     def forward(self, x: torch.Tensor, ctx=None) -> torch.Tensor:
         rt = self.rt
         n = x.shape[0]
         act = rt.buffer("mlp.act", (n, self.inter), rt.dtype)
         if rt.dtype == torch.bfloat16 and n <= SKINNY_MAX_ROWS:
-            ops.gated_linear_bf16(x, self.w_gu, act)
+            ops.gated_linear_bf16(x, self.p_gu if self.p_gu is not None else self.w_gu, act)
         else:
             gu = linear(rt, x, self.w_gu, None, "mlp.gu")
             ops.silu_mul(gu, act)
-        return linear(rt, act, self.w_down, None, "mlp.down")
+        return linear(rt, act, self.w_down, None, "mlp.down", packed=self.p_down)

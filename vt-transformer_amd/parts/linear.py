@@ -4,8 +4,9 @@ v1/tensortype/tensortype.cpp:222-229).
 
 float32: the hand-written fp32 kernel, always (no matrix-core mode).
 bfloat16: the hand-written matrix-core kernel while the rows are few enough
-that reading W dominates; above that the GEMM library, which is where the
-reference's engine uses a library too (hipblasGemmEx, hip_tensor.cpp:514-535).
+that reading W dominates, on a copy of W in the matrix instruction's own order;
+above that the GEMM library on the row-major W, which is where the reference's
+engine uses a library too (hipblasGemmEx, hip_tensor.cpp:514-535).
 """
 from __future__ import annotations
 
@@ -21,10 +22,12 @@ SKINNY_MAX_ROWS = 64
 
 
 def linear(rt: Runtime, x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], name: str,
-           out_dtype: Optional[torch.dtype] = None, bias_lowp: Optional[torch.Tensor] = None) -> torch.Tensor:
+           out_dtype: Optional[torch.dtype] = None, bias_lowp: Optional[torch.Tensor] = None,
+           packed=None) -> torch.Tensor:
     """x [N, K] in the runtime's dtype -> [N, M].  `name` keys the output's scratch buffer.
     Output dtype: float32 from the hand-written kernels unless `out_dtype` says otherwise; the
-    library path returns bfloat16 (its bias, if any, is `bias_lowp`, the same values in bfloat16)."""
+    library path returns bfloat16 (its bias, if any, is `bias_lowp`, the same values in bfloat16).
+    packed: W as rt.pack(w) made it, for the few-row kernel (made on the spot if missing: slow)."""
     n, k = x.shape
     m = w.shape[0]
     if rt.dtype == torch.float32:
@@ -34,7 +37,7 @@ def linear(rt: Runtime, x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.T
         out = rt.buffer(name, (n, m), out_dtype or torch.float32)
         need = ops.linear_bf16_workspace(n, m, k) if n > 16 else 0
         work = rt.buffer("linear.partials", (need,), torch.float32) if need else None
-        return ops.linear_bf16(x, w, bias, out, work)
+        return ops.linear_bf16(x, packed if packed is not None else w, bias, out, work)
     out = rt.buffer(name + ".lib", (n, m), torch.bfloat16)
     if bias is not None:
         if bias_lowp is None:
