@@ -76,6 +76,14 @@ extern "C" int vt_pack_matrix_bf16(const void* w, void* wp, int M, int K, hipStr
     return 0;
 }
 
+// Between a wave's writes to its own LDS buffer and its reads of what other lanes wrote: the LDS executes a wave's
+// operations in order, so all this has to do is to keep the compiler from moving the reads up.
+__device__ __forceinline__ void wave_lds_order() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 // x[row][k .. k + 8); beyond the end of the row its last eight values are read instead (W is zero there)
 __device__ __forceinline__ bf16x8_t load_x(const bf16_t* row, int k, int K) {
     Frag f;
@@ -85,8 +93,14 @@ __device__ __forceinline__ bf16x8_t load_x(const bf16_t* row, int k, int K) {
 
 // ---------------------------------------------------------------------------
 // Up to 16 tokens: a block owns one tile row of W (16 features; two for the gated product) and all of k, which
-// its WPB waves split; the tokens are the B operand, read from x as it lies in memory.  U tiles are in flight
-// per wave and matrix.
+// its WPB waves split; the tokens are the B operand.  U tiles are in flight per wave and matrix.
+//
+// The B fragment of a tile is 64 bytes of each of 16 token rows.  Read as the matrix instruction wants it (lane
+// 16 g + r: row r, piece g) the four pieces of a row sit in lanes 16 apart and the cache sees 64 separate
+// accesses; so lane l reads piece l % 4 of row l / 4 instead (the four lanes of a row are neighbours, 16 accesses
+// of 64 bytes) and hands it through LDS to the lane that needs it.  The slots of a piece index are 17 apart, which
+// keeps writes and reads off each other's banks; each wave has two such buffers of its own and no one else's, so
+// nothing but the order of its own LDS operations keeps them consistent.
 // ---------------------------------------------------------------------------
 template <int WPB, bool SWIGLU, typename TO>
 __global__ __launch_bounds__(WPB * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wp,
@@ -95,6 +109,7 @@ __global__ __launch_bounds__(WPB * 64) void gemm_skinny_kernel(const bf16_t* __r
     constexpr int NW = SWIGLU ? 2 : 1;
     constexpr int U = 4;
     __shared__ float red[NW][WPB][256];
+    __shared__ uint4 xt[WPB][2][4 * 17];
     const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63;
     const int r = lane & 15, g = lane >> 4;
     const int mt = blockIdx.x;
@@ -102,33 +117,46 @@ __global__ __launch_bounds__(WPB * 64) void gemm_skinny_kernel(const bf16_t* __r
     const bf16_t* wbase[NW];
     wbase[0] = wp + ((size_t)mt * KT * 64 + lane) * 8;
     if (SWIGLU) wbase[1] = wp + ((size_t)(mt + up_tiles) * KT * 64 + lane) * 8;
-    const bf16_t* xrow = x + (size_t)min(r, N - 1) * K;
+    const bf16_t* xrow = x + (size_t)min(lane >> 2, N - 1) * K;
+    const int xpiece = (lane & 3) * 8;
+    const int wslot = (lane & 3) * 17 + (lane >> 2), rslot = g * 17 + r;
     f32x4_t acc[NW];
 #pragma unroll
     for (int a = 0; a < NW; ++a) acc[a] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
     int t = t_begin;
     for (; t + U <= t_end; t += U) {
-        Frag wa[NW][U];
-        bf16x8_t xa[U];
+        Frag wa[NW][U], xa[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
 #pragma unroll
             for (int a = 0; a < NW; ++a) wa[a][u].u = *(const uint4*)(wbase[a] + (size_t)(t + u) * PK_TILE);
-            xa[u] = load_x(xrow, (t + u) * 32 + g * 8, K);
+            xa[u].v = load_x(xrow, (t + u) * 32 + xpiece, K);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            xt[wv][u & 1][wslot] = xa[u].u;
+            wave_lds_order();
+            xa[u].u = xt[wv][u & 1][rslot];
+            wave_lds_order();       // and the next write to this buffer after these reads
         }
 #pragma unroll
         for (int u = 0; u < U; ++u)
 #pragma unroll
             for (int a = 0; a < NW; ++a)
-                acc[a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[a][u].v, xa[u], acc[a], 0, 0, 0);
+                acc[a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[a][u].v, xa[u].v, acc[a], 0, 0, 0);
     }
     for (; t < t_end; ++t) {
-        const bf16x8_t xa = load_x(xrow, t * 32 + g * 8, K);
+        Frag xa;
+        xa.v = load_x(xrow, t * 32 + xpiece, K);
+        xt[wv][0][wslot] = xa.u;
+        wave_lds_order();
+        xa.u = xt[wv][0][rslot];
+        wave_lds_order();
 #pragma unroll
         for (int a = 0; a < NW; ++a) {
             Frag wa;
             wa.u = *(const uint4*)(wbase[a] + (size_t)t * PK_TILE);
-            acc[a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa.v, xa, acc[a], 0, 0, 0);
+            acc[a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa.v, xa.v, acc[a], 0, 0, 0);
         }
     }
     // acc[a][e] is feature 16 mt + 4 g + e of token r.  Sum the waves in wave order.
@@ -373,10 +401,9 @@ static int linear_bf16(const bf16_t* x, const bf16_t* wp, const float* bias, TO*
         return 0;
     }
     // How k is split over the waves of a block depends on the shape of W only, so that a token's sums are added
-    // in the same order whatever the number of rows: 8 waves where there are tile rows enough to fill the GPU
-    // with them, 16 for the smaller matrices.
+    // in the same order whatever the number of rows: 8 waves, 16 for matrices with few rows and a long k.
     const int tiles16 = (Mout + 15) / 16;
-    if (tiles16 >= 512) gemm_skinny_kernel<8, SWIGLU, TO><<<tiles16, 8 * 64, 0, stream>>>(x, wp, bias, y, N, Mout, K, KT, up_tiles);
+    if (tiles16 >= 512 || KT < 256) gemm_skinny_kernel<8, SWIGLU, TO><<<tiles16, 8 * 64, 0, stream>>>(x, wp, bias, y, N, Mout, K, KT, up_tiles);
     else gemm_skinny_kernel<16, SWIGLU, TO><<<tiles16, 16 * 64, 0, stream>>>(x, wp, bias, y, N, Mout, K, KT, up_tiles);
     VT_CHECK_LAUNCH("vt_linear_bf16");
     return 0;
