@@ -89,6 +89,10 @@ class CacheStorage:
     def n_groups(self) -> int:
         return len(self.group_needs)
 
+    def group_window(self, g: int) -> int:
+        """The window of group g's layers (0: they keep every key)."""
+        return int(self.group_needs[g].window)
+
     def bytes_per_token(self) -> int:
         item = torch.empty((), dtype=self.rt.dtype).element_size()
         return sum(2 * k.shape[0] * k.shape[2] * k.shape[4] * item for k in self.k)

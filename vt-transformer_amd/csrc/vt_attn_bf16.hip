@@ -35,6 +35,9 @@ VT_DEFINE_LAST_ERROR()
 static_assert(VT_HEAD_DIM % 16 == 0 && VT_HEAD_DIM >= 16 && VT_HEAD_DIM <= 256, "head size must be 16..256 in steps of 16");
 
 #define D VT_HEAD_DIM
+#ifndef VT_ATTN_RING
+#define VT_ATTN_RING 2          // key/value blocks of 16 keys in registers per wave: one multiplied, the others in flight
+#endif
 #define ITEM_INTS 8  // entry, q_tok0, q_len, pos0, q_row0, key_lo, key_hi, part (-1: final)
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
@@ -154,14 +157,17 @@ struct KVBlock {
     bool ok;
 };
 
-// `pg` is the page of the block (read from the block table ahead of time, so that the loads below do not wait for it)
-__device__ __forceinline__ void load_block(KVBlock& b, const AttnArgs& a, int pg, int j0, int kvh, int r, int g) {
+// `pg` is the page of the block (read from the block table ahead of time, so that the loads below do not wait for
+// it).  Nothing is tested before the loads: a block without a page (a window has passed it: its keys are masked for
+// every row) reads `spare`, a page that exists, and is marked so that it is not multiplied.  Loads under a branch
+// would make every later use wait for all the loads in flight.
+__device__ __forceinline__ void load_block(KVBlock& b, const AttnArgs& a, int pg, int spare, int j0, int kvh, int r, int g) {
     const int ps = a.page_size;
     const int blk = page_index(a, j0);
-    b.ok = pg >= 0 && pg < a.num_pages;   // a page the window has passed: its keys are masked for every row
-    if (!b.ok) return;
+    b.ok = pg >= 0 && pg < a.num_pages;
+    const int pgc = b.ok ? pg : spare;
     const int off = j0 - blk * ps;
-    const bf16_t* kb = a.k_pages + (((size_t)pg * a.n_kv + kvh) * ps + off + r) * D;
+    const bf16_t* kb = a.k_pages + (((size_t)pgc * a.n_kv + kvh) * ps + off + r) * D;
     if constexpr (WIDE) {
 #pragma unroll
         for (int st = 0; st < QSTEPS; ++st) b.k8[st] = *(const uint4*)(kb + st * 32 + g * 8);
@@ -169,7 +175,7 @@ __device__ __forceinline__ void load_block(KVBlock& b, const AttnArgs& a, int pg
 #pragma unroll
         for (int st = 0; st < QSTEPS; ++st) b.k4[st] = *(const uint2*)(kb + st * 16 + g * 4);
     }
-    const bf16_t* vb = a.v_pages + (((size_t)pg * a.n_kv + kvh) * D + r) * ps + off + 4 * g;
+    const bf16_t* vb = a.v_pages + (((size_t)pgc * a.n_kv + kvh) * D + r) * ps + off + 4 * g;
 #pragma unroll
     for (int t = 0; t < DT; ++t) b.v[t] = *(const uint2*)(vb + (size_t)t * 16 * ps);
 }
@@ -249,7 +255,9 @@ __device__ __forceinline__ void merge_parts(float (*sm)[16], float (*sl)[16], co
 // RT row tiles of 16 rows per wave share every key/value block they read.
 template <bool DECODE, int RT>
 __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_kernel(AttnArgs a) {
-    const int wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    // the wave's index as a scalar: its item and everything read from it then stay in scalar registers, and the
+    // tests on them are scalar branches
+    const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     // decoding: the four waves of a block share one item and take its key blocks in turn; otherwise one item per wave
     const int item = DECODE ? (int)blockIdx.x : (int)blockIdx.x * 4 + wv;
     if (item >= a.n_items) return;
@@ -364,23 +372,11 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_kernel(AttnArg
         __syncthreads();
     }
 
-    // Page ids of up to 64 pages at a time, one per lane: reading the table is then off the path of every block's
-    // loads.  (The lane index of a read is the same for the whole wave.)
     const int* bt = a.block_table + (size_t)entry * a.max_blocks;
     const int ps = a.page_size;
     const int last_page = (key_hi - 1) / ps;
-    int cache_base = key_lo / ps;
-    int pg_lane = (cache_base + lane <= last_page) ? bt[cache_base + lane] : -1;
-    auto page_of = [&](int j) {
-        int blk = page_index(a, j);
-        if (blk >= cache_base + 64) {
-            cache_base = blk;
-            pg_lane = (cache_base + lane <= last_page) ? bt[cache_base + lane] : -1;
-        }
-        return __builtin_amdgcn_readlane(pg_lane, __builtin_amdgcn_readfirstlane(blk - cache_base));
-    };
     // one block of 16 keys against the RT row tiles of this wave
-    auto multiply = [&](const KVBlock& cur, int j0) {
+    auto multiply = [&](const KVBlock& cur, int j0) __attribute__((always_inline)) {
         if (!cur.ok) return;
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
@@ -417,17 +413,35 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_kernel(AttnArg
             }
         }
     };
-    // Two register buffers in turn: while one block is multiplied the other one is on its way from memory.
-    KVBlock ba, bb;
-    ba.ok = bb.ok = false;
+    // A ring of register buffers: while one block is multiplied the next NB - 1 are on their way from memory, and
+    // the page id of the one after them comes from the block table (a scalar load).  Every turn loads, whether or
+    // not keys are left (then the wave's last block again, which nobody multiplies), so that the number of loads
+    // in flight is the same on every path through the loop.
+    constexpr int NB = VT_ATTN_RING;
+    KVBlock ring[NB];
     const int j_first = key_lo + (DECODE ? 16 * wv : 0), j_step = DECODE ? 64 : 16;
-    if (j_first < key_hi) load_block(ba, a, page_of(j_first), j_first, kvh, r, g);
-    for (int j0 = j_first; j0 < key_hi; j0 += 2 * j_step) {
-        const int j1 = j0 + j_step, j2 = j0 + 2 * j_step;
-        if (j1 < key_hi) load_block(bb, a, page_of(j1), j1, kvh, r, g);
-        multiply(ba, j0);
-        if (j2 < key_hi) load_block(ba, a, page_of(j2), j2, kvh, r, g);
-        if (j1 < key_hi) multiply(bb, j1);
+    // the last block this wave may read: the last one of its own, or for a wave without keys the item's first
+    const int j_end = j_first < key_hi ? j_first + (key_hi - 1 - j_first) / j_step * j_step : key_lo;
+    // (read through the constant address space: the kernel writes pages and results but never the block table,
+    // and only so is this a scalar load, which neither counts among the vector loads in flight nor waits for them)
+    typedef const __attribute__((address_space(4))) int* const_int_ptr;
+    const const_int_ptr btc = (const_int_ptr)(uintptr_t)bt;
+    auto page_at = [&](int j) __attribute__((always_inline)) { return btc[min(page_index(a, min(j, j_end)), last_page)]; };
+    const int spare = min(max(btc[last_page], 0), a.num_pages - 1);
+    int pg_next;                     // page of the next block to load
+#pragma unroll
+    for (int i = 0; i < NB - 1; ++i) load_block(ring[i], a, page_at(j_first + i * j_step), spare, min(j_first + i * j_step, j_end), kvh, r, g);
+    pg_next = page_at(j_first + (NB - 1) * j_step);
+    for (int j0 = j_first; j0 < key_hi; j0 += NB * j_step) {
+#pragma unroll
+        for (int ph = 0; ph < NB; ++ph) {
+            const int j = j0 + ph * j_step;
+            if (j >= key_hi) break;
+            load_block(ring[(ph + NB - 1) % NB], a, pg_next, spare, min(j + (NB - 1) * j_step, j_end), kvh, r, g);
+            pg_next = page_at(j + NB * j_step);
+            __builtin_amdgcn_sched_barrier(0);      // the loads stay here, ahead of this block's products
+            multiply(ring[ph], j);
+        }
     }
 
     if constexpr (DECODE) {

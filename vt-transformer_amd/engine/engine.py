@@ -118,7 +118,7 @@ class Engine:
         if plan:
             entries = []
             for s in plan:
-                toks = s.request.tokens[s.start:s.start + s.n_tokens]
+                toks = s.request.token_slice(s.start, s.n_tokens)
                 entries.append(StepEntry(s.request.uid, toks, [s.n_tokens - 1] if s.sample else []))
             logits = self.runner.step(entries)
             rows = [(s.request.params, s.request.seed, len(s.request.output)) for s in plan if s.sample]

@@ -64,6 +64,15 @@ class Request:
     def tokens(self) -> List[int]:
         return self.prompt + self.output
 
+    def token_slice(self, start: int, n: int) -> List[int]:
+        """tokens[start:start + n] without building the whole list (a decoding step asks for the last one)."""
+        np_ = len(self.prompt)
+        if start >= np_:
+            return self.output[start - np_:start - np_ + n]
+        if start + n <= np_:
+            return self.prompt[start:start + n]
+        return self.prompt[start:] + self.output[:start + n - np_]
+
     @property
     def total_len(self) -> int:
         return len(self.prompt) + len(self.output)

@@ -260,7 +260,13 @@ class _DecodeGraph:
         self.ctx: Optional[StepContext] = None
         self.meta: Optional[torch.Tensor] = None
         self.logits: Optional[torch.Tensor] = None
-        self.layout = None
+        # what the next step through this graph needs to patch the metadata instead of building it anew
+        self.rids = None            # the requests of the last step, in order
+        self.h = None               # its host arrays
+        self.flat = None            # its metadata as one int32 array
+        self.table_lens = None      # per group and entry, the block-table entries already written
+        self.wants = None
+        self.wanted = None          # the view of `logits` that the last step returned
 
 
 GRAPH_BATCHES = (1, 2, 4, 8, 16, 32, 64)
@@ -359,10 +365,13 @@ class ModelRunner:
         if dev.numel() != flat.size:
             raise RuntimeError("step metadata does not fit its device buffer")
         self._staging.upload(flat, dev)
-        views, off = [], 0
+        self._last_flat = flat
+        views, off, offs = [], 0, []
         for p in parts:
             views.append(dev[off:off + p.size])
+            offs.append(off)
             off += p.size
+        ctx.part_offsets = dict(ids=offs[0], positions=offs[1], pos0=offs[4], dec=offs[7], tables=offs[8:])
         (ctx.token_ids, ctx.positions, ctx.tok_entry, ctx.entry_start, ctx.entry_pos0, ctx.state_slots,
          ctx.logit_rows) = views[:7]
         ctx.decode_params = views[7] if decode else None
@@ -412,10 +421,14 @@ class ModelRunner:
     def _step_decode_graph(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
         n = len(entries)
         b = next(x for x in GRAPH_BATCHES if x >= n)
+        g = self._graphs.get(b)
+        rids = tuple(e.rid for e in entries)
+        if g is not None and g.rids == rids and self._advance_decode_meta(g, entries):
+            g.graph.replay()        # the same requests as in the last step, one token further: the metadata was patched
+            return g.wanted
         fixed_blocks = -(-self.max_seq_len // self.cache.page_size)
         h = self._host_arrays(entries, pad_to=b, fixed_blocks=fixed_blocks)
         all_rows = np.arange(b, dtype=np.int32)     # logits of every entry; the wanted ones are picked afterwards
-        g = self._graphs.get(b)
         with self.rt.scoped(f"graph{b}:"):
             if g is None:
                 g = _DecodeGraph()
@@ -433,8 +446,58 @@ class ModelRunner:
             else:
                 self._fill_context(g.ctx, h, all_rows, g.meta, decode=True)
             g.graph.replay()
+        # what the next step can patch instead of building anew: the host copy of the metadata and where its parts lie
+        g.rids, g.h, g.flat = rids, h, self._last_flat
+        g.table_lens = [[len(self.cache.get(e.rid).tables[gi]) for e in entries] for gi in range(self.storage.n_groups)]
+        g.wants = [tuple(e.want) for e in entries]
         if len(h["rows"]) == 0:
-            return None
-        if (h["rows"] == all_rows[:len(h["rows"])]).all():
-            return g.logits[:len(h["rows"])]     # the first entries in order: a view, no copy
-        return g.logits.index_select(0, torch.from_numpy(h["rows"].astype(np.int64)).to(self.rt.device))
+            g.wanted = None
+        elif (h["rows"] == all_rows[:len(h["rows"])]).all():
+            g.wanted = g.logits[:len(h["rows"])]     # the first entries in order: a view, no copy
+        else:
+            g.wanted = None
+            g.rids = None                            # wanted rows that are no plain prefix: no patching next time
+            return g.logits.index_select(0, torch.from_numpy(h["rows"].astype(np.int64)).to(self.rt.device))
+        return g.wanted
+
+    def _advance_decode_meta(self, g: "_DecodeGraph", entries: Sequence[StepEntry]) -> bool:
+        """The last step through this graph had the same requests in the same order, and each has since grown by
+        exactly its one token: patch token ids, positions, decode chunks and the block-table entries of pages that
+        were added, in the host copy of the metadata, and send it.  False if anything else changed (the caller then
+        builds the metadata anew)."""
+        cache, h, flat = self.cache, g.h, g.flat
+        n = len(entries)
+        rps = [cache.get(e.rid) for e in entries]
+        pos0 = h["pos0"]
+        for i, (e, rp) in enumerate(zip(entries, rps)):
+            if rp.length != pos0[i] + 1 or len(e.tokens) != 1 or tuple(e.want) != g.wants[i] or rp.fresh:
+                return False
+            t = e.tokens[0]
+            if not 0 <= t < self.vocab_size:
+                raise ValueError(f"token id {int(t)} is outside the vocabulary of {self.vocab_size}")
+        off = g.ctx.part_offsets
+        ids = flat[off["ids"]:off["ids"] + n]
+        ids[:] = [e.tokens[0] for e in entries]
+        flat[off["positions"]:off["positions"] + n] += 1
+        flat[off["pos0"]:off["pos0"] + n] += 1
+        pos0[:n] += 1
+        h["kv_lens"][:n] += 1
+        dec = flat[off["dec"]:off["dec"] + DECODE_BUCKETS]
+        for bkt in range(DECODE_BUCKETS):
+            dec[bkt] = decode_chunk(h["kv_lens"], self.decode_p_max, n_kv=1 << bkt)
+        mb = h["max_blocks"]
+        for gi in range(self.storage.n_groups):
+            base = off["tables"][gi]
+            lens = g.table_lens[gi]
+            windowed = self.storage.group_window(gi) > 0
+            for i, rp in enumerate(rps):
+                t = rp.tables[gi]
+                if windowed:                      # pages behind the window have gone: write the row anew
+                    row = flat[base + i * mb:base + i * mb + len(t)]
+                    row[:] = t
+                elif len(t) != lens[i]:
+                    flat[base + i * mb + lens[i]:base + i * mb + len(t)] = t[lens[i]:]
+                lens[i] = len(t)
+        g.ctx.fresh = [False] * len(g.ctx.fresh)
+        self._staging.upload(flat, g.meta)
+        return True
