@@ -554,3 +554,40 @@ def test_attention_decode_fused_kernel(nh, kvh, d, rot, window, chunk):
         assert torch.equal(kp, kp_ref) and torch.equal(vp, vp_ref)       # the same bits in the pages
         assert bool(torch.isfinite(out.float()).all())
         assert rel_err(out, out_ref.float().cpu()) < 2e-3                 # the same products, merged in the same order
+
+
+@pytest.mark.parametrize("n,m,k", [(1, 48, 64), (8, 3584, 3584), (16, 100, 200), (5, 4608, 1000), (3, 40, 24)])
+def test_linear_bf16_with_norm_in_front_and_residual_behind(n, m, k):
+    """The few-row product that applies an RMSNorm to its input on the way and adds its result to the residual
+    stream, against norm, product and addition in float64 from the same bfloat16 weights."""
+    o = ops()
+    g = torch.Generator().manual_seed(n * 7 + m + k)
+    h = (torch.randn(n, k, generator=g) * 3).to(DEV)
+    gain = (1 + 0.3 * torch.randn(k, generator=g)).to(DEV)
+    w = (torch.randn(m, k, generator=g) * 0.05).to(torch.bfloat16).to(DEV)
+    bias = torch.randn(m, generator=g).to(DEV)
+    resid = torch.randn(n, m, generator=g).to(DEV)
+    eps = 1e-5
+    hd = h.double()
+    normed = (gain.double() * hd) * torch.rsqrt((hd * hd).mean(-1, keepdim=True) + eps)
+    ref = normed @ w.double().t() + bias.double()
+    out = torch.empty(n, m, device=DEV)
+    o.linear_bf16(h, w, bias, out, norm_gain=gain, norm_eps=eps)
+    assert rel_err(out, ref) < 1e-2
+    out2 = resid.clone()
+    o.linear_bf16(h, w, None, out2, norm_gain=gain, norm_eps=eps, residual=out2)       # in place
+    assert rel_err(out2, ref - bias.double() + resid.double()) < 1e-2
+    x = normed.to(torch.bfloat16)
+    out3 = resid.clone()
+    o.linear_bf16(x, w, bias, out3, residual=out3)                                      # residual only
+    assert rel_err(out3, x.double() @ w.double().t() + bias.double() + resid.double()) < 2e-3
+    # the gated product with the norm in front
+    inter = m
+    wgu = (torch.randn(2 * inter, k, generator=g) * 0.05).to(torch.bfloat16).to(DEV)
+    act = torch.empty(n, inter, device=DEV)
+    o.gated_linear_bf16(h, wgu, act, norm_gain=gain, norm_eps=eps)
+    gate, up = normed @ wgu[:inter].double().t(), normed @ wgu[inter:].double().t()
+    assert rel_err(act, torch.nn.functional.silu(gate) * up) < 1e-2
+    # more than 16 rows are refused
+    with pytest.raises(Exception):
+        o.linear_bf16(torch.zeros(17, k, device=DEV), w, None, torch.empty(17, m, device=DEV), norm_gain=gain, norm_eps=eps)

@@ -84,6 +84,14 @@ __device__ __forceinline__ void wave_lds_order() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+// two floats to two bf16 (round to nearest even) in one instruction
+__device__ __forceinline__ unsigned pack_bf16x2(float a, float b) {
+    f32x2_t v = {a, b};
+    return __builtin_bit_cast(unsigned, __builtin_convertvector(v, bf16x2_t));
+}
+
 // x[row][k .. k + 8); beyond the end of the row its last eight values are read instead (W is zero there)
 __device__ __forceinline__ bf16x8_t load_x(const bf16_t* row, int k, int K) {
     Frag f;
@@ -102,14 +110,21 @@ __device__ __forceinline__ bf16x8_t load_x(const bf16_t* row, int k, int K) {
 // keeps writes and reads off each other's banks; each wave has two such buffers of its own and no one else's, so
 // nothing but the order of its own LDS operations keeps them consistent.
 // ---------------------------------------------------------------------------
-template <int WPB, bool SWIGLU, typename TO>
-__global__ __launch_bounds__(WPB * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wp,
+// NORM: the tokens come as the fp32 residual stream h [N][K] with the gains of an RMSNorm: the kernel reads h * gain
+// (rounded to bf16) as its tokens, adds up h^2 on the way (every block walks all of k, so every block has the whole
+// sum of every row) and multiplies the finished sums by 1/sqrt(mean(h^2) + eps): the norm costs no launch and no
+// pass over h of its own.  resid: fp32 [N][Mout] that the result is added to (y may be resid itself).
+template <int WPB, bool SWIGLU, bool NORM, typename TO>
+__global__ __launch_bounds__(WPB * 64) void gemm_skinny_kernel(const void* __restrict__ xin, const bf16_t* __restrict__ wp,
                                                               const float* __restrict__ bias, TO* __restrict__ y, int N,
-                                                              int Mout, int K, int KT, int up_tiles) {
+                                                              int Mout, int K, int KT, int up_tiles,
+                                                              const float* __restrict__ gain, float eps,
+                                                              const float* resid) {
     constexpr int NW = SWIGLU ? 2 : 1;
-    constexpr int U = 4;
+    constexpr int U = NORM ? 2 : 4;     // tiles in flight (fp32 tokens take three times the registers: measured)
     __shared__ float red[NW][WPB][256];
     __shared__ uint4 xt[WPB][2][4 * 17];
+    __shared__ float ssq[NORM ? WPB : 1][16];
     const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63;
     const int r = lane & 15, g = lane >> 4;
     const int mt = blockIdx.x;
@@ -117,47 +132,88 @@ __global__ __launch_bounds__(WPB * 64) void gemm_skinny_kernel(const bf16_t* __r
     const bf16_t* wbase[NW];
     wbase[0] = wp + ((size_t)mt * KT * 64 + lane) * 8;
     if (SWIGLU) wbase[1] = wp + ((size_t)(mt + up_tiles) * KT * 64 + lane) * 8;
-    const bf16_t* xrow = x + (size_t)min(lane >> 2, N - 1) * K;
+    // bf16 tokens: lane l reads piece l % 4 (8 values) of row l / 4 and writes one 16-byte slot.
+    const bf16_t* xrow = (const bf16_t*)xin + (size_t)min(lane >> 2, N - 1) * K;
     const int xpiece = (lane & 3) * 8;
     const int wslot = (lane & 3) * 17 + (lane >> 2), rslot = g * 17 + r;
+    // fp32 residual stream (NORM): a row's 32 values of a tile are 128 bytes, so lane l reads quarter-piece l % 8
+    // (4 values) of rows l / 8 and l / 8 + 8, two loads of eight whole cache lines, and writes two 8-byte halves
+    // of slots.
+    const float* hrow_a = (const float*)xin + (size_t)min(lane >> 3, N - 1) * K;
+    const float* hrow_b = (const float*)xin + (size_t)min((lane >> 3) + 8, N - 1) * K;
+    const int hq = (lane & 7) * 4;
+    uint2* const xt2 = (uint2*)&xt[wv][0][0];
+    const int hslot_a = 2 * ((lane & 7) / 2 * 17 + (lane >> 3)) + (lane & 1), hslot_b = hslot_a + 16;
+    float ss_a = 0.f, ss_b = 0.f;
+    struct Piece { Frag f; uint2 a, b; };
+    auto load_piece = [&](int t) __attribute__((always_inline)) {
+        Piece p;
+        if constexpr (NORM) {
+            const int k = t * 32 + hq, kc = min(k, K - 4);
+            const float4 ha = *(const float4*)(hrow_a + kc), hb = *(const float4*)(hrow_b + kc);
+            const float4 gg = *(const float4*)(gain + kc);
+            if (k < K) {
+                ss_a += (ha.x * ha.x + ha.y * ha.y) + (ha.z * ha.z + ha.w * ha.w);
+                ss_b += (hb.x * hb.x + hb.y * hb.y) + (hb.z * hb.z + hb.w * hb.w);
+            }
+            p.a = make_uint2(pack_bf16x2(ha.x * gg.x, ha.y * gg.y), pack_bf16x2(ha.z * gg.z, ha.w * gg.w));
+            p.b = make_uint2(pack_bf16x2(hb.x * gg.x, hb.y * gg.y), pack_bf16x2(hb.z * gg.z, hb.w * gg.w));
+        } else {
+            p.f.v = load_x(xrow, t * 32 + xpiece, K);
+        }
+        return p;
+    };
+    // through the wave's LDS buffer `b` to the lane that needs it
+    auto exchange = [&](Piece& p, int b) __attribute__((always_inline)) {
+        if constexpr (NORM) {
+            xt2[b * (2 * 4 * 17) + hslot_a] = p.a;
+            xt2[b * (2 * 4 * 17) + hslot_b] = p.b;
+        } else {
+            xt[wv][b][wslot] = p.f.u;
+        }
+        wave_lds_order();
+        p.f.u = xt[wv][b][rslot];
+        wave_lds_order();       // and the next write to this buffer after these reads
+    };
     f32x4_t acc[NW];
 #pragma unroll
     for (int a = 0; a < NW; ++a) acc[a] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
     int t = t_begin;
     for (; t + U <= t_end; t += U) {
-        Frag wa[NW][U], xa[U];
+        Frag wa[NW][U];
+        Piece xa[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
 #pragma unroll
             for (int a = 0; a < NW; ++a) wa[a][u].u = *(const uint4*)(wbase[a] + (size_t)(t + u) * PK_TILE);
-            xa[u].v = load_x(xrow, (t + u) * 32 + xpiece, K);
+            xa[u] = load_piece(t + u);
         }
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            xt[wv][u & 1][wslot] = xa[u].u;
-            wave_lds_order();
-            xa[u].u = xt[wv][u & 1][rslot];
-            wave_lds_order();       // and the next write to this buffer after these reads
-        }
+        for (int u = 0; u < U; ++u) exchange(xa[u], u & 1);
 #pragma unroll
         for (int u = 0; u < U; ++u)
 #pragma unroll
             for (int a = 0; a < NW; ++a)
-                acc[a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[a][u].v, xa[u].v, acc[a], 0, 0, 0);
+                acc[a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[a][u].v, xa[u].f.v, acc[a], 0, 0, 0);
     }
     for (; t < t_end; ++t) {
-        Frag xa;
-        xa.v = load_x(xrow, t * 32 + xpiece, K);
-        xt[wv][0][wslot] = xa.u;
-        wave_lds_order();
-        xa.u = xt[wv][0][rslot];
-        wave_lds_order();
+        Piece xa = load_piece(t);
+        exchange(xa, 0);
 #pragma unroll
         for (int a = 0; a < NW; ++a) {
             Frag wa;
             wa.u = *(const uint4*)(wbase[a] + (size_t)t * PK_TILE);
-            acc[a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa.v, xa.v, acc[a], 0, 0, 0);
+            acc[a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa.v, xa.f.v, acc[a], 0, 0, 0);
         }
+    }
+    if constexpr (NORM) {
+        // the eight lanes of a row hold its quarter-pieces: add them, then the waves' shares in wave order
+#pragma unroll
+        for (int o = 1; o < 8; o <<= 1) {
+            ss_a += __shfl_xor(ss_a, o, 64);
+            ss_b += __shfl_xor(ss_b, o, 64);
+        }
+        if ((lane & 7) == 0) { ssq[wv][lane >> 3] = ss_a; ssq[wv][(lane >> 3) + 8] = ss_b; }
     }
     // acc[a][e] is feature 16 mt + 4 g + e of token r.  Sum the waves in wave order.
 #pragma unroll
@@ -173,8 +229,16 @@ __global__ __launch_bounds__(WPB * 64) void gemm_skinny_kernel(const bf16_t* __r
         if (SWIGLU)
             for (int q = 0; q < WPB; ++q) u += red[NW - 1][q][c];
         if (m < Mout && n < N) {
+            if constexpr (NORM) {
+                float tot = 0.f;
+                for (int q = 0; q < WPB; ++q) tot += ssq[q][n];
+                const float rinv = 1.0f / sqrtf(tot / (float)K + eps);
+                v *= rinv;
+                u *= rinv;
+            }
             if (SWIGLU) v = v / (1.f + expf(-v)) * u;
             else if (bias) v += bias[m];
+            if (resid) v += resid[(size_t)n * Mout + m];
             store_f32<TO>(y, (size_t)n * Mout + m, v);
         }
     }
@@ -370,10 +434,16 @@ extern "C" long long vt_linear_bf16_workspace(int N, int M, int K, int gated) {
     return splits > 1 ? (long long)splits * N * M : 0;
 }
 
+// gain != null: x is the fp32 residual stream and the RMSNorm (gain, eps) is part of the product; resid != null: the
+// result is added to it.  Both only with up to 16 tokens.
 template <bool SWIGLU, typename TO>
-static int linear_bf16(const bf16_t* x, const bf16_t* wp, const float* bias, TO* y, float* workspace, int N, int Mout,
-                       int K, hipStream_t stream) {
+static int linear_bf16(const void* xv, const bf16_t* wp, const float* bias, TO* y, float* workspace, int N, int Mout,
+                       int K, const float* gain, float eps, const float* resid, hipStream_t stream) {
     if (N == 0) return 0;
+    const bf16_t* x = (const bf16_t*)xv;
+    VT_REQUIRE((!gain && !resid) || (N <= 16 && K % 8 == 0 && (((uintptr_t)xv) & 15) == 0),
+               "vt_linear_bf16: the fused norm and residual need at most 16 rows and k a multiple of 8 (N=%d K=%d)", N, K);
+    VT_REQUIRE(!gain || (((uintptr_t)gain) & 15) == 0, "vt_linear_bf16: the norm's gains are not 16-byte aligned");
     const int KT = pk_cols(K) / 32, up_tiles = pk_rows(Mout) / 16;
     VT_REQUIRE((((uintptr_t)wp) & 15) == 0, "vt_linear_bf16: the packed matrix is not 16-byte aligned");
     if (K % 8 != 0 || ((uintptr_t)x & 15)) {
@@ -403,8 +473,11 @@ static int linear_bf16(const bf16_t* x, const bf16_t* wp, const float* bias, TO*
     // How k is split over the waves of a block depends on the shape of W only, so that a token's sums are added
     // in the same order whatever the number of rows: 8 waves, 16 for matrices with few rows and a long k.
     const int tiles16 = (Mout + 15) / 16;
-    if (tiles16 >= 512 || KT < 256) gemm_skinny_kernel<8, SWIGLU, TO><<<tiles16, 8 * 64, 0, stream>>>(x, wp, bias, y, N, Mout, K, KT, up_tiles);
-    else gemm_skinny_kernel<16, SWIGLU, TO><<<tiles16, 16 * 64, 0, stream>>>(x, wp, bias, y, N, Mout, K, KT, up_tiles);
+    const bool wide = tiles16 >= 512 || KT < 256;
+#define VT_SKINNY(W, NRM) gemm_skinny_kernel<W, SWIGLU, NRM, TO><<<tiles16, W * 64, 0, stream>>>(x, wp, bias, y, N, Mout, K, KT, up_tiles, gain, eps, resid)
+    if (gain) { if (wide) VT_SKINNY(8, true); else VT_SKINNY(16, true); }
+    else { if (wide) VT_SKINNY(8, false); else VT_SKINNY(16, false); }
+#undef VT_SKINNY
     VT_CHECK_LAUNCH("vt_linear_bf16");
     return 0;
 }
@@ -413,16 +486,27 @@ static int linear_bf16(const bf16_t* x, const bf16_t* wp, const float* bias, TO*
 extern "C" int vt_linear_bf16(const void* x, const void* wp, const float* bias, void* y, int out_dtype, float* workspace,
                               int N, int M, int K, hipStream_t stream) {
     VT_REQUIRE(N >= 0 && M > 0 && K > 0, "vt_linear_bf16: bad sizes N=%d M=%d K=%d", N, M, K);
-    if (out_dtype == VT_F32) return linear_bf16<false, float>((const bf16_t*)x, (const bf16_t*)wp, bias, (float*)y, workspace, N, M, K, stream);
-    if (out_dtype == VT_BF16) return linear_bf16<false, bf16_t>((const bf16_t*)x, (const bf16_t*)wp, bias, (bf16_t*)y, workspace, N, M, K, stream);
+    if (out_dtype == VT_F32) return linear_bf16<false, float>(x, (const bf16_t*)wp, bias, (float*)y, workspace, N, M, K, nullptr, 0.f, nullptr, stream);
+    if (out_dtype == VT_BF16) return linear_bf16<false, bf16_t>(x, (const bf16_t*)wp, bias, (bf16_t*)y, workspace, N, M, K, nullptr, 0.f, nullptr, stream);
     return vt_fail("vt_linear_bf16: unknown out dtype %d", out_dtype);
 }
 
-// y[N, I] = silu(x . Wg^T) * (x . Wu^T); wp = Wg [I, K] packed, followed by Wu [I, K] packed
+// The same for up to 16 tokens with an RMSNorm in front and a residual addition behind, each optional:
+// gain != null: h is the fp32 residual stream [N, K] and y = (rmsnorm(h; gain, eps) . W^T) + bias, else h is x in bf16;
+// resid != null (fp32 [N, M], may be y): y = resid + that.  y is fp32.
+extern "C" int vt_linear_bf16_fused(const void* h, const float* gain, float eps, const void* wp, const float* bias,
+                                    const float* resid, float* y, int N, int M, int K, hipStream_t stream) {
+    VT_REQUIRE(N >= 0 && M > 0 && K > 0, "vt_linear_bf16_fused: bad sizes N=%d M=%d K=%d", N, M, K);
+    VT_REQUIRE(gain || resid, "vt_linear_bf16_fused: neither a norm nor a residual: use vt_linear_bf16");
+    return linear_bf16<false, float>(h, (const bf16_t*)wp, bias, y, nullptr, N, M, K, gain, eps, resid, stream);
+}
+
+// y[N, I] = silu(x . Wg^T) * (x . Wu^T); wp = Wg [I, K] packed, followed by Wu [I, K] packed.
+// gain != null: x is the fp32 residual stream and rmsnorm(x; gain, eps) takes its place (up to 16 tokens).
 extern "C" int vt_gated_linear_bf16(const void* x, const void* wp, void* y, int out_dtype, int N, int I, int K,
-                                    hipStream_t stream) {
+                                    const float* gain, float eps, hipStream_t stream) {
     VT_REQUIRE(N >= 0 && I > 0 && K > 0, "vt_gated_linear_bf16: bad sizes N=%d I=%d K=%d", N, I, K);
-    if (out_dtype == VT_F32) return linear_bf16<true, float>((const bf16_t*)x, (const bf16_t*)wp, nullptr, (float*)y, nullptr, N, I, K, stream);
-    if (out_dtype == VT_BF16) return linear_bf16<true, bf16_t>((const bf16_t*)x, (const bf16_t*)wp, nullptr, (bf16_t*)y, nullptr, N, I, K, stream);
+    if (out_dtype == VT_F32) return linear_bf16<true, float>(x, (const bf16_t*)wp, nullptr, (float*)y, nullptr, N, I, K, gain, eps, nullptr, stream);
+    if (out_dtype == VT_BF16) return linear_bf16<true, bf16_t>(x, (const bf16_t*)wp, nullptr, (bf16_t*)y, nullptr, N, I, K, gain, eps, nullptr, stream);
     return vt_fail("vt_gated_linear_bf16: unknown out dtype %d", out_dtype);
 }

@@ -218,10 +218,13 @@ def linear_bf16_workspace(n: int, m: int, k: int) -> int:
 
 
 def linear_bf16(x: torch.Tensor, w, bias: Optional[torch.Tensor], out: torch.Tensor,
-                workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+                workspace: Optional[torch.Tensor] = None, norm_gain: Optional[torch.Tensor] = None,
+                norm_eps: float = 0.0, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Few rows (decoding, short portions): W is read once per 64 rows.  w: a PackedMatrix (a plain [m, k] tensor
     is packed on the spot, which costs more than the product).  Shapes whose k range is split over blocks need
-    `workspace` (float32, at least linear_bf16_workspace(n, m, k) elements)."""
+    `workspace` (float32, at least linear_bf16_workspace(n, m, k) elements).
+    Up to 16 rows, float32 output: with norm_gain, x is the float32 residual stream and rmsnorm(x; gain, eps) is
+    what gets multiplied; with residual (float32 [n, m], may be `out`), out = residual + the product."""
     n, k = x.shape
     if not isinstance(w, PackedMatrix):
         _chk(w, "linear_bf16.w", torch.bfloat16, (w.shape[0], k))
@@ -229,11 +232,22 @@ def linear_bf16(x: torch.Tensor, w, bias: Optional[torch.Tensor], out: torch.Ten
     m = w.rows
     if w.cols != k or w.halves != 1:
         raise KernelError(f"linear_bf16: x [{n}, {k}] does not fit a packed matrix [{w.rows}, {w.cols}] x {w.halves}")
-    _chk(x, "linear_bf16.x", torch.bfloat16)
+    fused = norm_gain is not None or residual is not None
+    _chk(x, "linear_bf16.x", torch.float32 if norm_gain is not None else torch.bfloat16)
     _chk(w.data, "linear_bf16.w", torch.bfloat16)
-    _chk(out, "linear_bf16.out", None, (n, m))
+    _chk(out, "linear_bf16.out", torch.float32 if fused else None, (n, m))
     if bias is not None:
         _chk(bias, "linear_bf16.bias", torch.float32, (m,))
+    if fused:
+        if n > 16 or k % 8:
+            raise KernelError(f"linear_bf16: the fused norm and residual take at most 16 rows and k a multiple of 8 (n={n}, k={k})")
+        if norm_gain is not None:
+            _chk(norm_gain, "linear_bf16.norm_gain", torch.float32, (k,))
+        if residual is not None:
+            _chk(residual, "linear_bf16.residual", torch.float32, (n, m))
+        _run(load_lib("vt_gemm_bf16"), "vt_linear_bf16_fused", _ptr(x), _ptr(norm_gain), _f(norm_eps), _ptr(w.data), _ptr(bias),
+             _ptr(residual), _ptr(out), _i(n), _i(m), _i(k), _stream())
+        return out
     need = linear_bf16_workspace(n, m, k) if n > 16 else 0
     if need:
         if workspace is None:
@@ -246,9 +260,11 @@ def linear_bf16(x: torch.Tensor, w, bias: Optional[torch.Tensor], out: torch.Ten
     return out
 
 
-def gated_linear_bf16(x: torch.Tensor, w_gate_up, out: torch.Tensor) -> torch.Tensor:
+def gated_linear_bf16(x: torch.Tensor, w_gate_up, out: torch.Tensor, norm_gain: Optional[torch.Tensor] = None,
+                      norm_eps: float = 0.0) -> torch.Tensor:
     """out = silu(x Wg^T) * (x Wu^T).  w_gate_up: a PackedMatrix of two halves (pack_matrix_bf16(w, halves=2)), or
-    the stacked [2 I, k] tensor, which is packed on the spot."""
+    the stacked [2 I, k] tensor, which is packed on the spot.  With norm_gain (up to 16 rows), x is the float32
+    residual stream and rmsnorm(x; gain, eps) is what gets multiplied."""
     n, k = x.shape
     if not isinstance(w_gate_up, PackedMatrix):
         _chk(w_gate_up, "gated_linear_bf16.w", torch.bfloat16, (w_gate_up.shape[0], k))
@@ -256,11 +272,15 @@ def gated_linear_bf16(x: torch.Tensor, w_gate_up, out: torch.Tensor) -> torch.Te
     w = w_gate_up
     if w.cols != k or w.halves != 2:
         raise KernelError(f"gated_linear_bf16: x [{n}, {k}] does not fit a packed matrix [{w.rows}, {w.cols}] x {w.halves}")
-    _chk(x, "gated_linear_bf16.x", torch.bfloat16)
+    _chk(x, "gated_linear_bf16.x", torch.float32 if norm_gain is not None else torch.bfloat16)
     _chk(w.data, "gated_linear_bf16.w", torch.bfloat16)
     _chk(out, "gated_linear_bf16.out", None, (n, w.rows))
+    if norm_gain is not None:
+        if n > 16 or k % 8:
+            raise KernelError(f"gated_linear_bf16: the fused norm takes at most 16 rows and k a multiple of 8 (n={n}, k={k})")
+        _chk(norm_gain, "gated_linear_bf16.norm_gain", torch.float32, (k,))
     _run(load_lib("vt_gemm_bf16"), "vt_gated_linear_bf16", _ptr(x), _ptr(w.data), _ptr(out), _i(_code(out)), _i(n),
-         _i(w.rows), _i(k), _stream())
+         _i(w.rows), _i(k), _ptr(norm_gain), _f(norm_eps), _stream())
     return out
 
 

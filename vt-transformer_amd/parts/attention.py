@@ -31,6 +31,9 @@ def decode_bucket(n_kv: int) -> int:
 
 @MIXERS.register("attention")
 class PagedAttention(Part):
+    takes_normed_input = True     # the q/k/v product applies the norm in front of it when the rows are few
+    adds_residual = True          # the output product adds to the residual stream when the rows are few
+
     def __init__(self, *, rt: Runtime, width: int, prefix: str, num_heads: int, num_kv_heads: int, head_dim: int,
                  qkv_bias: bool = False, out_bias: bool = False, window: int = 0,
                  position: Optional[PartSpec] = None, scale: Optional[float] = None, shared: Optional[dict] = None,
@@ -92,7 +95,7 @@ class PagedAttention(Part):
         self.p_qkv, self.p_o = rt.pack(self.w_qkv), rt.pack(self.w_o)
 
     # -- one step --------------------------------------------------------------
-    def forward(self, x: torch.Tensor, ctx, cache, state=None) -> torch.Tensor:
+    def forward(self, x, ctx, cache, state=None, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
         rt, nh, nkv, d = self.rt, self.nh, self.nkv, self.d
         n = x.shape[0]
         nq = nh * d
@@ -125,7 +128,7 @@ class PagedAttention(Part):
             ops.attention_bf16_decode_fused(qkv, cos, sin, cache.k, cache.v, cache.block_table, ctx.entry_pos0,
                                             ctx.decode_params[b:b + 1], ctx.decode_p_max, out, part_o, part_ml, nh, nkv, d,
                                             self.window, self.scale)
-            return linear(rt, out, self.w_o, self.b_o, "attn.o", packed=self.p_o)
+            return linear(rt, out, self.w_o, self.b_o, "attn.o", packed=self.p_o, residual=residual)
         q = rt.buffer("attn.q", (n, nq), rt.dtype)
         ops.rope_store(qkv, cos, sin, ctx.positions, ctx.tok_entry, cache.block_table, q, cache.k, cache.v, nh, nkv, d,
                        write_kv=cache.writes)
@@ -149,4 +152,4 @@ class PagedAttention(Part):
             if plan.n_tile_items:   # long portions: key/value blocks through LDS, shared by four waves
                 ops.attention_bf16_tiles(q, cache.k, cache.v, cache.block_table, plan.tile_items, plan.n_tile_items,
                                          out, nh, nkv, d, self.window, self.scale, rt=plan.tile_rt)
-        return linear(rt, out, self.w_o, self.b_o, "attn.o", packed=self.p_o)
+        return linear(rt, out, self.w_o, self.b_o, "attn.o", packed=self.p_o, residual=residual)

@@ -130,6 +130,30 @@ class Runtime:
         return _Scope()
 
 
+class NormedInput:
+    """What a block hands to a mixer or feed-forward that says it `takes_normed_input`: the residual stream and the
+    norm that is to be applied to it, not yet applied, so that the part's first matrix product can do it on the way
+    (few rows in bfloat16).  `materialize()` is the norm as a kernel of its own, for whoever cannot."""
+
+    def __init__(self, h: torch.Tensor, norm):
+        self.h, self.norm = h, norm
+
+    @property
+    def shape(self):
+        return self.h.shape
+
+    @property
+    def gain(self) -> torch.Tensor:
+        return self.norm.gain
+
+    @property
+    def eps(self) -> float:
+        return self.norm.eps
+
+    def materialize(self) -> torch.Tensor:
+        return self.norm.forward(self.h, None)
+
+
 class HostStaging:
     """Pinned host buffers in rotation for copies to the device that do not make the host wait: a buffer is
     written again only after the copy that last read it has run."""

@@ -4,6 +4,12 @@
 norm -> mixer -> add -> norm -> feed-forward -> add.  The residual stream h is
 fp32.  A layer hands its last output on unadded (`delta`), so the next norm
 adds it in the same kernel that normalises.
+
+With few rows in bfloat16 (decoding) the norms and additions are not kernels of
+their own: a mixer or feed-forward that says so takes the residual stream with
+the norm still to be applied (`NormedInput`: its first matrix product applies
+it) and adds its result to the stream itself (`residual=`: its last matrix
+product does).
 """
 from __future__ import annotations
 
@@ -11,7 +17,9 @@ from typing import Optional, Tuple
 
 import torch
 
-from .base import BLOCKS, Part, Runtime
+from .base import BLOCKS, NormedInput, Part, Runtime
+from .linear import can_fuse
+from .norm import RMSNorm
 
 
 @BLOCKS.register("prenorm")
@@ -28,9 +36,19 @@ class PreNormBlock(Part):
     def parts(self):
         return [self.norm_in, self.mixer, self.norm_post, self.feed_forward]
 
-    def forward(self, h: torch.Tensor, delta: Optional[torch.Tensor], ctx, cache, state) -> Tuple[torch.Tensor, torch.Tensor]:
-        a = self.norm_in.forward(h, delta)
-        y = self.mixer.forward(a, ctx, cache, state)
-        b = self.norm_post.forward(h, y)
-        z = self.feed_forward.forward(b, ctx)
+    def forward(self, h: torch.Tensor, delta: Optional[torch.Tensor], ctx, cache, state) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+        fuse = can_fuse(self.rt, h.shape[0]) and h.shape[1] % 8 == 0
+        y = self._run(self.mixer, self.norm_in, h, delta, fuse, ctx, cache, state)
+        z = self._run(self.feed_forward, self.norm_post, h, y, fuse, ctx)
         return h, z
+
+    def _run(self, part, norm, h, delta, fuse, *args):
+        """norm (of h + delta), then the part; returns what is still to be added to h (None: the part added it)."""
+        if fuse and delta is None and isinstance(norm, RMSNorm) and getattr(part, "takes_normed_input", False):
+            x = NormedInput(h, norm)
+        else:
+            x = norm.forward(h, delta)
+        if fuse and getattr(part, "adds_residual", False):
+            part.forward(x, *args, residual=h)
+            return None
+        return part.forward(x, *args)

@@ -16,7 +16,8 @@ import torch
 
 from ..kernels import ops
 from .base import FEED_FORWARDS, Part, Runtime, TensorDecl
-from .linear import SKINNY_MAX_ROWS, linear
+from .base import NormedInput
+from .linear import SKINNY_MAX_ROWS, can_fuse, linear
 
 
 @FEED_FORWARDS.register("gated_mlp")
@@ -48,13 +49,23 @@ class GatedMLP(Part):
         self.w_down = rt.place(get(nm["down"] + ".weight"), "matrix")
         self.p_gu, self.p_down = rt.pack(self.w_gu, halves=2), rt.pack(self.w_down)
 
-    def forward(self, x: torch.Tensor, ctx=None) -> torch.Tensor:
+    takes_normed_input = True     # the gate/up product applies the norm in front of it when the rows are few
+    adds_residual = True          # the down product adds to the residual stream when the rows are few
+
+    def forward(self, x, ctx=None, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
         rt = self.rt
         n = x.shape[0]
         act = rt.buffer("mlp.act", (n, self.inter), rt.dtype)
+        normed = isinstance(x, NormedInput)
+        if normed and not (can_fuse(rt, n) and self.width % 8 == 0):
+            x, normed = x.materialize(), False
         if rt.dtype == torch.bfloat16 and n <= SKINNY_MAX_ROWS:
-            ops.gated_linear_bf16(x, self.p_gu if self.p_gu is not None else self.w_gu, act)
+            w = self.p_gu if self.p_gu is not None else self.w_gu
+            if normed:
+                ops.gated_linear_bf16(x.h, w, act, norm_gain=x.gain, norm_eps=x.eps)
+            else:
+                ops.gated_linear_bf16(x, w, act)
         else:
             gu = linear(rt, x, self.w_gu, None, "mlp.gu")
             ops.silu_mul(gu, act)
-        return linear(rt, act, self.w_down, None, "mlp.down", packed=self.p_down)
+        return linear(rt, act, self.w_down, None, "mlp.down", packed=self.p_down, residual=residual)

@@ -15,20 +15,41 @@ from typing import Optional
 import torch
 
 from ..kernels import ops
-from .base import Runtime
+from .base import NormedInput, Runtime
 
 # up to this many rows W is streamed once per 64 rows by the skinny kernel
 SKINNY_MAX_ROWS = 64
 
 
+# the few-row kernel applies an RMSNorm in front and adds a residual behind for up to this many rows
+FUSE_MAX_ROWS = 16
+
+
+def can_fuse(rt: Runtime, n: int) -> bool:
+    return rt.dtype == torch.bfloat16 and n <= FUSE_MAX_ROWS
+
+
 def linear(rt: Runtime, x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], name: str,
            out_dtype: Optional[torch.dtype] = None, bias_lowp: Optional[torch.Tensor] = None,
-           packed=None) -> torch.Tensor:
+           packed=None, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
     """x [N, K] in the runtime's dtype -> [N, M].  `name` keys the output's scratch buffer.
     Output dtype: float32 from the hand-written kernels unless `out_dtype` says otherwise; the
     library path returns bfloat16 (its bias, if any, is `bias_lowp`, the same values in bfloat16).
-    packed: W as rt.pack(w) made it, for the few-row kernel (made on the spot if missing: slow)."""
+    packed: W as rt.pack(w) made it, for the few-row kernel (made on the spot if missing: slow).
+    x may be a NormedInput (the norm then happens inside the few-row kernel, or before the product as a kernel of
+    its own where that is not possible).  residual (float32 [N, M]): the product is added to it in place and
+    `residual` is returned; only callers that checked `can_fuse(rt, n)` may pass it."""
     n, k = x.shape
+    if residual is not None or isinstance(x, NormedInput):
+        if can_fuse(rt, n) and k % 8 == 0:
+            norm = x if isinstance(x, NormedInput) else None
+            out = residual if residual is not None else rt.buffer(name, (n, w.shape[0]), torch.float32)
+            return ops.linear_bf16(norm.h if norm else x, packed if packed is not None else w, bias, out,
+                                   norm_gain=norm.gain if norm else None, norm_eps=norm.eps if norm else 0.0,
+                                   residual=residual)
+        if residual is not None:
+            raise ValueError("linear: a residual to add to needs the few-row kernel (see can_fuse)")
+        x = x.materialize()
     m = w.shape[0]
     if rt.dtype == torch.float32:
         out = rt.buffer(name, (n, m), torch.float32)
