@@ -281,6 +281,8 @@ def attention_case(dtype, nh, kvh, d, page_size, window, entries, seed, spike=Fa
         kpd, vpd, btd = kp.to(DEV), vp.to(DEV), bt.to(DEV)
         # 16-row items with keys unsplit and split, one and two row tiles; then the LDS-tiled kernel on all entries
         for target, rt in ((0, 1), (10 ** 9, 1), (0, 2), (10 ** 9, 2)):
+            if rt == 2 and d > 128:
+                continue            # two row tiles per wave do not fit the registers with heads above 128
             items, citems, n_parts = plan_attention_items(start, pos0, nh // kvh, window, kvh, target_waves=target,
                                                           min_chunk=16, rt=rt)
             part_o = torch.full((max(1, n_parts) * rt * kvh * 16 * d,), float("nan"), device=DEV)

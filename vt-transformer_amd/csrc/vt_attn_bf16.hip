@@ -149,11 +149,17 @@ constexpr bool WIDE = (D % 32 == 0);           // 16x16x32 instruction for the s
 constexpr int QSTEPS = WIDE ? D / 32 : D / 16;
 constexpr int DT = D / 16;
 
-// Keys and values of one block of 16 keys as this lane needs them for the two A operands.
+// Keys and values of one block of 16 keys as they lie in their page: the keys are 16 D consecutive elements, the
+// values 16 consecutive elements of each of D rows; lane l holds the 16-byte pieces l, l + 64, ... of each.  Read as
+// the matrix instruction wants its operands (lane 16 g + r: key r or dim r, piece g) the four pieces of a row would
+// sit in lanes 16 apart and every lane's load would be a cache access of its own; in this order a load of the wave
+// is whole cache lines, and the pieces reach the lanes that need them through an LDS buffer of the wave
+// (KV_LDS_ELEMS elements: keys [16][D + 8], values [D][24]).
+constexpr int KVP = (2 * D + 63) / 64;            // pieces per lane, of the keys and of the values
+constexpr int KL_ROW = D + 8, VL_ROW = 24;        // padded LDS rows: operand reads without bank conflicts
+constexpr int KV_LDS_ELEMS = 16 * KL_ROW + D * VL_ROW;
 struct KVBlock {
-    uint4 k8[WIDE ? QSTEPS : 1];
-    uint2 k4[WIDE ? 1 : QSTEPS];
-    uint2 v[DT];
+    u32x4_t k[KVP], v[KVP];
     bool ok;
 };
 
@@ -161,23 +167,34 @@ struct KVBlock {
 // it).  Nothing is tested before the loads: a block without a page (a window has passed it: its keys are masked for
 // every row) reads `spare`, a page that exists, and is marked so that it is not multiplied.  Loads under a branch
 // would make every later use wait for all the loads in flight.
-__device__ __forceinline__ void load_block(KVBlock& b, const AttnArgs& a, int pg, int spare, int j0, int kvh, int r, int g) {
+__device__ __forceinline__ void load_block(KVBlock& b, const AttnArgs& a, int pg, int spare, int j0, int kvh, int lane) {
     const int ps = a.page_size;
     const int blk = page_index(a, j0);
     b.ok = pg >= 0 && pg < a.num_pages;
     const int pgc = b.ok ? pg : spare;
     const int off = j0 - blk * ps;
-    const bf16_t* kb = a.k_pages + (((size_t)pgc * a.n_kv + kvh) * ps + off + r) * D;
-    if constexpr (WIDE) {
+    const bf16_t* kb = a.k_pages + (((size_t)pgc * a.n_kv + kvh) * ps + off) * D;
+    const bf16_t* vb = a.v_pages + ((size_t)pgc * a.n_kv + kvh) * D * ps + off;
 #pragma unroll
-        for (int st = 0; st < QSTEPS; ++st) b.k8[st] = *(const uint4*)(kb + st * 32 + g * 8);
-    } else {
-#pragma unroll
-        for (int st = 0; st < QSTEPS; ++st) b.k4[st] = *(const uint2*)(kb + st * 16 + g * 4);
+    for (int i = 0; i < KVP; ++i) {
+        const int x = min(lane + 64 * i, 2 * D - 1);
+        b.k[i] = *(const u32x4_t*)(kb + x * 8);
+        b.v[i] = *(const u32x4_t*)(vb + (size_t)(x >> 1) * ps + (x & 1) * 8);
     }
-    const bf16_t* vb = a.v_pages + (((size_t)pgc * a.n_kv + kvh) * D + r) * ps + off + 4 * g;
+}
+
+// the pieces of a block into the wave's LDS buffer, where the operands are read from
+__device__ __forceinline__ void park_block(const KVBlock& b, bf16_t* kl, int lane) {
+    bf16_t* vl = kl + 16 * KL_ROW;
 #pragma unroll
-    for (int t = 0; t < DT; ++t) b.v[t] = *(const uint2*)(vb + (size_t)t * 16 * ps);
+    for (int i = 0; i < KVP; ++i) {
+        const int x = lane + 64 * i;
+        if (2 * D % 64 == 0 || x < 2 * D) {
+            const int key = x / (D / 8), c = x - key * (D / 8);
+            *(u32x4_t*)(kl + key * KL_ROW + c * 8) = b.k[i];
+            *(u32x4_t*)(vl + (x >> 1) * VL_ROW + (x & 1) * 8) = b.v[i];
+        }
+    }
 }
 
 // CH consecutive elements (from c, a multiple of CH) of a head as the projection left them in fp32, rotated: the
@@ -376,8 +393,13 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_kernel(AttnArg
     const int ps = a.page_size;
     const int last_page = (key_hi - 1) / ps;
     // one block of 16 keys against the RT row tiles of this wave
+    extern __shared__ __attribute__((aligned(16))) bf16_t wave_lds[];
+    bf16_t* const kl = wave_lds + wv * KV_LDS_ELEMS;      // this wave's buffer: keys, then values
+    const bf16_t* const vl = kl + 16 * KL_ROW;
     auto multiply = [&](const KVBlock& cur, int j0) __attribute__((always_inline)) {
         if (!cur.ok) return;
+        park_block(cur, kl, lane);
+        wave_lds_order();
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
             if (j0 > tile_hi[rt] || j0 + 15 < tile_lo[rt]) continue;   // every key masked for every row of the tile
@@ -385,13 +407,13 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_kernel(AttnArg
             if constexpr (WIDE) {
 #pragma unroll
                 for (int st = 0; st < QSTEPS; ++st) {
-                    U16 t; t.u = cur.k8[st];
+                    U16 t; t.u = *(const uint4*)(kl + r * KL_ROW + st * 32 + g * 8);
                     s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(t.v, q8[rt][st], s, 0, 0, 0);
                 }
             } else {
 #pragma unroll
                 for (int st = 0; st < QSTEPS; ++st) {
-                    U8 t; t.u = cur.k4[st];
+                    U8 t; t.u = *(const uint2*)(kl + r * KL_ROW + st * 16 + g * 4);
                     s = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(t.v, q4[rt][st], s, 0, 0, 0);
                 }
             }
@@ -407,11 +429,12 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_kernel(AttnArg
             const bool rescale = __any(alpha != 1.f);      // the maximum of some row moved
 #pragma unroll
             for (int t = 0; t < DT; ++t) {
-                U8 vf; vf.u = cur.v[t];
+                U8 vf; vf.u = *(const uint2*)(vl + (t * 16 + r) * VL_ROW + 4 * g);
                 if (rescale) o[rt][t] *= alpha;
                 o[rt][t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf.v, pf.v, o[rt][t], 0, 0, 0);
             }
         }
+        wave_lds_order();       // the next block is parked after these reads
     };
     // A ring of register buffers: while one block is multiplied the next NB - 1 are on their way from memory, and
     // the page id of the one after them comes from the block table (a scalar load).  Every turn loads, whether or
@@ -430,14 +453,14 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_kernel(AttnArg
     const int spare = min(max(btc[last_page], 0), a.num_pages - 1);
     int pg_next;                     // page of the next block to load
 #pragma unroll
-    for (int i = 0; i < NB - 1; ++i) load_block(ring[i], a, page_at(j_first + i * j_step), spare, min(j_first + i * j_step, j_end), kvh, r, g);
+    for (int i = 0; i < NB - 1; ++i) load_block(ring[i], a, page_at(j_first + i * j_step), spare, min(j_first + i * j_step, j_end), kvh, lane);
     pg_next = page_at(j_first + (NB - 1) * j_step);
     for (int j0 = j_first; j0 < key_hi; j0 += NB * j_step) {
 #pragma unroll
         for (int ph = 0; ph < NB; ++ph) {
             const int j = j0 + ph * j_step;
             if (j >= key_hi) break;
-            load_block(ring[(ph + NB - 1) % NB], a, pg_next, spare, min(j + (NB - 1) * j_step, j_end), kvh, r, g);
+            load_block(ring[(ph + NB - 1) % NB], a, pg_next, spare, min(j + (NB - 1) * j_step, j_end), kvh, lane);
             pg_next = page_at(j + NB * j_step);
             __builtin_amdgcn_sched_barrier(0);      // the loads stay here, ahead of this block's products
             multiply(ring[ph], j);
@@ -448,7 +471,9 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_kernel(AttnArg
         // The four waves hold partial results over disjoint keys of the same rows: merge them through LDS, half
         // of a large head at a time, and let all 256 threads write the result.
         constexpr int DH = (D > 128) ? D / 2 : D;
-        __shared__ __attribute__((aligned(16))) float so[4][16][DH + 4];
+        __syncthreads();            // every wave is done with its key/value buffer: the merge takes the memory over
+        float (*so)[16][DH + 4] = (float (*)[16][DH + 4])wave_lds;
+        static_assert(4 * 16 * (DH + 4) * 4 <= 4 * KV_LDS_ELEMS * 2, "the merge fits where the waves' buffers were");
         __shared__ float sm[4][16], sl[4][16];
         float lt = l[0];
         lt += __shfl_xor(lt, 16, 64);
@@ -871,6 +896,22 @@ static int shift_of(int v) {
     return -1;
 }
 
+// LDS of the kernels whose waves hand key/value blocks to their lanes through buffers of their own: more than a
+// kernel gets without asking when the head is large
+constexpr int WAVE_LDS_BYTES = 4 * KV_LDS_ELEMS * (int)sizeof(bf16_t);
+static int wave_kernels_lds() {
+    static bool set = false;
+    if (set) return 0;
+    const void* fns[3] = {(const void*)attn_bf16_kernel<false, 1>, (const void*)attn_bf16_kernel<false, (D <= 128 ? 2 : 1)>,
+                          (const void*)attn_bf16_kernel<true, 1>};
+    for (const void* f : fns) {
+        hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, WAVE_LDS_BYTES);
+        VT_REQUIRE(e == hipSuccess, "attention: cannot get %d bytes of LDS: %s", WAVE_LDS_BYTES, hipGetErrorString(e));
+    }
+    set = true;
+    return 0;
+}
+
 static int check_common(const char* who, int n_heads, int n_kv, int page_size, int max_blocks, int num_pages) {
     VT_REQUIRE(n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "%s: bad heads %d/%d", who, n_heads, n_kv);
     VT_REQUIRE(page_size > 0 && page_size % 16 == 0, "%s: page size %d is not a multiple of 16", who, page_size);
@@ -887,6 +928,7 @@ extern "C" int vt_attn_bf16(const void* q, const void* k_pages, const void* v_pa
                             int num_pages, int window, float scale, hipStream_t stream) {
     if (check_common("vt_attn_bf16", n_heads, n_kv, page_size, max_blocks, num_pages)) return -1;
     VT_REQUIRE(rt == 1 || rt == 2, "vt_attn_bf16: %d row tiles per item (1 or 2)", rt);
+    VT_REQUIRE(rt == 1 || D <= 128, "vt_attn_bf16: two row tiles per item need a head size of at most 128 (this is %d)", D);
     VT_REQUIRE(n_citems == 0 || (part_o && part_ml), "vt_attn_bf16: split keys but no workspace");
     if (n_items <= 0) return 0;
     AttnArgs a;
@@ -897,8 +939,9 @@ extern "C" int vt_attn_bf16(const void* q, const void* k_pages, const void* v_pa
     a.entry_pos0 = nullptr; a.dec_params = nullptr; a.p_max = 0; a.ps_shift = shift_of(page_size);
     a.qkv = nullptr; a.qkv_stride = 0; a.cos_t = a.sin_t = nullptr; a.rot = a.max_pos = 0;
     dim3 grid((n_items + 3) / 4, n_kv);
-    if (rt == 1) attn_bf16_kernel<false, 1><<<grid, 256, 0, stream>>>(a);
-    else attn_bf16_kernel<false, 2><<<grid, 256, 0, stream>>>(a);
+    if (wave_kernels_lds()) return -1;
+    if (rt == 1) attn_bf16_kernel<false, 1><<<grid, 256, WAVE_LDS_BYTES, stream>>>(a);
+    else attn_bf16_kernel<false, (D <= 128 ? 2 : 1)><<<grid, 256, WAVE_LDS_BYTES, stream>>>(a);
     VT_CHECK_LAUNCH("vt_attn_bf16");
     if (n_citems > 0) {
         attn_combine_kernel<false><<<dim3(n_citems, n_kv), 256, 0, stream>>>(citems, part_o, part_ml, (bf16_t*)out,
@@ -960,7 +1003,8 @@ extern "C" int vt_attn_bf16_decode(const void* q, const void* k_pages, const voi
     a.num_pages = num_pages; a.window = window; a.scale_log2 = scale * 1.4426950408889634f;
     a.entry_pos0 = entry_pos0; a.dec_params = dec_params; a.p_max = p_max; a.ps_shift = shift_of(page_size);
     a.qkv = nullptr; a.qkv_stride = 0; a.cos_t = a.sin_t = nullptr; a.rot = a.max_pos = 0;
-    attn_bf16_kernel<true, 1><<<dim3(a.n_items, n_kv), 256, 0, stream>>>(a);
+    if (wave_kernels_lds()) return -1;
+    attn_bf16_kernel<true, 1><<<dim3(a.n_items, n_kv), 256, WAVE_LDS_BYTES, stream>>>(a);
     VT_CHECK_LAUNCH("vt_attn_bf16_decode");
     attn_combine_kernel<true><<<dim3(n_entries, n_kv), 256, 0, stream>>>(nullptr, part_o, part_ml, (bf16_t*)out, n_heads,
                                                                         n_kv, entry_pos0, dec_params, p_max, window, 1);
@@ -995,7 +1039,8 @@ extern "C" int vt_attn_bf16_decode_fused(const float* qkv, long long qkv_stride,
     a.num_pages = num_pages; a.window = window; a.scale_log2 = scale * 1.4426950408889634f;
     a.entry_pos0 = entry_pos0; a.dec_params = dec_params; a.p_max = p_max; a.ps_shift = shift_of(page_size);
     a.qkv = qkv; a.qkv_stride = qkv_stride; a.cos_t = cos_t; a.sin_t = sin_t; a.rot = rot; a.max_pos = max_pos;
-    attn_bf16_kernel<true, 1><<<dim3(a.n_items, n_kv), 256, 0, stream>>>(a);
+    if (wave_kernels_lds()) return -1;
+    attn_bf16_kernel<true, 1><<<dim3(a.n_items, n_kv), 256, WAVE_LDS_BYTES, stream>>>(a);
     VT_CHECK_LAUNCH("vt_attn_bf16_decode_fused");
     attn_combine_kernel<true><<<dim3(n_entries, n_kv), 256, 0, stream>>>(nullptr, part_o, part_ml, (bf16_t*)out, n_heads,
                                                                         n_kv, entry_pos0, dec_params, p_max, window, 1);

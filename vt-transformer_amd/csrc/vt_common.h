@@ -63,6 +63,14 @@ template <typename T> __device__ __forceinline__ void store_f32(T* p, size_t i, 
 template <> __device__ __forceinline__ void store_f32<float>(float* p, size_t i, float v) { p[i] = v; }
 template <> __device__ __forceinline__ void store_f32<bf16_t>(bf16_t* p, size_t i, float v) { p[i] = f32_to_bf16(v); }
 
+// Between a wave's writes to an LDS buffer that only it uses and its reads of what its other lanes wrote: the LDS
+// executes a wave's operations in order, so all this has to do is to keep the compiler from moving the reads up.
+__device__ __forceinline__ void wave_lds_order() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);

@@ -76,14 +76,6 @@ extern "C" int vt_pack_matrix_bf16(const void* w, void* wp, int M, int K, hipStr
     return 0;
 }
 
-// Between a wave's writes to its own LDS buffer and its reads of what other lanes wrote: the LDS executes a wave's
-// operations in order, so all this has to do is to keep the compiler from moving the reads up.
-__device__ __forceinline__ void wave_lds_order() {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
-
 typedef __attribute__((ext_vector_type(2))) float f32x2_t;
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
 // two floats to two bf16 (round to nearest even) in one instruction

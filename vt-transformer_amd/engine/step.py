@@ -213,7 +213,8 @@ class StepContext:
     def _make_plan(self, key) -> AttentionPlan:
         group, window, n_kv, head_dim = key
         short, long = split_entries(self.h_entry_start, group)
-        row_tiles = choose_row_tiles(self.h_entry_start, group, n_kv, short) if len(short) else 1
+        # (heads above 128: two row tiles per wave do not fit the registers)
+        row_tiles = choose_row_tiles(self.h_entry_start, group, n_kv, short) if len(short) and head_dim <= 128 else 1
         items, citems, n_parts = plan_attention_items(self.h_entry_start, self.h_entry_pos0, group, window, n_kv,
                                                       rt=row_tiles, entries=short)
         t_items, tile_rt = plan_tile_items(self.h_entry_start, self.h_entry_pos0, group, window, n_kv, long)
