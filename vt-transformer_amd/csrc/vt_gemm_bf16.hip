@@ -237,7 +237,7 @@ __global__ __launch_bounds__(WPB * 64) void gemm_skinny_kernel(const void* __res
 }
 
 // ---------------------------------------------------------------------------
-// 17 to 64 tokens per block (a large decoding batch, a short portion): a block of 4 waves takes 64*R features
+// 17 to 64 tokens per block (a large decoding batch, a short portion): a block of WM waves takes 16*WM*R features
 // and 64 tokens.  The tokens' values pass through LDS once per block (coalesced loads, two buffers), so they cost
 // a fraction of W's traffic instead of a multiple; each wave streams the tiles of its own R tile rows of W from
 // memory into registers a stage (128 k, four tiles) ahead.  For matrices with few rows the k range is split over
@@ -246,10 +246,11 @@ __global__ __launch_bounds__(WPB * 64) void gemm_skinny_kernel(const void* __res
 #define MID_BK 128                 // k values per stage = PK_KPAD: a stage never leaves the packed matrix
 #define MID_XROW (MID_BK + 8)
 #define MID_KU (MID_BK / 32)       // tiles along k per stage
-#define MID_XP (MID_BK / 32)       // 16-byte pieces of x per thread and stage (64 tokens * MID_BK / 8 / 256)
+#define MID_PIECES (64 * MID_BK / 8) // 16-byte pieces of x per stage
 
-template <int R, bool SWIGLU, typename TO>
-__global__ __launch_bounds__(256) void gemm_mid_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wp,
+// WM waves per block: the host picks it so that the blocks fill the compute units evenly.
+template <int R, bool SWIGLU, int WM, typename TO>
+__global__ __launch_bounds__(WM * 64) void gemm_mid_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wp,
                                                       const float* __restrict__ bias, TO* __restrict__ y,
                                                       float* __restrict__ partial, int N, int Mout, int K, int KT,
                                                       int up_tiles, int k_per_split) {
@@ -258,7 +259,8 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const bf16_t* __restrict_
     __shared__ __attribute__((aligned(16))) bf16_t xs[2][64][MID_XROW];
     const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63;
     const int r = lane & 15, g = lane >> 4;
-    const int mt0 = (blockIdx.x * 4 + wv) * R, n0 = blockIdx.y * 64;
+    constexpr int MID_XP = (MID_PIECES + WM * 64 - 1) / (WM * 64);  // pieces of x per thread and stage
+    const int mt0 = (blockIdx.x * WM + wv) * R, n0 = blockIdx.y * 64;
     const int k_begin = blockIdx.z * k_per_split, k_end = min(pk_cols(K), k_begin + k_per_split);
     const int m_tiles = pk_rows(Mout) >> 4;
 
@@ -275,7 +277,7 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const bf16_t* __restrict_
     int xtok[MID_XP], xcol[MID_XP];
 #pragma unroll
     for (int q = 0; q < MID_XP; ++q) {
-        const int pidx = tid + 256 * q;
+        const int pidx = min(tid + WM * 64 * q, MID_PIECES - 1);  // spare threads repeat the last piece
         xtok[q] = pidx / (MID_BK / 8);
         xcol[q] = (pidx % (MID_BK / 8)) * 8;
         xsrc[q] = x + (size_t)min(n0 + xtok[q], N - 1) * K;
@@ -408,15 +410,48 @@ __global__ void gemm_plain_kernel(const bf16_t* __restrict__ x, const bf16_t* __
     store_f32<TO>(y, (size_t)n * Mout + m, v);
 }
 
+static int compute_units() {
+    static int cus = 0;
+    if (!cus) {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+            cus = 256;
+    }
+    return cus;
+}
+
 // Number of k ranges for the 64-token kernel: from the shape of W only (so the order of additions does not depend
-// on the batch), enough blocks to fill the GPU, every range a multiple of the stage length.
+// on the batch).  A launch lasts (rounds of blocks over the compute units) x (stages of a block); every further
+// range costs half a stage for the launch that adds the partial sums, and their traffic: 64 tokens x 128 rows
+// x 8 bytes per row block, where a stage reads 32 KB of W per block.
 static int mid_splits(int Mout, int K, int rows_per_block) {
     const int row_blocks = (Mout + rows_per_block - 1) / rows_per_block;
-    const int stages = pk_cols(K) / MID_BK;
-    int splits = (512 + row_blocks - 1) / row_blocks;
-    if (splits > 16) splits = 16;
-    if (splits > stages / 4) splits = stages / 4 > 0 ? stages / 4 : 1;
-    return splits < 1 ? 1 : splits;
+    const int stages = pk_cols(K) / MID_BK, cus = compute_units();
+    int best = 1;
+    double best_cost = -1.;
+    for (int s = 1; s <= 16 && s <= stages; ++s) {
+        const long rounds = ((long)row_blocks * s + cus - 1) / cus;
+        const double cost = (double)(rounds * ((stages + s - 1) / s)) + (s > 1 ? s * (0.5 + 2. * row_blocks / cus) : 0.);
+        if (best_cost < 0. || cost < best_cost) { best = s; best_cost = cost; }
+    }
+    return best;
+}
+
+// Waves per block of the 64-token kernel when k is not split: the blocks of a launch all take the same time, so
+// the launch lasts (rounds of blocks over the compute units) x (work of a block); pick the smallest product.
+static int mid_waves(int Mout, int rows_per_wave, int token_blocks) {
+    const int cus = compute_units();
+    const int choices[4] = {4, 5, 6, 8};
+    int best = 4;
+    long best_cost = -1;
+    for (int c = 0; c < 4; ++c) {
+        const int w = choices[c], rows = rows_per_wave * w;
+        const long blocks = (long)((Mout + rows - 1) / rows) * token_blocks;
+        const long cost = ((blocks + cus - 1) / cus) * w;
+        if (best_cost < 0 || cost < best_cost) { best = w; best_cost = cost; }
+    }
+    return best;
 }
 
 extern "C" long long vt_linear_bf16_workspace(int N, int M, int K, int gated) {
@@ -451,9 +486,15 @@ static int linear_bf16(const void* xv, const bf16_t* wp, const float* bias, TO* 
         const int splits = SWIGLU ? 1 : mid_splits(Mout, K, 64 * RR);
         VT_REQUIRE(splits == 1 || workspace, "vt_linear_bf16: this shape needs a workspace (vt_linear_bf16_workspace)");
         int kps = ((pk_cols(K) + splits - 1) / splits + MID_BK - 1) / MID_BK * MID_BK;
-        dim3 grid((Mout + 64 * RR - 1) / (64 * RR), (N + 63) / 64, splits);
+        const int wm = SWIGLU ? mid_waves(Mout, 16 * RR, (N + 63) / 64) : 4;
+        dim3 grid((Mout + 16 * wm * RR - 1) / (16 * wm * RR), (N + 63) / 64, splits);
         VT_REQUIRE(grid.y <= 65535, "vt_linear_bf16: too many rows (%d)", N);
-        gemm_mid_kernel<RR, SWIGLU, TO><<<grid, 256, 0, stream>>>(x, wp, bias, y, workspace, N, Mout, K, KT, up_tiles, kps);
+#define VT_MID(W) gemm_mid_kernel<RR, SWIGLU, W, TO><<<grid, W * 64, 0, stream>>>(x, wp, bias, y, workspace, N, Mout, K, KT, up_tiles, kps)
+        if (wm == 4) VT_MID(4);
+        else if (wm == 5) VT_MID(5);
+        else if (wm == 6) VT_MID(6);
+        else VT_MID(8);
+#undef VT_MID
         VT_CHECK_LAUNCH("vt_linear_bf16(64 tokens)");
         if (splits > 1) {
             const size_t n = (size_t)N * Mout;
