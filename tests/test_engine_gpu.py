@@ -36,9 +36,15 @@ def runner_for(model, pool_tokens, max_requests=8):
 
 
 def report(name, worst):
-    os.makedirs("gpurun_out", exist_ok=True)
-    with open("gpurun_out/engine_errors.txt", "a") as f:
-        f.write(f"{name}: worst relative error {worst:.3e}\n")
+    """The worst error of a comparison: printed (pytest -s shows it) and, with VT_TEST_REPORT_DIR set, appended
+    to engine_errors.txt in that folder."""
+    line = f"{name}: worst relative error {worst:.3e}"
+    print(line)
+    folder = os.environ.get("VT_TEST_REPORT_DIR")
+    if folder:
+        os.makedirs(folder, exist_ok=True)
+        with open(os.path.join(folder, "engine_errors.txt"), "a") as f:
+            f.write(line + "\n")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

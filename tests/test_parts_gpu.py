@@ -204,10 +204,36 @@ def test_run_order_is_data(dtype):
 
 
 # ---------------------------------------------------------------------------
-# parts of the test's own: a mixer with per-request state, and another position encoding
+# parts of the test's own: a mixer with per-request state, another position encoding, a feed-forward with routing
 # ---------------------------------------------------------------------------
 def register_toy_parts():
-    from vt_transformer_amd.parts import MIXERS, POSITIONS, Part, StateNeed, TensorDecl
+    from vt_transformer_amd.parts import FEED_FORWARDS, MIXERS, POSITIONS, Part, StateNeed, TensorDecl
+
+    @FEED_FORWARDS.register("toy_routed")
+    class ToyRouted(Part):
+        """Every token goes to the one expert (a matrix) whose router logit is largest, weighted by the softmax
+        of the router's logits."""
+
+        def __init__(self, *, rt, width, prefix, experts):
+            self.rt, self.width, self.experts, self.prefix = rt, width, int(experts), prefix
+
+        def tensors(self):
+            t = {self.prefix + "router.weight": TensorDecl((self.experts, self.width), "matrix")}
+            for e in range(self.experts):
+                t[f"{self.prefix}experts.{e}.weight"] = TensorDecl((self.width, self.width), "matrix")
+            return t
+
+        def load(self, get, rt):
+            self.router = rt.place(get(self.prefix + "router.weight"), "matrix").float()
+            self.w = torch.stack([rt.place(get(f"{self.prefix}experts.{e}.weight"), "matrix").float()
+                                  for e in range(self.experts)])
+
+        def forward(self, x, ctx=None):
+            xf = x.float()
+            p = torch.softmax(xf @ self.router.t(), dim=-1)
+            top = p.argmax(dim=-1)
+            y = torch.einsum("tk,tmk->tm", xf, self.w[top]) * p.gather(1, top[:, None])
+            return y.to(x.dtype)
 
     @MIXERS.register("toy_decay")
     class ToyDecay(Part):
@@ -282,8 +308,11 @@ class ToyConfig(ModelConfig):
             else:
                 mixer = PartSpec("attention", {"num_heads": 2, "num_kv_heads": 1, "head_dim": 16, "prefix": "attn.",
                                                "position": PartSpec("toy_offset", {"slope": d["slope"]})})
-            layers.append(LayerSpec(PartSpec("prenorm", {}), mixer,
-                                    PartSpec("gated_mlp", {"intermediate_size": d["inter"], "prefix": "ffn."}),
+            if i % 4 == 3:
+                ffn = PartSpec("toy_routed", {"experts": d["experts"], "prefix": "moe."})
+            else:
+                ffn = PartSpec("gated_mlp", {"intermediate_size": d["inter"], "prefix": "ffn."})
+            layers.append(LayerSpec(PartSpec("prenorm", {}), mixer, ffn,
                                     {"input": norm("n1.weight"), "post_mixer": norm("n2.weight")}, f"blocks.{i}."))
         return ModelSpec("ToyStateForCausalLM", d["vocab"], d["width"], PartSpec("embedding", {"name": "emb.weight"}),
                          layers, [ScheduleEntry(i) for i in range(d["n_layer"])], norm("final.weight"),
@@ -314,11 +343,16 @@ def toy_plain(d, w, ids):
             y = pm.linear(pm.attention(q, k, v).reshape(t, 32), w[p + "attn.o_proj.weight"])
         x = x + y
         b = pm.rmsnorm(x, w[p + "n2.weight"], d["eps"])
-        x = x + pm.swiglu(b, w[p + "ffn.gate_proj.weight"], w[p + "ffn.up_proj.weight"], w[p + "ffn.down_proj.weight"])
+        if i % 4 == 3:
+            pr = torch.softmax(b @ w[p + "moe.router.weight"].t(), dim=-1)
+            top = pr.argmax(dim=-1)
+            x = x + torch.stack([(w[f"{p}moe.experts.{int(top[j])}.weight"] @ b[j]) * pr[j, top[j]] for j in range(t)])
+        else:
+            x = x + pm.swiglu(b, w[p + "ffn.gate_proj.weight"], w[p + "ffn.up_proj.weight"], w[p + "ffn.down_proj.weight"])
     return pm.rmsnorm(x, w["final.weight"], d["eps"]) @ w["emb.weight"].t()
 
 
-def test_toy_mixer_with_state_and_toy_position_encoding():
+def test_toy_mixer_with_state_toy_position_encoding_and_toy_routing():
     """Registered here, built by the framework's model builder from a spec, stepped by its step function in
     portions and beside another request, with the state slot cleared when a slot is used again."""
     from vt_transformer_amd.config import config_from_dict, register_architecture
@@ -327,7 +361,7 @@ def test_toy_mixer_with_state_and_toy_position_encoding():
     register_toy_parts()
     register_architecture("ToyStateForCausalLM", ToyConfig)
     d = {"architectures": ["ToyStateForCausalLM"], "n_layer": 4, "width": 48, "inter": 64, "vocab": 90, "eps": 1e-6,
-         "decay": 0.9, "slope": 0.01}
+         "decay": 0.9, "slope": 0.01, "experts": 3}
     cfg = config_from_dict(d)
     assert isinstance(cfg, ToyConfig)
     model = build_model(cfg, "float32")

@@ -633,11 +633,11 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_tile_kernel(At
     // the wave's index as a scalar: what depends only on it (which keys the wave's tiles see) then stays in scalar
     // registers and its tests are scalar branches
     const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int* it = a.items + (size_t)blockIdx.x * ITEM_INTS;
+    const int* it = a.items + (size_t)blockIdx.y * ITEM_INTS;
     const int entry = it[0], q_tok0 = it[1], q_len = it[2], pos0 = it[3], q_row0 = it[4];
     const int key_lo = it[5], key_hi = it[6];
     if (entry < 0) return;
-    const int kvh = blockIdx.y;
+    const int kvh = blockIdx.x;
     const int G = a.n_heads / a.n_kv;
     const int r = lane & 15, g = lane >> 4;
     const int n_rows = q_len * G;
@@ -966,7 +966,10 @@ extern "C" int vt_attn_bf16_tiles(const void* q, const void* k_pages, const void
     a.num_pages = num_pages; a.window = window; a.scale_log2 = scale * 1.4426950408889634f;
     a.entry_pos0 = nullptr; a.dec_params = nullptr; a.p_max = 0; a.ps_shift = shift_of(page_size);
     a.qkv = nullptr; a.qkv_stride = 0; a.cos_t = a.sin_t = nullptr; a.rot = a.max_pos = 0;
-    dim3 grid(n_items, n_kv);
+    // blocks start in the order of their index, x fastest: all kv heads of the first (longest) item, then the next
+    // item's, so that the longest items of every head start first and the rest fill in as blocks finish
+    dim3 grid(n_kv, n_items);
+    VT_REQUIRE(grid.y <= 65535, "vt_attn_bf16_tiles: too many items (%d)", n_items);
     // more LDS than a kernel gets without asking
     static bool lds_set = false;
     if (!lds_set) {

@@ -58,7 +58,10 @@ class AttentionPlan:
 MAX_PARTS = 128     # the merge kernel holds the weights of at most this many items per row tile
 
 
-TILE_RT2_MIN_BLOCKS = 384
+# the tiled kernel: blocks that run at a time (two per compute unit), and microseconds per step of 64 keys of a block
+# with one and two row tiles per wave (measured on 512 to 4,096-token portions with and without earlier keys)
+TILE_SLOTS = 512
+TILE_STEP_US = {1: 2.1, 2: 2.45}
 LONG_ENTRY_ROWS = 256   # entries with at least this many (token, head-of-group) rows go to the LDS-tiled kernel
 
 
@@ -71,33 +74,50 @@ def split_entries(entry_start: np.ndarray, group: int) -> Tuple[np.ndarray, np.n
 
 
 def plan_tile_items(entry_start: np.ndarray, entry_pos0: np.ndarray, group: int, window: int, n_kv: int,
-                    entries: np.ndarray, rt: Optional[int] = None) -> Tuple[np.ndarray, int]:
+                    entries: np.ndarray, rt: Optional[int] = None, slots: int = TILE_SLOTS) -> Tuple[np.ndarray, int]:
     """Items of the LDS-tiled kernel: 64 * rt rows of one entry and every key they may see, longest first so that
-    the blocks that finish last start first.  Returns (items [n, 8], rt)."""
+    the blocks that finish last start first.  Returns (items [n, 8], rt).
+
+    rt (row tiles per wave) is chosen by an estimate of the launch's length.  A block's step over 64 keys takes
+    about as long with two row tiles as with one (TILE_STEP_US), because a wave waits on its own chain of loads,
+    products and exponentials more than on the machine; `slots` blocks run at a time and the others follow as
+    blocks finish, so a launch lasts as long as its longest item or as all items' steps shared out over the
+    slots, whichever is more."""
     q_len = (entry_start[1:] - entry_start[:-1]).astype(np.int64)[entries]
     rows = q_len * group
+    e_pos0_all = entry_pos0[entries].astype(np.int64)
+
+    def items_for(rt_: int):
+        rpi = 64 * rt_
+        n_tiles = (rows + rpi - 1) // rpi
+        total = int(n_tiles.sum())
+        if total == 0:
+            return np.zeros((0, ATTN_ITEM_INTS), np.int64), np.zeros((0,), np.int64)
+        which = np.repeat(np.arange(len(entries)), n_tiles)
+        first = np.cumsum(n_tiles) - n_tiles
+        row0 = (np.arange(total) - np.repeat(first, n_tiles)) * rpi
+        ent = entries[which]
+        e_rows, e_len = rows[which], q_len[which]
+        e_pos0, e_start = e_pos0_all[which], entry_start[:-1][ent].astype(np.int64)
+        min_p = e_pos0 + row0 // group
+        max_p = e_pos0 + np.minimum(e_rows - 1, row0 + rpi - 1) // group
+        lo = np.maximum(0, min_p - window + 1) if window > 0 else np.zeros_like(min_p)
+        key_lo, key_hi = (lo // 16) * 16, max_p + 1
+        return np.stack([ent, e_start, e_len, e_pos0, row0, key_lo, key_hi, np.full(total, -1)], axis=1), key_hi - key_lo
+
+    def estimate(span: np.ndarray, rt_: int) -> float:
+        steps = (span + 63) // 64
+        return max(float(steps.max()), float(steps.sum()) * n_kv / slots) * TILE_STEP_US[rt_]
+
     if rt is None:
-        # 128-row items (rt = 2) read every operand from LDS half as often, but halve the number of blocks: they
-        # pay once the machine's 256 compute units still get well over one block each (measured on 2,048 and
-        # 1,024-token portions)
-        rt = 2 if int(((rows + 127) // 128).sum()) * n_kv >= TILE_RT2_MIN_BLOCKS else 1
-    rpi = 64 * rt
-    n_tiles = (rows + rpi - 1) // rpi
-    total = int(n_tiles.sum())
-    if total == 0:
-        return np.zeros((0, ATTN_ITEM_INTS), np.int32), rt
-    which = np.repeat(np.arange(len(entries)), n_tiles)
-    first = np.cumsum(n_tiles) - n_tiles
-    row0 = (np.arange(total) - np.repeat(first, n_tiles)) * rpi
-    ent = entries[which]
-    e_rows, e_len = rows[which], q_len[which]
-    e_pos0, e_start = entry_pos0[ent].astype(np.int64), entry_start[:-1][ent].astype(np.int64)
-    min_p = e_pos0 + row0 // group
-    max_p = e_pos0 + np.minimum(e_rows - 1, row0 + rpi - 1) // group
-    lo = np.maximum(0, min_p - window + 1) if window > 0 else np.zeros_like(min_p)
-    key_lo, key_hi = (lo // 16) * 16, max_p + 1
-    items = np.stack([ent, e_start, e_len, e_pos0, row0, key_lo, key_hi, np.full(total, -1)], axis=1)
-    order = np.argsort(-(key_hi - key_lo), kind="stable")
+        cands = [items_for(1), items_for(2)]
+        if cands[0][0].shape[0] == 0:
+            return cands[0][0].astype(np.int32), 1
+        rt = 1 if estimate(cands[0][1], 1) <= estimate(cands[1][1], 2) else 2
+        items, span = cands[rt - 1]
+    else:
+        items, span = items_for(rt)
+    order = np.argsort(-span, kind="stable")
     return items[order].astype(np.int32), rt
 
 
@@ -217,7 +237,9 @@ class StepContext:
         row_tiles = choose_row_tiles(self.h_entry_start, group, n_kv, short) if len(short) and head_dim <= 128 else 1
         items, citems, n_parts = plan_attention_items(self.h_entry_start, self.h_entry_pos0, group, window, n_kv,
                                                       rt=row_tiles, entries=short)
-        t_items, tile_rt = plan_tile_items(self.h_entry_start, self.h_entry_pos0, group, window, n_kv, long)
+        # (heads above 128: one block per compute unit at a time)
+        t_items, tile_rt = plan_tile_items(self.h_entry_start, self.h_entry_pos0, group, window, n_kv, long,
+                                           slots=TILE_SLOTS if head_dim <= 128 else TILE_SLOTS // 2)
         rt = self.rt
         tag = f"attnplan.{group}.{window}.{n_kv}.{head_dim}"
         flat = np.concatenate([items.reshape(-1), citems.reshape(-1), t_items.reshape(-1)])
