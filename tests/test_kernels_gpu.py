@@ -79,9 +79,9 @@ def test_rmsnorm_rows_gather():
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_silu_mul(dtype):
+@pytest.mark.parametrize("n,inter", [(5, 200), (3, 204), (2, 203), (300, 1184)])   # widths in steps of 8, of 4, odd
+def test_silu_mul(dtype, n, inter):
     g = torch.Generator().manual_seed(4)
-    n, inter = 5, 200
     gu = (torch.randn(n, 2 * inter, generator=g) * 4).to(dtype)
     gate, up = gu[:, :inter].double(), gu[:, inter:].double()
     ref = gate / (1 + torch.exp(-gate)) * up

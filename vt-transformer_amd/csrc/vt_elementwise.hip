@@ -244,8 +244,57 @@ __global__ __launch_bounds__(256) void silu_mul_vec_kernel(const TI* __restrict_
     }
 }
 
+// bfloat16 in and out, widths that are a multiple of 8: 16 bytes per access, two accesses of gate and of up in
+// flight per thread.
+__device__ __forceinline__ unsigned silu_mul_pair(unsigned g, unsigned u) {
+    const float g0 = __uint_as_float(g << 16), g1 = __uint_as_float(g & 0xffff0000u);
+    const float u0 = __uint_as_float(u << 16), u1 = __uint_as_float(u & 0xffff0000u);
+    return (unsigned)f32_to_bf16(g0 / (1.f + __expf(-g0)) * u0) | ((unsigned)f32_to_bf16(g1 / (1.f + __expf(-g1)) * u1) << 16);
+}
+__global__ __launch_bounds__(256) void silu_mul_bf16x8_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ out,
+                                                             int inter, int n) {
+    const int opr = inter >> 3;                                   // groups of 8 per row
+    const long long total = (long long)opr * n;
+    const long long stride = (long long)gridDim.x * 256;
+    for (long long base = (long long)blockIdx.x * 256 + threadIdx.x; base < total; base += 2 * stride) {
+        uint4 g[2], u[2];
+        long long idx[2];
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+            idx[k] = base + k * stride;
+            if (idx[k] < total) {
+                const long long t = idx[k] / opr;
+                const int i = (int)(idx[k] - t * opr) * 8;
+                const bf16_t* row = gu + (size_t)t * 2 * inter;
+                g[k] = *(const uint4*)(row + i);
+                u[k] = *(const uint4*)(row + inter + i);
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+            if (idx[k] < total) {
+                const long long t = idx[k] / opr;
+                const int i = (int)(idx[k] - t * opr) * 8;
+                uint4 o;
+                o.x = silu_mul_pair(g[k].x, u[k].x); o.y = silu_mul_pair(g[k].y, u[k].y);
+                o.z = silu_mul_pair(g[k].z, u[k].z); o.w = silu_mul_pair(g[k].w, u[k].w);
+                *(uint4*)(out + (size_t)t * inter + i) = o;
+            }
+        }
+    }
+}
+
 template <typename TI, typename TO>
 static void launch_silu_mul(const void* gu, void* out, int n, int inter, hipStream_t stream) {
+    if constexpr (sizeof(TI) == 2 && sizeof(TO) == 2) {
+        if (inter % 8 == 0 && !((uintptr_t)gu & 15) && !((uintptr_t)out & 15)) {
+            const long long total = (long long)(inter / 8) * n;
+            long long blocks = (total + 511) / 512;
+            if (blocks > 8192) blocks = 8192;
+            silu_mul_bf16x8_kernel<<<(unsigned)(blocks < 1 ? 1 : blocks), 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, inter, n);
+            return;
+        }
+    }
     if (inter % 4 == 0 && !((uintptr_t)gu & 15) && !((uintptr_t)out & 15)) {
         const long long total = (long long)(inter / 4) * n;
         long long blocks = (total + 1023) / 1024;
