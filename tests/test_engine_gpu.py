@@ -282,6 +282,32 @@ def test_decode_graph_replays_match_eager(model_folders):
     assert len(graph._graphs) >= 1
 
 
+def test_group_of_17_query_heads_is_not_replayed_and_right(tmp_path):
+    """More query heads per kv head than the decoding kernels' one tile of 16 rows: the model says that its steps
+    cannot be replayed, decoding goes through the planned kernel step by step, and the logits are those of the
+    plain implementation."""
+    from vt_transformer_amd.config import config_from_dict
+    from vt_transformer_amd.engine import StepEntry, load_model
+    from vt_transformer_amd.weights import write_random_model
+    d = dict(TINY["A"], num_attention_heads=17, num_key_value_heads=1, head_dim=16, hidden_size=48, num_hidden_layers=2)
+    folder = str(tmp_path / "g17")
+    write_random_model(config_from_dict(d), folder, seed=9)
+    cfg, w = plain_model.read_folder(folder)
+    toks = random_requests(d["vocab_size"], [40], seed=3)["r0"]
+    ref = plain_model.forward(cfg, w, toks)
+    for dtype, tol in (("float32", 2e-5), ("bfloat16", 3e-2)):
+        runner = runner_for(load_model(folder, dtype), 128)
+        runner.decode_graphs = True
+        assert not runner._replayable
+        runner.admit("r")
+        got = [runner.step([StepEntry("r", toks[:25], list(range(25)))]).cpu()]
+        for i in range(25, 40):
+            got.append(runner.step([StepEntry("r", toks[i:i + 1], [0])]).cpu())
+        assert not runner._graphs
+        got = torch.cat(got).double()
+        assert float((got - ref).abs().max() / ref.abs().max()) < tol, dtype
+
+
 def test_library_algorithm_search_keeps_results(model_folders):
     """With the GEMM library's algorithm search on, a long portion gives the same logits to rounding."""
     from vt_transformer_amd.engine import Engine, StepEntry

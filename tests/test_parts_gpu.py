@@ -388,4 +388,4 @@ def test_toy_mixer_with_state_toy_position_encoding_and_toy_routing():
     assert runner.cache.get("c").slot == 0
     got_c = runner.step([StepEntry("c", c, list(range(12)))]).cpu()
     assert rel(got_c, rc) < 2e-5
-    assert not runner._stateless                        # such a model is never replayed from a captured graph
+    assert not runner._stateless and not runner._replayable     # such a model is never replayed from a captured graph

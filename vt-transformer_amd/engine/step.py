@@ -310,10 +310,14 @@ class ModelRunner:
         self._staging = HostStaging(torch.int32)
         self.decode_p_max = max(1, min(16, -(-self.max_seq_len // 64)))   # items one entry's keys are cut into at most
         # Decoding steps of a bfloat16 model are captured once per batch size and replayed, unless a mixer keeps
-        # state of its own between steps (the warm-up run before a capture would advance it twice).
+        # state of its own between steps (the warm-up run before a capture would advance it twice) or a part does
+        # not declare that its step can be replayed.
         self.decode_graphs = False
         self._graphs: Dict[int, _DecodeGraph] = {}
         self._stateless = all(s is None for s in self.storage.state)
+        parts = model.parts() if hasattr(model, "parts") else None
+        self._replayable = (self._stateless and parts is not None
+                            and all(bool(getattr(p, "replayable", False)) for p in parts))
 
     # -- requests -----------------------------------------------------------
     def admit(self, rid: Hashable) -> bool:
@@ -426,7 +430,7 @@ class ModelRunner:
             raise OutOfPages(f"the step needs more pages than are free ({cache.available_pages()} free per group)")
         fresh_slots = [cache.get(e.rid).slot for e in entries if cache.get(e.rid).fresh]
         self.storage.clear_state(fresh_slots)
-        use_graph = (self.decode_graphs and self._stateless and self.rt.dtype == torch.bfloat16
+        use_graph = (self.decode_graphs and self._replayable and self.rt.dtype == torch.bfloat16
                      and len(entries) <= GRAPH_BATCHES[-1] and all(len(e.tokens) == 1 for e in entries))
         if use_graph:
             logits = self._step_decode_graph(entries)

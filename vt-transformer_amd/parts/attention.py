@@ -59,6 +59,12 @@ class PagedAttention(Part):
         self.position = shared[key]
         self.w_qkv = self.b_qkv = self.b_qkv_lowp = self.w_o = self.b_o = self.p_qkv = self.p_o = None
 
+    @property
+    def replayable(self) -> bool:
+        # the decoding kernels cut the keys from positions in device memory; a group of more than 16 query heads
+        # takes the kernel whose work items the host plans anew every step
+        return self.nh // self.nkv <= 16 and bool(getattr(self.position, "replayable", False))
+
     # -- what the cache manager must hold for this mixer --------------------
     def cache_need(self) -> Optional[CacheNeed]:
         return CacheNeed(self.nkv, self.d, self.window)

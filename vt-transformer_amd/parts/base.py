@@ -182,6 +182,12 @@ class HostStaging:
 class Part:
     """Base of all parts."""
 
+    # True: a decoding step through this part can be recorded once and replayed, i.e. between one step and the
+    # next only values in device memory change (token ids, positions, block tables), never the launches, their
+    # sizes or host values baked into them.  The step function replays decoding steps only if every part of the
+    # model says so; a part that does not know stays with the default and its model is run step by step.
+    replayable = False
+
     def tensors(self) -> Dict[str, TensorDecl]:
         """Full tensor names this part loads, with their shapes."""
         return {}

@@ -25,6 +25,7 @@ from .norm import RMSNorm
 @BLOCKS.register("prenorm")
 class PreNormBlock(Part):
     norm_roles = ("input", "post_mixer")
+    replayable = True
 
     def __init__(self, *, rt: Runtime, norms, mixer, feed_forward):
         self.rt = rt

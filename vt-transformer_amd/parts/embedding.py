@@ -19,6 +19,8 @@ from .linear import SKINNY_MAX_ROWS
 
 @EMBEDDINGS.register("embedding")
 class TokenEmbedding(Part):
+    replayable = True
+
     def __init__(self, *, rt: Runtime, width: int, vocab_size: int, name: str):
         self.rt, self.width, self.vocab, self.name = rt, int(width), int(vocab_size), name
         self.table: Optional[torch.Tensor] = None
@@ -36,6 +38,8 @@ class TokenEmbedding(Part):
 
 @HEADS.register("linear_head")
 class LinearHead(Part):
+    replayable = True
+
     def __init__(self, *, rt: Runtime, width: int, vocab_size: int, name: str, tied_to: Optional[str] = None):
         self.rt, self.width, self.vocab, self.name, self.tied_to = rt, int(width), int(vocab_size), name, tied_to
         self.weight: Optional[torch.Tensor] = None

@@ -22,6 +22,8 @@ from .linear import SKINNY_MAX_ROWS, can_fuse, linear
 
 @FEED_FORWARDS.register("gated_mlp")
 class GatedMLP(Part):
+    replayable = True
+
     def __init__(self, *, rt: Runtime, width: int, prefix: str, intermediate_size: int, activation: str = "silu",
                  names: Optional[Dict[str, str]] = None):
         if activation != "silu":

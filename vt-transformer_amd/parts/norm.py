@@ -18,6 +18,8 @@ from .base import NORMS, Part, Runtime, TensorDecl
 
 @NORMS.register("rmsnorm")
 class RMSNorm(Part):
+    replayable = True
+
     def __init__(self, *, rt: Runtime, width: int, prefix: str, eps: float, name: str = "weight", scratch: str = "norm"):
         self.rt = rt
         self.width = int(width)

@@ -33,6 +33,8 @@ def rotary_table(n_positions: int, dims: int, theta: float) -> Tuple[np.ndarray,
 
 @POSITIONS.register("rotary")
 class RotaryEncoding(Part):
+    replayable = True
+
     def __init__(self, *, rt: Runtime, theta: float, dim: int):
         if dim % 2:
             raise ValueError(f"rotary dims {dim} must be even")
@@ -51,6 +53,8 @@ class RotaryEncoding(Part):
 
 @POSITIONS.register("none")
 class NoPositionEncoding(Part):
+    replayable = True
+
     """Queries and keys as they are."""
 
     def __init__(self, *, rt: Runtime):
