@@ -312,7 +312,8 @@ ATT_TOL = {torch.float32: 1e-5, torch.bfloat16: 1.5e-2}
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("nh,kvh,d", [(4, 2, 16), (3, 3, 32), (5, 1, 48), (14, 2, 64), (7, 7, 80), (28, 4, 128), (2, 1, 256)])
+@pytest.mark.parametrize("nh,kvh,d", [(4, 2, 16), (3, 3, 32), (5, 1, 48), (14, 2, 64), (7, 7, 80), (28, 4, 128), (6, 2, 144),
+                                      (2, 1, 256)])
 def test_attention_mixed_batch(dtype, nh, kvh, d):
     # a whole prompt, a decoded token with a long cache, a portion in the middle of a prompt, a first token
     entries = [(0, 37), (300, 1), (45, 19), (0, 1), (16, 2)]
@@ -486,7 +487,7 @@ def test_sample_top_k_and_top_p():
     assert set(_draw(logits, 5.0, 1, 1.0, 100, 4).tolist()) == {int(order[0])}
 
 
-@pytest.mark.parametrize("nh,kvh,d", [(28, 4, 128), (4, 2, 16), (16, 1, 48)])
+@pytest.mark.parametrize("nh,kvh,d", [(28, 4, 128), (4, 2, 16), (16, 1, 48), (6, 2, 144)])   # 144: nine tiles of 16 dims
 @pytest.mark.parametrize("window", [0, 37])
 @pytest.mark.parametrize("chunk", [64, 128, 1024])
 def test_attention_decode_kernel(nh, kvh, d, window, chunk):
@@ -515,7 +516,8 @@ def test_attention_decode_kernel(nh, kvh, d, window, chunk):
     assert rel_err(out, ref) < ATT_TOL[torch.bfloat16]
 
 
-@pytest.mark.parametrize("nh,kvh,d,rot", [(28, 4, 128, 128), (4, 2, 64, 32), (6, 2, 80, 0), (16, 1, 256, 256), (3, 1, 48, 32)])
+@pytest.mark.parametrize("nh,kvh,d,rot", [(28, 4, 128, 128), (4, 2, 64, 32), (6, 2, 80, 0), (16, 1, 256, 256), (3, 1, 48, 32),
+                                          (6, 2, 256, 256), (6, 2, 144, 128)])
 @pytest.mark.parametrize("window", [0, 37])
 @pytest.mark.parametrize("chunk", [64, 1024])
 def test_attention_decode_fused_kernel(nh, kvh, d, rot, window, chunk):

@@ -219,11 +219,11 @@ __device__ __forceinline__ void rotated_chunk(float (&x)[CH], const float* row, 
         for (int i = 0; i < CH; i += 4) {
             const float4 y = *(const float4*)(other + i), cc = *(const float4*)(ct + i), sn = *(const float4*)(st + i);
             if (low) {
-                x[i] = cc.x * x[i] - sn.x * y.x; x[i + 1] = cc.y * x[i + 1] - sn.y * y.y;
-                x[i + 2] = cc.z * x[i + 2] - sn.z * y.z; x[i + 3] = cc.w * x[i + 3] - sn.w * y.w;
+                x[i] = rotate_low(cc.x, sn.x, x[i], y.x); x[i + 1] = rotate_low(cc.y, sn.y, x[i + 1], y.y);
+                x[i + 2] = rotate_low(cc.z, sn.z, x[i + 2], y.z); x[i + 3] = rotate_low(cc.w, sn.w, x[i + 3], y.w);
             } else {
-                x[i] = cc.x * x[i] + sn.x * y.x; x[i + 1] = cc.y * x[i + 1] + sn.y * y.y;
-                x[i + 2] = cc.z * x[i + 2] + sn.z * y.z; x[i + 3] = cc.w * x[i + 3] + sn.w * y.w;
+                x[i] = rotate_high(cc.x, sn.x, x[i], y.x); x[i + 1] = rotate_high(cc.y, sn.y, x[i + 1], y.y);
+                x[i + 2] = rotate_high(cc.z, sn.z, x[i + 2], y.z); x[i + 3] = rotate_high(cc.w, sn.w, x[i + 3], y.w);
             }
         }
     }
@@ -470,7 +470,9 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_kernel(AttnArg
     if constexpr (DECODE) {
         // The four waves hold partial results over disjoint keys of the same rows: merge them through LDS, half
         // of a large head at a time, and let all 256 threads write the result.
-        constexpr int DH = (D > 128) ? D / 2 : D;
+        // (a large head in two passes of TH tiles of 16 dims; the second pass is a tile shorter when DT is odd)
+        constexpr int TH = (D > 128) ? (DT + 1) / 2 : DT;
+        constexpr int DH = TH * 16;
         __syncthreads();            // every wave is done with its key/value buffer: the merge takes the memory over
         float (*so)[16][DH + 4] = (float (*)[16][DH + 4])wave_lds;
         static_assert(4 * 16 * (DH + 4) * 4 <= 4 * KV_LDS_ELEMS * 2, "the merge fits where the waves' buffers were");
@@ -481,13 +483,15 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_kernel(AttnArg
         if (g == 0) { sm[wv][r] = m[0]; sl[wv][r] = lt; }
         const int n_valid = min(16, n_rows);
 #pragma unroll
-        for (int half = 0; half < D / DH; ++half) {
+        for (int half = 0; half * TH < DT; ++half) {
             if (half) __syncthreads();
+            const int dims = min(DH, D - half * DH);      // dims of this pass
 #pragma unroll
-            for (int t = 0; t < DH / 16; ++t) *(f32x4_t*)&so[wv][r][t * 16 + 4 * g] = o[0][half * (DH / 16) + t];
+            for (int t = 0; t < TH; ++t)
+                if (half * TH + t < DT) *(f32x4_t*)&so[wv][r][t * 16 + 4 * g] = o[0][half * TH + t];
             __syncthreads();
-            for (int idx = threadIdx.x; idx < n_valid * DH; idx += 256) {
-                const int rr = idx / DH, dd = idx - rr * DH;
+            for (int idx = threadIdx.x; idx < n_valid * dims; idx += 256) {
+                const int rr = idx / dims, dd = idx - rr * dims;
                 const float mx = fmaxf(fmaxf(sm[0][rr], sm[1][rr]), fmaxf(sm[2][rr], sm[3][rr]));
                 float num = 0.f, den = 0.f;
 #pragma unroll

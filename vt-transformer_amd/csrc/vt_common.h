@@ -106,3 +106,9 @@ __device__ __forceinline__ float block_max(float v, float* red) {
     for (int i = 1; i < nw; ++i) t = fmaxf(t, red[i]);
     return t;
 }
+
+// One pair of a rotary encoding, x with its partner y: the low element is c x - s y, the high one c x + s y.  Every
+// kernel that rotates goes through these two, with the product and the fused multiply-add spelled out, so that
+// all of them round alike whatever the compiler would contract on its own.
+__device__ __forceinline__ float rotate_low(float c, float s, float x, float y) { return __fmaf_rn(c, x, -__fmul_rn(s, y)); }
+__device__ __forceinline__ float rotate_high(float c, float s, float x, float y) { return __fmaf_rn(c, x, __fmul_rn(s, y)); }

@@ -374,10 +374,10 @@ __global__ void rope_store_kernel(RopeStoreArgs a) {
         if (!is_v && i < a.rot) {
             if (i < half) {
                 float y = load_f32<TI>(in, i + half);
-                o = c[i] * x - s[i] * y;
+                o = rotate_low(c[i], s[i], x, y);
             } else {
                 float y = load_f32<TI>(in, i - half);
-                o = c[i - half] * x + s[i - half] * y;
+                o = rotate_high(c[i - half], s[i - half], x, y);
             }
         }
         if (is_q) {
@@ -420,10 +420,12 @@ __global__ __launch_bounds__(256) void rope_store_vec_kernel(RopeStoreArgs a) {
         if (!is_v && i < a.rot) {
             if (i < half) {
                 float4 y = load4(hp + i + half), cc = load4(c + i), sn = load4(s + i);
-                o = make_float4(cc.x * x.x - sn.x * y.x, cc.y * x.y - sn.y * y.y, cc.z * x.z - sn.z * y.z, cc.w * x.w - sn.w * y.w);
+                o = make_float4(rotate_low(cc.x, sn.x, x.x, y.x), rotate_low(cc.y, sn.y, x.y, y.y), rotate_low(cc.z, sn.z, x.z, y.z),
+                                rotate_low(cc.w, sn.w, x.w, y.w));
             } else {
                 float4 y = load4(hp + i - half), cc = load4(c + i - half), sn = load4(s + i - half);
-                o = make_float4(cc.x * x.x + sn.x * y.x, cc.y * x.y + sn.y * y.y, cc.z * x.z + sn.z * y.z, cc.w * x.w + sn.w * y.w);
+                o = make_float4(rotate_high(cc.x, sn.x, x.x, y.x), rotate_high(cc.y, sn.y, x.y, y.y), rotate_high(cc.z, sn.z, x.z, y.z),
+                                rotate_high(cc.w, sn.w, x.w, y.w));
             }
         }
         if (is_q) {
