@@ -561,6 +561,17 @@ def test_attention_decode_fused_kernel(nh, kvh, d, rot, window, chunk):
         assert rel_err(out, out_ref.float().cpu()) < 2e-3                 # the same products, merged in the same order
 
 
+@pytest.mark.parametrize("d", list(range(16, 257, 16)))
+def test_attention_every_head_size(d):
+    """Every head size the kernels are compiled for, through every bfloat16 attention kernel: portions (per-wave and
+    tiled, keys split and unsplit), decoding, and decoding that rotates and writes the pages itself."""
+    entries = [(0, 37), (300, 1), (45, 19), (0, 1), (16, 2), (0, 150)]
+    got, ref = attention_case(torch.bfloat16, 6, 2, d, 16, 0, entries, seed=d)
+    assert rel_err(got, ref) < ATT_TOL[torch.bfloat16]
+    test_attention_decode_kernel(6, 2, d, 37, 128)
+    test_attention_decode_fused_kernel(6, 2, d, d if d % 32 == 0 else d - 16, 0, 64)
+
+
 @pytest.mark.parametrize("n,m,k", [(1, 48, 64), (8, 3584, 3584), (16, 100, 200), (5, 4608, 1000), (3, 40, 24)])
 def test_linear_bf16_with_norm_in_front_and_residual_behind(n, m, k):
     """The few-row product that applies an RMSNorm to its input on the way and adds its result to the residual

@@ -31,7 +31,7 @@ FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC", "-shared",
 
 # libraries that every model needs; attention for bf16 is built per head size
 BASE_LIBS = ["vt_elementwise", "vt_gemm_f32", "vt_gemm_bf16", "vt_attn_f32", "vt_sampling"]
-DEFAULT_HEAD_DIMS = [16, 32, 48, 64, 80, 96, 128, 144, 256]
+DEFAULT_HEAD_DIMS = list(range(16, 257, 16))
 
 
 class KernelBuildError(RuntimeError):
