@@ -1,0 +1,61 @@
+"""Configurations drawn at random (heads, groups, head sizes in steps of 16, widths and vocabularies that are no
+power of two, windows on some layers, eps, tied or untied head): the engine against the plain implementation, whole,
+cut at random, decoded one by one, and decoded through captured graphs."""
+import numpy as np
+import pytest
+import torch
+
+import plain_model
+
+pytestmark = pytest.mark.gpu
+
+
+def draw_config(seed: int) -> dict:
+    rs = np.random.RandomState(seed)
+    kvh = int(rs.choice([1, 2, 3, 4]))
+    group = int(rs.choice([1, 2, 3, 5, 7, 8, 16]))
+    d = int(rs.choice(range(16, 257, 16)))
+    if kvh * group * d > 4096:
+        group = max(1, 4096 // (kvh * d))
+    layers = int(rs.randint(1, 5))
+    return dict(architectures=["Qwen2ForCausalLM"], model_type="qwen2", vocab_size=int(rs.choice([97, 203, 320, 1001, 4099])),
+                hidden_size=int(rs.choice([40, 72, 96, 104, 120, 200, 328])), intermediate_size=int(rs.choice([56, 88, 136, 200, 520])),
+                num_hidden_layers=layers, num_attention_heads=kvh * group, num_key_value_heads=kvh, head_dim=d,
+                rope_theta=float(rs.choice([1e4, 5e4, 1e6])), rms_norm_eps=float(rs.choice([1e-6, 1e-5, 3e-3])),
+                tie_word_embeddings=bool(rs.rand() < 0.5), max_position_embeddings=1024, hidden_act="silu",
+                use_sliding_window=bool(rs.rand() < 0.4), sliding_window=int(rs.choice([5, 17, 40, 64])),
+                max_window_layers=int(rs.randint(0, layers + 1)), torch_dtype="bfloat16")
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_configuration(seed, tmp_path):
+    from vt_transformer_amd.config import config_from_dict
+    from vt_transformer_amd.engine import StepEntry, load_model, make_runner
+    from vt_transformer_amd.weights import write_random_model
+    cfg = draw_config(100 + seed)
+    folder = str(tmp_path / "m")
+    write_random_model(config_from_dict(cfg), folder, seed=seed)
+    pcfg, w = plain_model.read_folder(folder)
+    rs = np.random.RandomState(seed)
+    n = int(rs.randint(70, 200))
+    toks = rs.randint(0, cfg["vocab_size"], size=n).tolist()
+    ref = plain_model.forward(pcfg, w, toks)
+    for dtype, tol in (("float32", 3e-5), ("bfloat16", 4e-2)):
+        model = load_model(folder, dtype)
+        for mode in ("whole", "cut", "decode", "graph"):
+            runner = make_runner(model, pool_tokens=-(-n // 16) * 16 + 32, page_size=16, max_requests=2, max_seq_len=512)
+            runner.decode_graphs = mode == "graph"
+            runner.admit("r")
+            if mode == "whole":
+                cuts = [(0, n)]
+            elif mode == "cut":
+                cuts, a = [], 0
+                while a < n:
+                    b = min(n, a + int(rs.choice([2, 3, 5, 16, 17, 31, 64])))
+                    cuts.append((a, b))
+                    a = b
+            else:
+                cuts = [(0, n - 32)] + [(i, i + 1) for i in range(n - 32, n)]
+            got = torch.cat([runner.step([StepEntry("r", toks[a:b], list(range(b - a)))]).float().cpu() for a, b in cuts])
+            err = float((got.double() - ref).abs().max() / ref.abs().max())
+            assert err < tol, (cfg, dtype, mode, err)
