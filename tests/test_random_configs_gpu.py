@@ -6,6 +6,7 @@ import pytest
 import torch
 
 import plain_model
+from replay_helpers import check_against_plain, cut, max_live_tokens, random_requests, run_in_process, trace_mixed
 
 pytestmark = pytest.mark.gpu
 
@@ -59,3 +60,15 @@ def test_random_configuration(seed, tmp_path):
             got = torch.cat([runner.step([StepEntry("r", toks[a:b], list(range(b - a)))]).float().cpu() for a, b in cuts])
             err = float((got.double() - ref).abs().max() / ref.abs().max())
             assert err < tol, (cfg, dtype, mode, err)
+        # several requests at a time, portions of some beside decoded tokens of others, pages used again
+        reqs = random_requests(cfg["vocab_size"], [int(x) for x in rs.randint(1, 70, size=7)], seed=seed)
+        portions = {}
+        for r, t in reqs.items():
+            n_head = max(0, len(t) - int(rs.randint(1, 10)))
+            parts = cut(t[:n_head], [int(x) for x in rs.choice([2, 3, 5, 8, 11, 16, 17], size=2)]) if n_head else []
+            portions[r] = parts + [(j, j + 1) for j in range(n_head, len(t))]
+        steps = trace_mixed(reqs, portions, max_live=4, seed=seed)
+        runner = make_runner(model, pool_tokens=max_live_tokens(steps), page_size=16, max_requests=4, max_seq_len=512)
+        runner.decode_graphs = True
+        check_against_plain(folder, reqs, steps, run_in_process(runner, steps), dtype)
+        assert sum(runner.cache.held_pages()) == 0
