@@ -236,6 +236,18 @@ __device__ __forceinline__ void merge_parts(float (*sm)[16], float (*sl)[16], co
                                             bf16_t* out, size_t slot0, size_t slot_step, int n_parts, int n_valid,
                                             int q_tok0, int q_row0, int G, int kvh, int n_heads) {
     const int tid = threadIdx.x;
+    // With few rows and parts (decoding) a thread's share of the partial outputs is on its way from memory while
+    // the weights of the parts are worked out, instead of being asked for only after them.
+    constexpr int PRE = 16, Q = D / 4;
+    const bool pre = n_valid * Q <= 256 && n_parts <= PRE;
+    const int pr = tid / Q, pd = (tid - pr * Q) * 4;
+    f32x4_t pv[PRE];
+    if (pre && tid < n_valid * Q) {
+        const float* po = part_o + (slot0 + pr) * D + pd;
+#pragma unroll
+        for (int pi = 0; pi < PRE; ++pi)
+            if (pi < n_parts) pv[pi] = *(const f32x4_t*)(po + (size_t)pi * slot_step * D);
+    }
     for (int i = tid; i < n_parts * 16; i += 256) {
         const int pi = i >> 4, r = i & 15;
         const size_t sl_ = slot0 + pi * slot_step + r;
@@ -257,6 +269,21 @@ __device__ __forceinline__ void merge_parts(float (*sm)[16], float (*sl)[16], co
         for (int pi = 0; pi < n_parts; ++pi) sm[pi][tid] *= inv;
     }
     __syncthreads();
+    if (pre) {
+        if (tid < n_valid * Q) {
+            f32x4_t acc = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int pi = 0; pi < PRE; ++pi)
+                if (pi < n_parts) acc += sm[pi][pr] * pv[pi];     // parts in order, as below
+            const int row = q_row0 + pr;
+            const int ti = row / G, head = kvh * G + (row - ti * G);
+            uint2 w;
+            w.x = pack2(acc[0], acc[1]);
+            w.y = pack2(acc[2], acc[3]);
+            *(uint2*)(out + ((size_t)(q_tok0 + ti) * n_heads + head) * D + pd) = w;
+        }
+        return;
+    }
     for (int idx = tid; idx < n_valid * D; idx += 256) {
         const int r = idx / D, d = idx - r * D;
         const float* po = part_o + (slot0 + r) * D + d;
