@@ -100,8 +100,14 @@ __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(float* __restrict__ h,
     float* hr = h + src * hidden;
     const TD* dr = HAS_DELTA ? delta + src * hidden : nullptr;
     const int nq = hidden >> 2;
-    float4 x[NV];
+    float4 x[NV], gn[NV];
     float ss = 0.f;
+    // the gains are asked for together with the values, not after the sum: one trip to memory instead of two
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        const int qi = tid + v * 256;
+        if (qi < nq) gn[v] = load4(gain + 4 * qi);
+    }
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
         const int qi = tid + v * 256;
@@ -122,7 +128,7 @@ __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(float* __restrict__ h,
     for (int v = 0; v < NV; ++v) {
         const int qi = tid + v * 256;
         if (qi < nq) {
-            float4 g = load4(gain + 4 * qi);
+            const float4 g = gn[v];
             store4(o + 4 * qi, make_float4((g.x * x[v].x) * rinv, (g.y * x[v].y) * rinv, (g.z * x[v].z) * rinv,
                                            (g.w * x[v].w) * rinv));
         }
