@@ -203,29 +203,32 @@ __device__ __forceinline__ void park_block(const KVBlock& b, bf16_t* kl, int lan
 template <int CH>
 __device__ __forceinline__ void rotated_chunk(float (&x)[CH], const float* row, int c, int rot, const float* cos_t,
                                               const float* sin_t, int pos, int max_pos) {
+    if (rot == 0) {     // (the same for every lane and every call of a launch: no tables to read from)
+#pragma unroll
+        for (int i = 0; i < CH; i += 4) {
+            const float4 v = *(const float4*)(row + c + i);
+            x[i] = v.x; x[i + 1] = v.y; x[i + 2] = v.z; x[i + 3] = v.w;
+        }
+        return;
+    }
+    // No load below sits under a test of c: a chunk outside the rotary dims reads its own elements and the tables'
+    // first entries and drops them.  So the loads of all the chunks of a row are in flight together; under
+    // branches every chunk would wait for its own before the next one's could start.
+    const int half = rot >> 1;
+    const bool in = c < rot, low = c < half;
+    const int tp = pos < max_pos ? (pos < 0 ? 0 : pos) : max_pos - 1;
+    const int ti = in ? (low ? c : c - half) : 0;
+    const float* ct = cos_t + (size_t)tp * half + ti;
+    const float* st = sin_t + (size_t)tp * half + ti;
+    const float* other = row + (in ? (low ? c + half : c - half) : c);
 #pragma unroll
     for (int i = 0; i < CH; i += 4) {
         const float4 v = *(const float4*)(row + c + i);
-        x[i] = v.x; x[i + 1] = v.y; x[i + 2] = v.z; x[i + 3] = v.w;
-    }
-    if (c < rot) {
-        const int half = rot >> 1;
-        const bool low = c < half;
-        const int tp = pos < max_pos ? (pos < 0 ? 0 : pos) : max_pos - 1;
-        const float* ct = cos_t + (size_t)tp * half + (low ? c : c - half);
-        const float* st = sin_t + (size_t)tp * half + (low ? c : c - half);
-        const float* other = row + (low ? c + half : c - half);
-#pragma unroll
-        for (int i = 0; i < CH; i += 4) {
-            const float4 y = *(const float4*)(other + i), cc = *(const float4*)(ct + i), sn = *(const float4*)(st + i);
-            if (low) {
-                x[i] = rotate_low(cc.x, sn.x, x[i], y.x); x[i + 1] = rotate_low(cc.y, sn.y, x[i + 1], y.y);
-                x[i + 2] = rotate_low(cc.z, sn.z, x[i + 2], y.z); x[i + 3] = rotate_low(cc.w, sn.w, x[i + 3], y.w);
-            } else {
-                x[i] = rotate_high(cc.x, sn.x, x[i], y.x); x[i + 1] = rotate_high(cc.y, sn.y, x[i + 1], y.y);
-                x[i + 2] = rotate_high(cc.z, sn.z, x[i + 2], y.z); x[i + 3] = rotate_high(cc.w, sn.w, x[i + 3], y.w);
-            }
-        }
+        const float4 y = *(const float4*)(other + i), cc = *(const float4*)(ct + i), sn = *(const float4*)(st + i);
+        x[i] = in ? rotate_pair(cc.x, sn.x, v.x, y.x, low) : v.x;
+        x[i + 1] = in ? rotate_pair(cc.y, sn.y, v.y, y.y, low) : v.y;
+        x[i + 2] = in ? rotate_pair(cc.z, sn.z, v.z, y.z, low) : v.z;
+        x[i + 3] = in ? rotate_pair(cc.w, sn.w, v.w, y.w, low) : v.w;
     }
 }
 

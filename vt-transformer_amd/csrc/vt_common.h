@@ -112,3 +112,8 @@ __device__ __forceinline__ float block_max(float v, float* red) {
 // all of them round alike whatever the compiler would contract on its own.
 __device__ __forceinline__ float rotate_low(float c, float s, float x, float y) { return __fmaf_rn(c, x, -__fmul_rn(s, y)); }
 __device__ __forceinline__ float rotate_high(float c, float s, float x, float y) { return __fmaf_rn(c, x, __fmul_rn(s, y)); }
+// the one or the other by a flag, without a branch (the same bits: only the product's sign differs)
+__device__ __forceinline__ float rotate_pair(float c, float s, float x, float y, bool low) {
+    const float p = __fmul_rn(s, y);
+    return __fmaf_rn(c, x, low ? -p : p);
+}
