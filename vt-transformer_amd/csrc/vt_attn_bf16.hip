@@ -232,6 +232,46 @@ __device__ __forceinline__ void rotated_chunk(float (&x)[CH], const float* row, 
     }
 }
 
+// The same in two steps, so that the loads of several chunks are in flight together: the compiler keeps a chunk's
+// loads next to its arithmetic, and a row's chunks then wait for memory one after the other.
+template <int CH>
+struct RotIn {
+    float4 x[CH / 4], y[CH / 4], c[CH / 4], s[CH / 4];
+    bool in, low;
+};
+template <int CH>
+__device__ __forceinline__ void rot_load(RotIn<CH>& r, const float* row, int c, int rot, const float* cos_t,
+                                         const float* sin_t, int pos, int max_pos) {
+    // nothing here sits under a test: a chunk outside the rotary dims (all of them if there are none) reads its own
+    // elements again in place of a partner and of table entries, and drops them
+    const int half = rot >> 1;
+    r.in = c < rot;
+    r.low = c < half;
+    const int tp = pos < max_pos ? (pos < 0 ? 0 : pos) : max_pos - 1;
+    const int ti = r.low ? c : c - half;
+    const float* ct = r.in ? cos_t + (size_t)tp * half + ti : row + c;
+    const float* st = r.in ? sin_t + (size_t)tp * half + ti : row + c;
+    const float* other = row + (r.in ? (r.low ? c + half : c - half) : c);
+#pragma unroll
+    for (int i = 0; i < CH / 4; ++i) {
+        r.x[i] = *(const float4*)(row + c + 4 * i);
+        r.y[i] = *(const float4*)(other + 4 * i);
+        r.c[i] = *(const float4*)(ct + 4 * i);
+        r.s[i] = *(const float4*)(st + 4 * i);
+    }
+}
+template <int CH>
+__device__ __forceinline__ void rot_apply(float (&x)[CH], const RotIn<CH>& r) {
+#pragma unroll
+    for (int i = 0; i < CH / 4; ++i) {
+        const float4 v = r.x[i], y = r.y[i], cc = r.c[i], sn = r.s[i];
+        x[4 * i] = r.in ? rotate_pair(cc.x, sn.x, v.x, y.x, r.low) : v.x;
+        x[4 * i + 1] = r.in ? rotate_pair(cc.y, sn.y, v.y, y.y, r.low) : v.y;
+        x[4 * i + 2] = r.in ? rotate_pair(cc.z, sn.z, v.z, y.z, r.low) : v.z;
+        x[4 * i + 3] = r.in ? rotate_pair(cc.w, sn.w, v.w, y.w, r.low) : v.w;
+    }
+}
+
 // Merge the partial results of a tile of 16 rows whose keys were split over n_parts items; all 256 threads of a
 // block.  sm and sl are [MAX_PARTS][16] floats of LDS.  Slot of (part pi, row r) = slot0 + pi * slot_step + r.
 #define MAX_PARTS 128
@@ -364,16 +404,27 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_kernel(AttnArg
             // the query as the projection left it: rotate its pairs (i, i + rot/2) by the angles of its position
             const float* qrow = a.qkv + (size_t)q_tok0 * a.qkv_stride + (size_t)head[rt] * D;
             constexpr int CH = WIDE ? 8 : 4, STEP = WIDE ? 32 : 16;
+            constexpr int QB = (WIDE ? 4 : 8) < QSTEPS ? (WIDE ? 4 : 8) : QSTEPS;     // chunks whose loads fly together
 #pragma unroll
-            for (int s = 0; s < QSTEPS; ++s) {
-                float x[CH];
-                rotated_chunk<CH>(x, qrow, s * STEP + g * CH, a.rot, a.cos_t, a.sin_t, pos0, a.max_pos);
-                if constexpr (WIDE) {
-                    U16 t; t.u = make_uint4(pack2(x[0], x[1]), pack2(x[2], x[3]), pack2(x[4], x[5]), pack2(x[6], x[7]));
-                    q8[rt][s] = t.v;
-                } else {
-                    U8 t; t.u = make_uint2(pack2(x[0], x[1]), pack2(x[2], x[3]));
-                    q4[rt][s] = t.v;
+            for (int s0 = 0; s0 < QSTEPS; s0 += QB) {
+                RotIn<CH> rin[QB];
+#pragma unroll
+                for (int u = 0; u < QB; ++u)
+                    if (s0 + u < QSTEPS)
+                        rot_load<CH>(rin[u], qrow, (s0 + u) * STEP + g * CH, a.rot, a.cos_t, a.sin_t, pos0, a.max_pos);
+                __builtin_amdgcn_sched_barrier(0);      // all of them asked for before the first is used
+#pragma unroll
+                for (int u = 0; u < QB; ++u) {
+                    if (s0 + u >= QSTEPS) continue;
+                    float x[CH];
+                    rot_apply<CH>(x, rin[u]);
+                    if constexpr (WIDE) {
+                        U16 t; t.u = make_uint4(pack2(x[0], x[1]), pack2(x[2], x[3]), pack2(x[4], x[5]), pack2(x[6], x[7]));
+                        q8[rt][s0 + u] = t.v;
+                    } else {
+                        U8 t; t.u = make_uint2(pack2(x[0], x[1]), pack2(x[2], x[3]));
+                        q4[rt][s0 + u] = t.v;
+                    }
                 }
             }
         } else {
