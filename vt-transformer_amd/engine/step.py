@@ -264,10 +264,10 @@ def decode_bucket(n_kv: int) -> int:
     return min(DECODE_BUCKETS - 1, max(1, int(n_kv)).bit_length() - 1)
 
 
-def decode_chunk(kv_lens: np.ndarray, p_max: int, n_kv: int = 4, want_blocks: int = 512, min_chunk: int = 64) -> int:
+def decode_chunk(kv_lens: np.ndarray, p_max: int, n_kv: int = 4, want_blocks: int = 768, min_chunk: int = 64) -> int:
     """Keys per attention item of a decoding step.  A block of four waves takes one item of one (entry, kv head);
     with enough entries every entry is one item, otherwise the keys are cut so that about `want_blocks` blocks
-    run, never into more than p_max items; a multiple of 64 (the four waves take 16 keys each in turn)."""
+    run (three to a compute unit: measured inside whole decoding steps, where the keys come from memory), never into more than p_max items; a multiple of 64 (the four waves take 16 keys each in turn)."""
     pairs = max(1, len(kv_lens) * n_kv)
     splits = min(p_max, max(1, -(-want_blocks // pairs)))
     longest = int(kv_lens.max())
