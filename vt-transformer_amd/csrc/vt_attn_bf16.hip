@@ -35,9 +35,6 @@ VT_DEFINE_LAST_ERROR()
 static_assert(VT_HEAD_DIM % 16 == 0 && VT_HEAD_DIM >= 16 && VT_HEAD_DIM <= 256, "head size must be 16..256 in steps of 16");
 
 #define D VT_HEAD_DIM
-#ifndef VT_ATTN_RING
-#define VT_ATTN_RING 2          // key/value blocks of 16 keys in registers per wave: one multiplied, the others in flight
-#endif
 #define ITEM_INTS 8  // entry, q_tok0, q_len, pos0, q_row0, key_lo, key_hi, part (-1: final)
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
@@ -477,9 +474,7 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_kernel(AttnArg
     extern __shared__ __attribute__((aligned(16))) bf16_t wave_lds[];
     bf16_t* const kl = wave_lds + wv * KV_LDS_ELEMS;      // this wave's buffer: keys, then values
     const bf16_t* const vl = kl + 16 * KL_ROW;
-    auto multiply = [&](const KVBlock& cur, int j0) __attribute__((always_inline)) {
-        if (!cur.ok) return;
-        park_block(cur, kl, lane);
+    auto compute = [&](int j0) __attribute__((always_inline)) {
         wave_lds_order();
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
@@ -517,12 +512,12 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_kernel(AttnArg
         }
         wave_lds_order();       // the next block is parked after these reads
     };
-    // A ring of register buffers: while one block is multiplied the next NB - 1 are on their way from memory, and
-    // the page id of the one after them comes from the block table (a scalar load).  Every turn loads, whether or
-    // not keys are left (then the wave's last block again, which nobody multiplies), so that the number of loads
-    // in flight is the same on every path through the loop.
-    constexpr int NB = VT_ATTN_RING;
-    KVBlock ring[NB];
+    // One register buffer: a block is parked in LDS as soon as it has arrived, the next one is asked for into the
+    // same registers at once and is on its way while this one is multiplied; the page id of the one after comes
+    // from the block table meanwhile (a scalar load).  Every turn loads, whether or not keys are left (then the
+    // wave's last block again, which nobody multiplies), so that no load sits under a branch.  (Two and three
+    // buffers were slower inside whole decoding steps.)
+    KVBlock cur;
     const int j_first = key_lo + (DECODE ? 16 * wv : 0), j_step = DECODE ? 64 : 16;
     // the last block this wave may read: the last one of its own, or for a wave without keys the item's first
     const int j_end = j_first < key_hi ? j_first + (key_hi - 1 - j_first) / j_step * j_step : key_lo;
@@ -533,19 +528,15 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_kernel(AttnArg
     auto page_at = [&](int j) __attribute__((always_inline)) { return btc[min(page_index(a, min(j, j_end)), last_page)]; };
     const int spare = min(max(btc[last_page], 0), a.num_pages - 1);
     int pg_next;                     // page of the next block to load
-#pragma unroll
-    for (int i = 0; i < NB - 1; ++i) load_block(ring[i], a, page_at(j_first + i * j_step), spare, min(j_first + i * j_step, j_end), kvh, lane);
-    pg_next = page_at(j_first + (NB - 1) * j_step);
-    for (int j0 = j_first; j0 < key_hi; j0 += NB * j_step) {
-#pragma unroll
-        for (int ph = 0; ph < NB; ++ph) {
-            const int j = j0 + ph * j_step;
-            if (j >= key_hi) break;
-            load_block(ring[(ph + NB - 1) % NB], a, pg_next, spare, min(j + (NB - 1) * j_step, j_end), kvh, lane);
-            pg_next = page_at(j + NB * j_step);
-            __builtin_amdgcn_sched_barrier(0);      // the loads stay here, ahead of this block's products
-            multiply(ring[ph], j);
-        }
+    load_block(cur, a, page_at(j_first), spare, min(j_first, j_end), kvh, lane);
+    pg_next = page_at(j_first + j_step);
+    for (int j = j_first; j < key_hi; j += j_step) {
+        const bool ok = cur.ok;
+        if (ok) park_block(cur, kl, lane);
+        load_block(cur, a, pg_next, spare, min(j + j_step, j_end), kvh, lane);
+        pg_next = page_at(j + 2 * j_step);
+        __builtin_amdgcn_sched_barrier(0);
+        if (ok) compute(j);
     }
 
     if constexpr (DECODE) {
