@@ -123,7 +123,7 @@ def test_linear_f32_is_true_fp32_and_batch_invariant():
     assert torch.equal(one[0], big[11])
 
 
-@pytest.mark.parametrize("n", [1, 3, 16, 17, 33, 64, 100])
+@pytest.mark.parametrize("n", [1, 3, 16, 17, 33, 64, 100, 300])
 @pytest.mark.parametrize("m,k", [(320, 96), (200, 200), (1030, 3584), (96, 18944 // 8)])
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
 def test_linear_bf16(n, m, k, out_dtype):
@@ -189,7 +189,7 @@ def test_linear_bf16_batch_invariant():
     assert rel_err(small, full[:16]) < 1e-5
 
 
-@pytest.mark.parametrize("n", [1, 9, 40, 64])
+@pytest.mark.parametrize("n", [1, 9, 40, 64, 300])
 @pytest.mark.parametrize("inter,k", [(200, 96), (128, 64), (1184, 3584), (18944, 40), (22016, 32), (29568, 24)])
 def test_gated_linear_bf16(n, inter, k):
     # the three wide ones make the 64-token kernel take 5, 6 and 8 waves a block

@@ -64,6 +64,8 @@ def build_parser() -> argparse.ArgumentParser:
     p.add_argument("--chunk-size", type=int, default=2048)
     p.add_argument("--no-decode-graphs", action="store_true")
     p.add_argument("--tune-gemm", action="store_true", help="let the GEMM library search its algorithms at start-up (seconds)")
+    p.add_argument("--single-weight-copy", action="store_true",
+                   help="keep the bfloat16 matrices once instead of twice (half the memory, slower prompts)")
     # random weights
     p.add_argument("--write-random-model", type=str, metavar="DIR", help="write config.json and model.safetensors with random weights")
     p.add_argument("--config", type=str, help="config.json for --write-random-model")
@@ -115,7 +117,8 @@ def main(argv: Optional[List[str]] = None) -> int:
     eng = Engine(args.model, dtype=args.dtype, seed=args.seed, max_running_reqs=args.max_running_reqs,
                  num_pages=num_pages, max_seq_len=args.max_seq_len, page_size=args.page_size,
                  max_extend_tokens=args.max_extend_tokens, default_max_output=args.default_max_output,
-                 chunk_size=args.chunk_size, decode_graphs=not args.no_decode_graphs, tune_gemm=args.tune_gemm)
+                 chunk_size=args.chunk_size, decode_graphs=not args.no_decode_graphs, tune_gemm=args.tune_gemm,
+                 single_weight_copy=args.single_weight_copy)
 
     def params() -> SamplingParams:
         return SamplingParams(temperature=temperature, top_k=top_k, top_p=top_p, ignore_eos=args.ignore_eos,

@@ -26,21 +26,23 @@ class Engine:
     def __init__(self, model: Optional[str] = None, *, config: Optional[ModelConfig] = None,
                  random_weights_seed: Optional[int] = None, dtype: str = "bfloat16", seed: int = 0,
                  scheduler_config: Optional[SchedulerConfig] = None, decode_graphs: bool = True,
-                 tune_gemm: bool = False, **options):
+                 tune_gemm: bool = False, single_weight_copy: bool = False, **options):
         """model: a folder with config.json and model.safetensors.  Or `config` with `random_weights_seed`
         for random weights drawn on the device.  `options` override fields of SchedulerConfig
         (max_running_reqs, num_pages, max_seq_len, page_size, max_extend_tokens, default_max_output, chunk_size).
         tune_gemm: let the GEMM library try its algorithms on this model's products at chunk_size rows once, at
-        start-up (some seconds), and use the fastest from then on."""
+        start-up (some seconds), and use the fastest from then on.
+        single_weight_copy: keep the bfloat16 matrices once (in the few-row kernels' order) instead of twice; long
+        prompt portions are then several times slower.  For models that fit the GPU's memory once but not twice."""
         sc = scheduler_config or SchedulerConfig()
         for k, v in options.items():
             if not hasattr(sc, k):
                 raise TypeError(f"unknown engine option '{k}'")
             setattr(sc, k, v)
         if model is not None:
-            self.model = load_model(model, dtype)
+            self.model = load_model(model, dtype, keep_row_major=not single_weight_copy)
         elif config is not None and random_weights_seed is not None:
-            self.model = random_model(config, random_weights_seed, dtype)
+            self.model = random_model(config, random_weights_seed, dtype, keep_row_major=not single_weight_copy)
         else:
             raise ValueError("give a model folder, or a config and random_weights_seed")
         spec = self.model.spec

@@ -28,22 +28,24 @@ def parse_dtype(name) -> torch.dtype:
         raise ValueError(f"dtype '{name}' is not supported (bfloat16 and float32 are)") from None
 
 
-def build_model(config: ModelConfig, dtype, device: Optional[torch.device] = None) -> DecoderModel:
+def build_model(config: ModelConfig, dtype, device: Optional[torch.device] = None,
+                keep_row_major: bool = True) -> DecoderModel:
     device = device or require_gpu()
-    return DecoderModel(config.to_spec(), Runtime(device, parse_dtype(dtype)))
+    return DecoderModel(config.to_spec(), Runtime(device, parse_dtype(dtype), keep_row_major))
 
 
-def load_model(folder: str, dtype, device: Optional[torch.device] = None) -> DecoderModel:
+def load_model(folder: str, dtype, device: Optional[torch.device] = None, keep_row_major: bool = True) -> DecoderModel:
     """config.json chooses the architecture; model.safetensors (or its shards) gives the tensors."""
-    model = build_model(load_config(folder), dtype, device)
+    model = build_model(load_config(folder), dtype, device, keep_row_major)
     load_model_weights(model, folder)
     return model
 
 
-def random_model(config: ModelConfig, seed: int, dtype, device: Optional[torch.device] = None) -> DecoderModel:
+def random_model(config: ModelConfig, seed: int, dtype, device: Optional[torch.device] = None,
+                 keep_row_major: bool = True) -> DecoderModel:
     """The same tensors that `write_random_model` would store for this seed's generator on this device,
     drawn on the device one at a time (a 145 GB model never exists on the host)."""
-    model = build_model(config, dtype, device)
+    model = build_model(config, dtype, device, keep_row_major)
     expected = model.tensors()
     rt = model.rt
 

@@ -99,6 +99,7 @@ class PagedAttention(Part):
         if self.out_bias:
             self.b_o = rt.place(get(nm["o"] + ".bias"), "bias")
         self.p_qkv, self.p_o = rt.pack(self.w_qkv), rt.pack(self.w_o)
+        self.w_qkv, self.w_o = rt.row_major(self.w_qkv, self.p_qkv), rt.row_major(self.w_o, self.p_o)
 
     # -- one step --------------------------------------------------------------
     def forward(self, x, ctx, cache, state=None, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -110,7 +111,7 @@ class PagedAttention(Part):
         else:  # keys and values of another layer: only queries are made
             bq = self.b_qkv[:nq] if self.b_qkv is not None else None
             bql = self.b_qkv_lowp[:nq] if self.b_qkv_lowp is not None else None
-            qkv = linear(rt, x, self.w_qkv[:nq], bq, "attn.qonly", bias_lowp=bql,
+            qkv = linear(rt, x, self.w_qkv[:nq] if self.w_qkv is not None else None, bq, "attn.qonly", bias_lowp=bql,
                          packed=self.p_qkv.first_rows(nq) if self.p_qkv is not None else None)
         tables = self.position.rotary_tables(ctx.n_positions)
         if tables is None and hasattr(self.position, "apply") and self.position.dim != 0:

@@ -71,11 +71,16 @@ class StateNeed:
 class Runtime:
     """Device, dtype and scratch buffers shared by the parts of one model."""
 
-    def __init__(self, device: torch.device, dtype: torch.dtype):
+    def __init__(self, device: torch.device, dtype: torch.dtype, keep_row_major: bool = True):
         if dtype not in (torch.bfloat16, torch.float32):
             raise ValueError(f"dtype {dtype} is not supported (bfloat16 and float32 are)")
         self.device = device
         self.dtype = dtype
+        # bfloat16 keeps every matrix twice: row-major for the GEMM library (long portions) and packed for the
+        # few-row kernels.  False: the packed copy only, and long portions go through the few-row kernels 64 rows
+        # at a time, which reads W once per 64 rows: several times slower on prompts, half the memory (a model
+        # that fits the GPU once but not twice).
+        self.keep_row_major = bool(keep_row_major) or dtype != torch.bfloat16
         self._buffers: Dict[str, torch.Tensor] = {}
         self._scope = ""
 
@@ -98,6 +103,10 @@ class Runtime:
             return None
         from ..kernels import ops
         return ops.pack_matrix_bf16(w, halves)
+
+    def row_major(self, w: torch.Tensor, packed) -> Optional[torch.Tensor]:
+        """The row-major matrix to keep beside its packed copy: `w`, or None where only the packed copy stays."""
+        return w if (self.keep_row_major or packed is None) else None
 
     def buffer(self, name: str, shape, dtype: torch.dtype) -> torch.Tensor:
         """A scratch tensor that keeps its address between steps (grown when a step needs more)."""

@@ -50,6 +50,7 @@ class GatedMLP(Part):
                                rt.place(get(nm["up"] + ".weight"), "matrix")], dim=0).contiguous()
         self.w_down = rt.place(get(nm["down"] + ".weight"), "matrix")
         self.p_gu, self.p_down = rt.pack(self.w_gu, halves=2), rt.pack(self.w_down)
+        self.w_gu, self.w_down = rt.row_major(self.w_gu, self.p_gu), rt.row_major(self.w_down, self.p_down)
 
     takes_normed_input = True     # the gate/up product applies the norm in front of it when the rows are few
     adds_residual = True          # the down product adds to the residual stream when the rows are few
@@ -61,7 +62,7 @@ class GatedMLP(Part):
         normed = isinstance(x, NormedInput)
         if normed and not (can_fuse(rt, n) and self.width % 8 == 0):
             x, normed = x.materialize(), False
-        if rt.dtype == torch.bfloat16 and n <= SKINNY_MAX_ROWS:
+        if rt.dtype == torch.bfloat16 and (n <= SKINNY_MAX_ROWS or self.w_gu is None):
             w = self.p_gu if self.p_gu is not None else self.w_gu
             if normed:
                 ops.gated_linear_bf16(x.h, w, act, norm_gain=x.gain, norm_eps=x.eps)

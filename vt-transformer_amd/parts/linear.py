@@ -40,21 +40,21 @@ def linear(rt: Runtime, x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.T
     its own where that is not possible).  residual (float32 [N, M]): the product is added to it in place and
     `residual` is returned; only callers that checked `can_fuse(rt, n)` may pass it."""
     n, k = x.shape
+    m = w.shape[0] if w is not None else packed.rows      # (no row-major copy: the runtime keeps the packed one only)
     if residual is not None or isinstance(x, NormedInput):
         if can_fuse(rt, n) and k % 8 == 0:
             norm = x if isinstance(x, NormedInput) else None
-            out = residual if residual is not None else rt.buffer(name, (n, w.shape[0]), torch.float32)
+            out = residual if residual is not None else rt.buffer(name, (n, m), torch.float32)
             return ops.linear_bf16(norm.h if norm else x, packed if packed is not None else w, bias, out,
                                    norm_gain=norm.gain if norm else None, norm_eps=norm.eps if norm else 0.0,
                                    residual=residual)
         if residual is not None:
             raise ValueError("linear: a residual to add to needs the few-row kernel (see can_fuse)")
         x = x.materialize()
-    m = w.shape[0]
     if rt.dtype == torch.float32:
         out = rt.buffer(name, (n, m), torch.float32)
         return ops.linear_f32(x, w, bias, out)
-    if n <= SKINNY_MAX_ROWS:
+    if n <= SKINNY_MAX_ROWS or w is None:
         out = rt.buffer(name, (n, m), out_dtype or torch.float32)
         need = ops.linear_bf16_workspace(n, m, k) if n > 16 else 0
         work = rt.buffer("linear.partials", (need,), torch.float32) if need else None
