@@ -22,7 +22,10 @@ QWEN2_7B = dict(architectures=["Qwen2ForCausalLM"], vocab_size=152064, hidden_si
                 num_hidden_layers=28, num_attention_heads=28, num_key_value_heads=4, head_dim=128,
                 rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=8192,
                 hidden_act="silu", use_sliding_window=False)
-FULL_LAYERS = 28
+# Qwen2-72B layer sizes: about 145 GB of bfloat16 weights, which fit one MI355X once (--sizes 72b keeps one copy)
+QWEN2_72B = dict(QWEN2_7B, hidden_size=8192, intermediate_size=29568, num_hidden_layers=80, num_attention_heads=64,
+                 num_key_value_heads=8)
+SIZES = {"7b": ("Qwen2-7B", QWEN2_7B, (1, 64)), "72b": ("Qwen2-72B", QWEN2_72B, (1, 16))}
 HBM_GBPS = 8000.0          # MI355X HBM3E, published
 PEAK_FLOPS = {"bf16": 2.5e15, "fp16": 2.5e15, "fp8": 5.0e15, "fp32": 157.3e12}   # dense MFMA, published
 
@@ -34,7 +37,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--prompt-len", type=int, default=1024)
-    ap.add_argument("--layers", type=int, default=FULL_LAYERS, help="fewer layers than the model has (named in config)")
+    ap.add_argument("--sizes", choices=sorted(SIZES), default="7b",
+                    help="layer sizes; 72b keeps one copy of the weights (prompts then go through the few-row kernels)")
+    ap.add_argument("--layers", type=int, default=0, help="fewer layers than the model has (named in config)")
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--no-graphs", action="store_true")
@@ -51,20 +56,24 @@ def main() -> int:
     from vt_transformer_amd.engine import Engine, StepEntry
     from vt_transformer_amd.sampling import SamplingParams
 
-    cfg_d = dict(QWEN2_7B)
-    cfg_d["num_hidden_layers"] = args.layers
+    model_name, sizes, point_batches = SIZES[args.sizes]
+    FULL_LAYERS = sizes["num_hidden_layers"]
+    single_copy = args.sizes == "72b"
+    cfg_d = dict(sizes)
+    cfg_d["num_hidden_layers"] = args.layers or FULL_LAYERS
     cfg = config_from_dict(cfg_d)
     ctx_len = cfg.max_position_embeddings
-    max_batch = 64 if not args.no_points else max(args.batch, 1)
+    max_batch = max(point_batches) if not args.no_points else max(args.batch, 1)
+    max_batch = max(max_batch, args.batch)
     per_req = -(-(args.prompt_len + args.steps + args.warmup + 32) // 16) * 16
     pool_tokens = max(max_batch * per_req, args.prefill_tokens + 64)
     t0 = time.time()
     eng = Engine(config=cfg, random_weights_seed=0, dtype="bfloat16", page_size=16, num_pages=pool_tokens // 16,
                  max_running_reqs=max(max_batch, 1), max_seq_len=ctx_len, max_extend_tokens=8192, chunk_size=2048,
-                 decode_graphs=not args.no_graphs)
+                 decode_graphs=not args.no_graphs, single_weight_copy=single_copy)
     torch.cuda.synchronize()
     print(f"[bench] model ready in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
-    if not args.no_tune and not args.no_prefill:
+    if not args.no_tune and not args.no_prefill and not single_copy:
         print(f"[bench] GEMM library algorithm search at {args.prefill_tokens} rows: "
               f"{eng.tune_library_products(args.prefill_tokens):.1f} s", file=sys.stderr, flush=True)
     rs = np.random.RandomState(0)
@@ -129,20 +138,21 @@ def main() -> int:
 
     points = {}
     if not args.no_points:
-        for b in (1, 64):
+        for b in point_batches:
             k = max(16, args.steps // 2)
             points[f"decode_b{b}"] = round(decode_run(b, k, 8)[0], 1)
 
     line = {
-        "metric": "decode tok/s at batch 8, Qwen2-7B layer sizes, 1,024-token prompts",
+        "metric": f"decode tok/s at batch {args.batch}, {model_name} layer sizes, {args.prompt_len:,}-token prompts",
         "value": round(tps, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic (random weights N(0,0.02), uniform random token ids)",
-        "config": {"model": "Qwen2-7B sizes", "layers": L, "layers_full": FULL_LAYERS, "hidden": H,
+        "config": {"model": f"{model_name} sizes", "layers": L, "layers_full": FULL_LAYERS, "hidden": H,
                    "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
                    "intermediate": I, "vocab": V, "global_batch": args.batch, "seq_len": args.prompt_len,
                    "prompt_len": args.prompt_len, "context_len": ctx_len, "kv_block": 16, "rope_theta": cfg.rope_theta,
-                   "parallelism": "1 GPU", "decode_graphs": not args.no_graphs, "gemm_tuning": not args.no_tune},
+                   "parallelism": "1 GPU", "decode_graphs": not args.no_graphs, "gemm_tuning": not (args.no_tune or single_copy),
+                   "weight_copies": 1 if single_copy else 2},
         "prefill": {"value": round(T / p_dt, 1), "tokens": T, "ms": round(p_dt * 1e3, 3),
                     "frac": round(p_flops / p_dt / PEAK_FLOPS["bf16"], 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBPS, "unit": "GB/s",
