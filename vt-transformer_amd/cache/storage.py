@@ -93,10 +93,6 @@ class CacheStorage:
         """The window of group g's layers (0: they keep every key)."""
         return int(self.group_needs[g].window)
 
-    def bytes_per_token(self) -> int:
-        item = torch.empty((), dtype=self.rt.dtype).element_size()
-        return sum(2 * k.shape[0] * k.shape[2] * k.shape[4] * item for k in self.k)
-
     def layer_caches(self, block_tables: List[torch.Tensor]) -> List[Optional[LayerCache]]:
         out: List[Optional[LayerCache]] = []
         for i, g in enumerate(self.entry_group):

@@ -196,41 +196,9 @@ __device__ __forceinline__ void park_block(const KVBlock& b, bf16_t* kl, int lan
 
 // CH consecutive elements (from c, a multiple of CH) of a head as the projection left them in fp32, rotated: the
 // pairs are (i, i + rot/2) for i < rot/2, elements from rot on pass through; rot is a multiple of 2 CH.  The same
-// arithmetic as the separate rotation kernel (vt_rope_store).
-template <int CH>
-__device__ __forceinline__ void rotated_chunk(float (&x)[CH], const float* row, int c, int rot, const float* cos_t,
-                                              const float* sin_t, int pos, int max_pos) {
-    if (rot == 0) {     // (the same for every lane and every call of a launch: no tables to read from)
-#pragma unroll
-        for (int i = 0; i < CH; i += 4) {
-            const float4 v = *(const float4*)(row + c + i);
-            x[i] = v.x; x[i + 1] = v.y; x[i + 2] = v.z; x[i + 3] = v.w;
-        }
-        return;
-    }
-    // No load below sits under a test of c: a chunk outside the rotary dims reads its own elements and the tables'
-    // first entries and drops them.  So the loads of all the chunks of a row are in flight together; under
-    // branches every chunk would wait for its own before the next one's could start.
-    const int half = rot >> 1;
-    const bool in = c < rot, low = c < half;
-    const int tp = pos < max_pos ? (pos < 0 ? 0 : pos) : max_pos - 1;
-    const int ti = in ? (low ? c : c - half) : 0;
-    const float* ct = cos_t + (size_t)tp * half + ti;
-    const float* st = sin_t + (size_t)tp * half + ti;
-    const float* other = row + (in ? (low ? c + half : c - half) : c);
-#pragma unroll
-    for (int i = 0; i < CH; i += 4) {
-        const float4 v = *(const float4*)(row + c + i);
-        const float4 y = *(const float4*)(other + i), cc = *(const float4*)(ct + i), sn = *(const float4*)(st + i);
-        x[i] = in ? rotate_pair(cc.x, sn.x, v.x, y.x, low) : v.x;
-        x[i + 1] = in ? rotate_pair(cc.y, sn.y, v.y, y.y, low) : v.y;
-        x[i + 2] = in ? rotate_pair(cc.z, sn.z, v.z, y.z, low) : v.z;
-        x[i + 3] = in ? rotate_pair(cc.w, sn.w, v.w, y.w, low) : v.w;
-    }
-}
-
-// The same in two steps, so that the loads of several chunks are in flight together: the compiler keeps a chunk's
-// loads next to its arithmetic, and a row's chunks then wait for memory one after the other.
+// arithmetic as the separate rotation kernel (vt_rope_store).  In two steps (loads, then arithmetic), so that the
+// loads of several chunks are in flight together: the compiler keeps a chunk's loads next to its arithmetic, and a
+// row's chunks then wait for memory one after the other.
 template <int CH>
 struct RotIn {
     float4 x[CH / 4], y[CH / 4], c[CH / 4], s[CH / 4];
@@ -450,8 +418,10 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_kernel(AttnArg
             const int tid = threadIdx.x;
             if (tid < D / 4) {
                 float x[4];
-                rotated_chunk<4>(x, a.qkv + (size_t)q_tok0 * a.qkv_stride + (size_t)(a.n_heads + kvh) * D, tid * 4, a.rot,
-                                 a.cos_t, a.sin_t, pos0, a.max_pos);
+                RotIn<4> rk;
+                rot_load<4>(rk, a.qkv + (size_t)q_tok0 * a.qkv_stride + (size_t)(a.n_heads + kvh) * D, tid * 4, a.rot,
+                            a.cos_t, a.sin_t, pos0, a.max_pos);
+                rot_apply<4>(x, rk);
                 bf16_t* kp = (bf16_t*)a.k_pages + (((size_t)pg * a.n_kv + kvh) * ps_ + slot) * D + tid * 4;
                 *(uint2*)kp = make_uint2(pack2(x[0], x[1]), pack2(x[2], x[3]));
             } else if (tid >= 64 && tid < 64 + D / 4) {
@@ -963,8 +933,6 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const int* __restrict
     const size_t slot_step = (size_t)rt_per_item * n_kv * 16;
     merge_parts(sm, sl, part_o, part_ml, out, slot0, slot_step, n_parts, n_valid, q_tok0, q_row0, G, kvh, n_heads);
 }
-
-extern "C" int vt_attn_bf16_head_dim() { return D; }
 
 static int shift_of(int v) {
     for (int sft = 0; sft < 31; ++sft)
