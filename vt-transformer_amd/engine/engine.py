@@ -30,8 +30,8 @@ class Engine:
         """model: a folder with config.json and model.safetensors.  Or `config` with `random_weights_seed`
         for random weights drawn on the device.  `options` override fields of SchedulerConfig
         (max_running_reqs, num_pages, max_seq_len, page_size, max_extend_tokens, default_max_output, chunk_size).
-        tune_gemm: let the GEMM library try its algorithms on this model's products at chunk_size rows once, at
-        start-up (some seconds), and use the fastest from then on.
+        tune_gemm: let the GEMM library try its algorithms on this model's products at chunk_size rows (and at 128
+        and 256 rows, if so many requests may run) once, at start-up (some seconds), and use the fastest from then on.
         single_weight_copy: keep the bfloat16 matrices once (in the few-row kernels' order) instead of twice; long
         prompt portions are then several times slower.  For models that fit the GPU's memory once but not twice."""
         sc = scheduler_config or SchedulerConfig()
@@ -59,6 +59,9 @@ class Engine:
         self.requests: Dict[Hashable, Request] = {}
         if tune_gemm:
             self.tune_library_products()
+            for rows in (128, 256):     # decoding batches beyond the few-row kernels' 64 rows take the library too
+                if rows <= sc.max_running_reqs:
+                    self.tune_library_products(rows)
 
     def tune_library_products(self, rows: Optional[int] = None) -> float:
         """Long portions multiply through the GEMM library (parts/linear.py).  This runs one portion of `rows`
