@@ -176,6 +176,15 @@ def test_trace_run_program(model_folders, dtype, tmp_path):
                         TINY[cfg]["vocab_size"])
     worst = check_against_plain(model_folders[cfg], reqs, steps, got, dtype, _plain_cache)
     report(f"trace_run {cfg} {dtype}", worst)
+    # most of each request in one step, its last tokens one by one beside the others' (decoding steps, which the
+    # program runs through captured graphs as the engine does), with so few pages that they are used again
+    reqs = random_requests(TINY[cfg]["vocab_size"], [40, 33, 52, 45, 38, 47], seed=13)
+    portions = {r: [(0, len(t) - 14)] + [(j, j + 1) for j in range(len(t) - 14, len(t))] for r, t in reqs.items()}
+    steps = trace_mixed(reqs, portions, max_live=3, seed=14)
+    got = run_trace_run(model_folders[cfg], dtype, steps, str(tmp_path / "out2"), max_live_tokens(steps),
+                        TINY[cfg]["vocab_size"])
+    worst = check_against_plain(model_folders[cfg], reqs, steps, got, dtype, _plain_cache)
+    report(f"trace_run decode {cfg} {dtype}", worst)
 
 
 def test_random_weights_on_device_match_written_folder(model_folders):
