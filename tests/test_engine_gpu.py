@@ -290,6 +290,96 @@ def test_tight_engine_with_arrivals_gives_each_request_what_it_gets_alone(model_
     assert eng.scheduler.counters["preemptions"] > 0      # the draws below leave too few pages for the live requests
 
 
+@pytest.mark.parametrize("cfg", ["A", "W"])
+def test_decoding_ahead_of_the_host_gives_the_same_tokens(cfg, tmp_path):
+    """The engine starts the next decoding step before this one's tokens have reached the host.  With requests
+    that end at different times (end-of-sequence tokens, output limits of their own), with temperature and without,
+    it produces exactly the tokens and finish reasons of the engine that waits for every step."""
+    from vt_transformer_amd.config import config_from_dict
+    from vt_transformer_amd.engine import Engine
+    from vt_transformer_amd.sampling import SamplingParams
+    from vt_transformer_amd.weights import write_random_model
+    vocab = TINY[cfg]["vocab_size"]
+    d = dict(TINY[cfg], eos_token_id=list(range(3, vocab, 9)))          # one token in nine ends a request
+    folder = str(tmp_path / "m")
+    write_random_model(config_from_dict(d), folder, seed=17)
+    rs = np.random.RandomState(5)
+    prompts = [rs.randint(0, vocab, size=int(rs.randint(3, 40))).tolist() for _ in range(12)]
+    sps = [SamplingParams(temperature=float(rs.choice([0.0, 0.9])), top_k=int(rs.choice([-1, 8])),
+                          max_tokens=int(rs.randint(2, 40)), ignore_eos=bool(i % 4 == 0), seed=300 + i) for i in range(12)]
+    outs = []
+    for ahead in (False, True):
+        eng = Engine(folder, dtype="bfloat16", num_pages=64, max_running_reqs=12, max_seq_len=128)
+        eng.pipeline_decode = ahead
+        launched = []
+        orig = eng._launch
+        eng._launch = lambda plan, ids, orig=orig: (launched.append(ids is not None), orig(plan, ids))[1]
+        toks = eng.generate(prompts, sps)
+        outs.append((toks, [eng.finish_reason(i) for i in range(12)]))
+        assert any(launched) == ahead                                   # steps were started ahead, or none was
+        assert sum(eng.runner.cache.held_pages()) == 0 and not eng.has_work()
+    assert outs[0] == outs[1]
+    reasons = set(outs[0][1])
+    assert "eos" in reasons and "max_tokens" in reasons                 # both ways of ending happened
+
+
+def test_decoding_ahead_with_arrivals_aborts_and_few_pages(model_folders):
+    """Steps started ahead while requests arrive, are aborted and are preempted for want of pages: every request
+    ends with a reason, within its limit, no page or slot stays held, and requests that were never disturbed
+    (no preemption) have the tokens they get alone."""
+    from vt_transformer_amd.engine import Engine
+    from vt_transformer_amd.sampling import SamplingParams
+    cfg = "B"
+    rs = np.random.RandomState(9)
+    n = 24
+    prompts = [rs.randint(0, TINY[cfg]["vocab_size"], size=int(rs.randint(1, 60))).tolist() for _ in range(n)]
+    sps = [SamplingParams(temperature=0.0, max_tokens=int(rs.randint(1, 50)), ignore_eos=True, seed=i) for i in range(n)]
+    eng = Engine(model_folders[cfg], dtype="bfloat16", num_pages=9, max_running_reqs=6, max_seq_len=128, chunk_size=32,
+                 max_extend_tokens=64)
+    ahead = []
+    orig = eng._launch
+    eng._launch = lambda plan, ids: (ahead.append(ids is not None), orig(plan, ids))[1]
+    pending, aborted, steps = list(range(n)), set(), 0
+    while pending or eng.has_work():
+        for _ in range(int(rs.randint(0, 3))):
+            if pending:
+                i = pending.pop(0)
+                eng.add_request(prompts[i], sps[i], uid=i)
+        if steps % 7 == 3:
+            live = [u for u, r in eng.requests.items() if r.state == "running" and u not in aborted]
+            if live:
+                u = live[int(rs.randint(0, len(live)))]
+                assert eng.abort_request(u)
+                aborted.add(u)
+        eng.step()
+        steps += 1
+        assert steps < 5000, "the engine does not finish"
+    assert any(ahead) and sum(eng.runner.cache.held_pages()) == 0
+    assert eng.runner.cache.slots.available == 6
+    one = Engine(model_folders[cfg], dtype="bfloat16", num_pages=16, max_running_reqs=1, max_seq_len=128, chunk_size=32,
+                 max_extend_tokens=64)
+    one.pipeline_decode = False
+    pcfg, pw = plain_model.read_folder(model_folders[cfg])
+    checked = 0
+    for i in range(n):
+        r = eng.requests[i]
+        assert r.state == "finished" and r.finish_reason in ("max_tokens", "abort", "max_seq_len")
+        assert len(r.output) <= sps[i].max_tokens
+        if r.finish_reason == "max_tokens":
+            assert len(r.output) == sps[i].max_tokens
+            if r.preemptions == 0:
+                # alone it goes through other kernels where it shared steps with others (rows per product), so a
+                # near tie may fall the other way: where the tokens part, the two candidates' logits are close
+                alone = one.generate([prompts[i]], [sps[i]])[0]
+                if alone != r.output:
+                    j = next(k for k in range(len(alone)) if alone[k] != r.output[k])
+                    lg = plain_model.forward(pcfg, pw, prompts[i] + alone[:j])[-1]
+                    assert float(abs(lg[alone[j]] - lg[r.output[j]]) / lg.abs().max()) < 2e-2, (i, j)
+                    assert float((lg.max() - max(lg[alone[j]], lg[r.output[j]])) / lg.abs().max()) < 2e-2, (i, j)
+                checked += 1
+    assert checked >= 3 and eng.scheduler.counters["preemptions"] > 0 and aborted
+
+
 def test_decode_graph_replays_match_eager(model_folders):
     """Captured decoding steps against the same steps launched one by one: several replays, with eager work
     (prompt portions of other requests, synchronisations) between them, all equal."""

@@ -57,6 +57,8 @@ class Engine:
         self.seed = int(seed)
         self._next_uid = 0
         self.requests: Dict[Hashable, Request] = {}
+        self.pipeline_decode = True     # start the next decoding step before this one's tokens are on the host
+        self._ahead = None              # (plan, pending tokens) of a step that is already queued on the GPU
         if tune_gemm:
             self.tune_library_products()
             for rows in (128, 256):     # decoding batches beyond the few-row kernels' 64 rows take the library too
@@ -114,24 +116,67 @@ class Engine:
         return self.scheduler.abort_request(uid)
 
     def has_work(self) -> bool:
-        return self.scheduler.has_work()
+        return self.scheduler.has_work() or self._ahead is not None
 
     # -- one step ------------------------------------------------------------
     def step(self) -> List[ReqResult]:
-        plan = self.scheduler.schedule()
+        """One step of the scheduler's loop: choose a batch, run it, take the sampled tokens, finish and free.
+
+        While every running request is decoding and nobody waits, the step after this one is started before this
+        one's tokens have reached the host (its input is what the sampler left on the device), so the GPU does not
+        wait while the host does its bookkeeping.  What that step computes for a request that turns out to have
+        finished in this one is dropped; its pages are only reused by work that is queued behind it."""
+        cur, self._ahead = self._ahead, None
+        if cur is None:
+            plan = self.scheduler.schedule()
+            if not plan:
+                return self.scheduler.update(plan, {})
+            cur = self._launch(plan, None)
+        if self.pipeline_decode:
+            nxt = self._plan_ahead(cur[0])
+            if nxt is not None:
+                self._ahead = self._launch(nxt, cur[1].tokens_dev)
+        plan, pending = cur
         sampled: Dict[Hashable, int] = {}
-        if plan:
-            entries = []
-            for s in plan:
-                toks = s.request.token_slice(s.start, s.n_tokens)
-                entries.append(StepEntry(s.request.uid, toks, [s.n_tokens - 1] if s.sample else []))
-            logits = self.runner.step(entries)
-            rows = [(s.request.params, s.request.seed, len(s.request.output)) for s in plan if s.sample]
-            if rows:
-                toks = self.sampler.sample(logits, rows)
-                for s, t in zip((s for s in plan if s.sample), toks):
-                    sampled[s.request.uid] = t
-        return self.scheduler.update(plan, sampled)
+        if pending is not None:
+            toks = self.sampler.collect(pending)
+            for s, t in zip((s for s in plan if s.sample), toks):
+                sampled[s.request.uid] = t
+        results = self.scheduler.update(plan, sampled)
+        if self._ahead is not None and not any(s.request.state == "running" for s in self._ahead[0]):
+            self._ahead = None      # everybody in it has finished meanwhile: nothing of it is wanted
+        return results
+
+    def _launch(self, plan: List[Scheduled], ids_dev):
+        """Queue the plan's step and its sampling on the GPU; returns (plan, pending tokens or None)."""
+        ahead = ids_dev is not None         # the requests' newest tokens are not on the host yet
+        entries = []
+        for s in plan:
+            toks = [0] if ahead else s.request.token_slice(s.start, s.n_tokens)
+            entries.append(StepEntry(s.request.uid, toks, [s.n_tokens - 1] if s.sample else []))
+        logits = self.runner.step(entries, ids_dev)
+        rows = [(s.request.params, s.request.seed, len(s.request.output) + (1 if ahead else 0)) for s in plan if s.sample]
+        return plan, (self.sampler.launch(logits, rows) if rows else None)
+
+    def _plan_ahead(self, plan: List[Scheduled]) -> Optional[List[Scheduled]]:
+        """The step after `plan`, if it can be told without `plan`'s tokens: `plan` is every running request's one
+        decoding token, nobody waits, nobody reaches a limit with the token it is about to get (an end-of-sequence
+        token may still finish a request: its part of the step ahead is then dropped), the pages are there, and
+        the step goes through a captured graph."""
+        sch = self.scheduler
+        if sch.waiting or sch.finished_early or len(plan) != len(sch.running) or not self.runner.replays(len(plan)):
+            return None
+        nxt = []
+        for s in plan:
+            r = s.request
+            if s.n_tokens != 1 or not s.sample or r.state != "running":
+                return None
+            if len(r.output) + 2 > r.params.max_tokens or r.total_len + 2 > sch.config.max_seq_len:
+                return None     # its last or last but one token: the plain way finishes it
+            nxt.append(Scheduled(r, s.start + 1, 1, True))
+        if not sch._fits([(s.request, s.start + 1) for s in nxt]):
+            return None
+        return nxt
 
     # -- the whole loop --------------------------------------------------------
     def generate(self, prompts: Union[Sequence[int], Sequence[Sequence[int]]],

@@ -417,11 +417,21 @@ class ModelRunner:
         self._fill_context(ctx, h, h["rows"], dev, decode)
         return ctx
 
-    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+    def replays(self, n_entries: int) -> bool:
+        """Whether a decoding step of this many entries goes through a captured graph."""
+        return (self.decode_graphs and self._replayable and self.rt.dtype == torch.bfloat16
+                and 0 < n_entries <= GRAPH_BATCHES[-1])
+
+    def step(self, entries: Sequence[StepEntry], ids_dev: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         """Run the entries' tokens as one batch.  Returns fp32 logits [wanted places, vocab] on the device in the
         order of the entries and of their `want`, or None if nothing is wanted.  Raises OutOfPages (with nothing
-        changed) if the cache cannot hold the new tokens."""
+        changed) if the cache cannot hold the new tokens.
+        ids_dev (int32 on the device, one per entry): the entries' one token each, where the host does not know
+        them yet (the entries then carry placeholders); only for decoding steps that `replays()` says are captured."""
         cache = self.cache
+        use_graph = self.replays(len(entries)) and all(len(e.tokens) == 1 for e in entries)
+        if ids_dev is not None and not use_graph:
+            raise RuntimeError("token ids that are still on the device can only be fed to a captured decoding step")
         targets = [(e.rid, cache.get(e.rid).length + len(e.tokens)) for e in entries]
         for rid, new_len in targets:
             if new_len > self.max_seq_len:
@@ -430,10 +440,8 @@ class ModelRunner:
             raise OutOfPages(f"the step needs more pages than are free ({cache.available_pages()} free per group)")
         fresh_slots = [cache.get(e.rid).slot for e in entries if cache.get(e.rid).fresh]
         self.storage.clear_state(fresh_slots)
-        use_graph = (self.decode_graphs and self._replayable and self.rt.dtype == torch.bfloat16
-                     and len(entries) <= GRAPH_BATCHES[-1] and all(len(e.tokens) == 1 for e in entries))
         if use_graph:
-            logits = self._step_decode_graph(entries)
+            logits = self._step_decode_graph(entries, ids_dev)
         else:
             ctx = self.build_context(entries)
             caches = self.storage.layer_caches(ctx.block_tables)
@@ -445,12 +453,20 @@ class ModelRunner:
         return logits
 
     # -- decoding through a captured graph ---------------------------------------
-    def _step_decode_graph(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+    def _feed_ids(self, g: "_DecodeGraph", ids_dev: Optional[torch.Tensor], n: int) -> None:
+        """Token ids that the sampler left on the device go into the step's metadata there, after the host's copy
+        of it (which holds placeholders for them) has been sent and before the step runs."""
+        if ids_dev is not None:
+            o = g.ctx.part_offsets["ids"]
+            g.meta[o:o + n].copy_(ids_dev[:n])
+
+    def _step_decode_graph(self, entries: Sequence[StepEntry], ids_dev: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         n = len(entries)
         b = next(x for x in GRAPH_BATCHES if x >= n)
         g = self._graphs.get(b)
         rids = tuple(e.rid for e in entries)
         if g is not None and g.rids == rids and self._advance_decode_meta(g, entries):
+            self._feed_ids(g, ids_dev, n)
             g.graph.replay()        # the same requests as in the last step, one token further: the metadata was patched
             return g.wanted
         fixed_blocks = -(-self.max_seq_len // self.cache.page_size)
@@ -472,6 +488,7 @@ class ModelRunner:
                 self._graphs[b] = g
             else:
                 self._fill_context(g.ctx, h, all_rows, g.meta, decode=True)
+            self._feed_ids(g, ids_dev, n)
             g.graph.replay()
         # what the next step can patch instead of building anew: the host copy of the metadata and where its parts lie
         g.rids, g.h, g.flat = rids, h, self._last_flat

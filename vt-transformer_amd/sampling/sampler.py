@@ -42,13 +42,32 @@ def request_seed(engine_seed: int, request_key) -> int:
     return _splitmix64((engine_seed & _M64) ^ _splitmix64(key))
 
 
+class Pending:
+    """Tokens that have been chosen on the device and are on their way to the host."""
+
+    def __init__(self, tokens_dev: torch.Tensor, host: torch.Tensor, event, rows: int):
+        self.tokens_dev, self.host, self.event, self.rows = tokens_dev, host, event, rows
+
+
 class Sampler:
     def __init__(self, rt: Runtime):
         self.rt = rt
         self._staging = HostStaging(torch.float32)
+        self._turn = 0
+        self._host: dict = {}
 
     def sample(self, logits: torch.Tensor, rows: Sequence[Tuple[SamplingParams, int, int]]) -> List[int]:
         """logits [R, V] fp32 on the device; rows[i] = (params, seed, counter) of row i."""
+        return self.collect(self.launch(logits, rows))
+
+    def collect(self, pending: Pending) -> List[int]:
+        pending.event.synchronize()
+        return pending.host[:pending.rows].tolist()
+
+    def launch(self, logits: torch.Tensor, rows: Sequence[Tuple[SamplingParams, int, int]]) -> Pending:
+        """Choose the tokens and start their copy to the host without waiting for either: `collect` waits.  The
+        tokens also stay on the device (`tokens_dev`) for a next step that starts before the host has read them.
+        Two sets of buffers take turns, so one launch may be outstanding while the next is made."""
         r, v = logits.shape
         if r != len(rows):
             raise ValueError(f"{r} rows of logits for {len(rows)} requests")
@@ -61,11 +80,19 @@ class Sampler:
             host[3, i] = np.int32(p.top_k).view(np.float32)
         dev = self.rt.buffer("sample.params", (4, r), torch.float32)
         self._staging.upload(host, dev)
-        out = self.rt.buffer("sample.out", (r,), torch.int32)
+        self._turn ^= 1
+        out = self.rt.buffer(f"sample.out{self._turn}", (r,), torch.int32)
         if any(host[0, i] > 0 for i in range(r)):
             work = self.rt.buffer("sample.work", (r * v,), torch.float32)   # probabilities of the stochastic rows
         else:
             work = logits.view(-1)   # greedy rows never touch the workspace
         partials = self.rt.buffer("sample.partials", (ops.sample_partials_size(r),), torch.float32)
         ops.sample(logits, dev[0], dev[3].view(torch.int32), dev[1], dev[2], work, out, partials)
-        return out.cpu().tolist()
+        host = self._host.get(self._turn)
+        if host is None or host.numel() < r:
+            host = torch.empty(max(r, 64), dtype=torch.int32, pin_memory=True)
+            self._host[self._turn] = host
+        host[:r].copy_(out, non_blocking=True)
+        event = torch.cuda.Event()
+        event.record()
+        return Pending(out, host, event, r)
