@@ -131,7 +131,7 @@ def main() -> int:
     achieved = step_bytes / (ms * 1e-3) / 1e9
 
     T = args.prefill_tokens
-    p_dt = prefill_run(T) if not args.no_prefill else float("nan")
+    p_dt = prefill_run(T) if not args.no_prefill else None
     mm_flops = 2.0 * T * L * (qkv * H + cfg.num_attention_heads * cfg.head_dim * H + 3 * I * H) + 2.0 * V * H
     attn_flops = L * 4.0 * cfg.num_attention_heads * cfg.head_dim * (T * (T + 1) / 2)   # causal: QK^T and PV
     p_flops = mm_flops + attn_flops
@@ -153,8 +153,8 @@ def main() -> int:
                    "prompt_len": args.prompt_len, "context_len": ctx_len, "kv_block": 16, "rope_theta": cfg.rope_theta,
                    "parallelism": "1 GPU", "decode_graphs": not args.no_graphs, "gemm_tuning": not (args.no_tune or single_copy),
                    "weight_copies": 1 if single_copy else 2},
-        "prefill": {"value": round(T / p_dt, 1), "tokens": T, "ms": round(p_dt * 1e3, 3),
-                    "frac": round(p_flops / p_dt / PEAK_FLOPS["bf16"], 4)},
+        "prefill": None if p_dt is None else {"value": round(T / p_dt, 1), "tokens": T, "ms": round(p_dt * 1e3, 3),
+                                              "frac": round(p_flops / p_dt / PEAK_FLOPS["bf16"], 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_GBPS, 4)},
         "points": points,
