@@ -6,7 +6,8 @@
 Prints one JSON line.  `value` is decoded tokens per second at batch 8 after 1,024-token prompts (a step is one
 decode step of the whole batch through scheduler, step function and sampler).  The line also carries the
 prefill of one 2,048-token prompt, the decode step's achieved HBM bandwidth against the bytes it has to read,
-and decode at batch 1 and 64.  The reference publishes no number to compare with (vs_baseline is null).
+decode at batch 1 and 64, and what this GPU's memory and matrix cores were measured to deliver (a kernel that only
+reads; the library's square product), beside the published peaks that the fractions are taken against.  The reference publishes no number to compare with (vs_baseline is null).
 """
 import argparse
 import json
@@ -44,6 +45,8 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--no-graphs", action="store_true")
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill measurement (profiling runs)")
+    ap.add_argument("--no-peaks", action="store_true", help="skip the measurement of what this GPU's memory and matrix "
+                    "cores deliver to a kernel that only reads and to the library's square product")
     ap.add_argument("--no-tune", action="store_true", help="do not let the GEMM library search its algorithms at start-up")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -119,6 +122,34 @@ def main() -> int:
         print(f"[bench] prefill {tokens} tokens: {best * 1e3:.2f} ms", file=sys.stderr, flush=True)
         return best
 
+    def measured_peaks():
+        """What this machine delivers: GB/s of a kernel that only reads 2 GB (beyond the last-level cache), and
+        TFLOP/s of the GEMM library on an 8,192-cube in bfloat16."""
+        from vt_transformer_amd.kernels import ops
+        buf = torch.randint(0, 1 << 30, (1 << 29,), dtype=torch.int32, device="cuda")
+        sums = torch.empty(256 * 16, dtype=torch.int32, device="cuda")
+        a = torch.randn(8192, 8192, device="cuda").to(torch.bfloat16)
+        b = torch.randn(8192, 8192, device="cuda").to(torch.bfloat16)
+        c = torch.empty(8192, 8192, dtype=torch.bfloat16, device="cuda")
+
+        def best_ms(fn, reps=6):
+            best = None
+            for i in range(reps):
+                st, en = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                st.record()
+                fn()
+                en.record()
+                torch.cuda.synchronize()
+                if i:
+                    best = st.elapsed_time(en) if best is None else min(best, st.elapsed_time(en))
+            return best
+        read_ms = best_ms(lambda: ops.stream_read(buf, sums))
+        mm_ms = best_ms(lambda: torch.mm(a, b.t(), out=c))
+        out = {"hbm_read_GBps": round(buf.numel() * 4 / read_ms / 1e6, 1),
+               "gemm_bf16_TFLOPs": round(2 * 8192 ** 3 / mm_ms / 1e9, 1)}
+        print(f"[bench] measured peaks: {out}", file=sys.stderr, flush=True)
+        return out
+
     # ---- sizes for the roofline -------------------------------------------------
     H, I, V, L = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size, cfg.num_hidden_layers
     qkv = (cfg.num_attention_heads + 2 * cfg.num_key_value_heads) * cfg.head_dim
@@ -159,6 +190,8 @@ def main() -> int:
                      "frac": round(achieved / HBM_GBPS, 4)},
         "points": points,
     }
+    if not args.no_peaks:
+        line["measured_peaks"] = measured_peaks()
     print(json.dumps(line), flush=True)
     return 0
 

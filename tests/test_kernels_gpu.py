@@ -607,3 +607,19 @@ def test_linear_bf16_with_norm_in_front_and_residual_behind(n, m, k):
     # more than 16 rows are refused
     with pytest.raises(Exception):
         o.linear_bf16(torch.zeros(17, k, device=DEV), w, None, torch.empty(17, m, device=DEV), norm_gain=gain, norm_eps=eps)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("nbytes, blocks", [(16, 1), (48 * 1024, 3), (1 << 20, 16), ((1 << 22) + 16 * 77, 256)])
+def test_stream_read_reads_every_word_once(nbytes, blocks):
+    # the kernel that measures the memory's ceiling: its checksum is the XOR of all words, tails included
+    o = ops()
+    rs = np.random.RandomState(nbytes % 1000)
+    host = rs.randint(0, 1 << 31, size=nbytes // 4).astype(np.int32)
+    buf = torch.from_numpy(host).cuda()
+    sums = torch.zeros(blocks * 16, dtype=torch.int32, device="cuda")
+    o.stream_read(buf, sums, blocks)
+    got = np.bitwise_xor.reduce(sums.cpu().numpy().view(np.uint32))
+    assert got == np.bitwise_xor.reduce(host.view(np.uint32))
+    with pytest.raises(o.KernelError):
+        o.stream_read(buf.view(torch.int16)[:4], sums, blocks)

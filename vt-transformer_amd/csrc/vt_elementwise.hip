@@ -513,3 +513,44 @@ extern "C" int vt_gather_rows(const void* in, int in_dtype, const int* rows, voi
     VT_CHECK_LAUNCH("vt_gather_rows");
     return 0;
 }
+
+// ---------------------------------------------------------------------------
+// Streaming read: what the memory delivers to a kernel that only reads (the measured ceiling that the weight
+// streaming kernels are compared with).  Every wave reads a contiguous share, 1 KB per load instruction and
+// eight loads in flight, and leaves the XOR of its 32-bit words in sums[wave]; the words behind the last full
+// share of all waves are read by the last wave one load at a time.
+__global__ __launch_bounds__(1024) void stream_read_kernel(const uint4* __restrict__ p, size_t n16,
+                                                          unsigned* __restrict__ sums) {
+    constexpr int U = 8;
+    const size_t waves = (size_t)gridDim.x * (blockDim.x >> 6);
+    const size_t wave = (size_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    const size_t per = n16 / (waves * 64 * U) * (64 * U);      // 16-byte pieces per wave, whole turns only
+    const uint4* q = p + wave * per + lane;
+    unsigned acc = 0;
+    for (size_t i = 0; i < per; i += 64 * U) {
+        uint4 v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) v[u] = q[i + 64 * u];
+#pragma unroll
+        for (int u = 0; u < U; ++u) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+    }
+    if (wave == waves - 1)
+        for (size_t i = waves * per + lane; i < n16; i += 64) {
+            const uint4 v = p[i];
+            acc ^= v.x ^ v.y ^ v.z ^ v.w;
+        }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) acc ^= __shfl_xor(acc, off);
+    if (lane == 0) sums[wave] = acc;
+}
+
+// sums: blocks * 16 words; the XOR of all of them is the XOR of the buffer's 32-bit words (bytes a multiple of 16)
+extern "C" int vt_stream_read(const void* p, long long bytes, unsigned* sums, int blocks, hipStream_t stream) {
+    VT_REQUIRE(bytes >= 0 && bytes % 16 == 0 && (((uintptr_t)p) & 15) == 0,
+               "vt_stream_read: %lld bytes at %p are not whole 16-byte pieces", bytes, p);
+    VT_REQUIRE(blocks > 0 && blocks <= 65535, "vt_stream_read: %d blocks", blocks);
+    stream_read_kernel<<<blocks, 1024, 0, stream>>>((const uint4*)p, (size_t)bytes / 16, sums);
+    VT_CHECK_LAUNCH("vt_stream_read");
+    return 0;
+}

@@ -126,6 +126,18 @@ def gather_rows(x: torch.Tensor, rows: Optional[torch.Tensor], out: torch.Tensor
     return out
 
 
+def stream_read(buf: torch.Tensor, sums: torch.Tensor, blocks: int = 256) -> torch.Tensor:
+    """Read `buf` once with a kernel that does nothing else (the measured ceiling of weight streaming).
+    sums: int32 [blocks * 16]; the XOR of its words is the XOR of the buffer's 32-bit words."""
+    _chk(buf, "stream_read.buf")
+    _chk(sums, "stream_read.sums", torch.int32, (blocks * 16,))
+    nbytes = buf.numel() * buf.element_size()
+    if nbytes % 16:
+        raise KernelError(f"stream_read: {nbytes} bytes are not whole 16-byte pieces")
+    _run(load_lib("vt_elementwise"), "vt_stream_read", _ptr(buf), ctypes.c_longlong(nbytes), _ptr(sums), _i(blocks), _stream())
+    return sums
+
+
 def rope_store(qkv: torch.Tensor, cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], positions: torch.Tensor,
                tok_entry: torch.Tensor, block_table: Optional[torch.Tensor], q_out: torch.Tensor,
                k_pages: Optional[torch.Tensor], v_pages: Optional[torch.Tensor], n_heads: int, n_kv: int, head_dim: int,
