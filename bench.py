@@ -26,7 +26,11 @@ QWEN2_7B = dict(architectures=["Qwen2ForCausalLM"], vocab_size=152064, hidden_si
 # Qwen2-72B layer sizes: about 145 GB of bfloat16 weights, which fit one MI355X once (--sizes 72b keeps one copy)
 QWEN2_72B = dict(QWEN2_7B, hidden_size=8192, intermediate_size=29568, num_hidden_layers=80, num_attention_heads=64,
                  num_key_value_heads=8)
-SIZES = {"7b": ("Qwen2-7B", QWEN2_7B, (1, 64)), "72b": ("Qwen2-72B", QWEN2_72B, (1, 16))}
+# Qwen2-1.5B layer sizes (tied head)
+QWEN2_15B = dict(QWEN2_7B, vocab_size=151936, hidden_size=1536, intermediate_size=8960, num_attention_heads=12,
+                 num_key_value_heads=2, tie_word_embeddings=True, max_position_embeddings=32768)
+SIZES = {"7b": ("Qwen2-7B", QWEN2_7B, (1, 64)), "72b": ("Qwen2-72B", QWEN2_72B, (1, 16)),
+         "1.5b": ("Qwen2-1.5B", QWEN2_15B, (1, 64))}
 HBM_GBPS = 8000.0          # MI355X HBM3E, published
 PEAK_FLOPS = {"bf16": 2.5e15, "fp16": 2.5e15, "fp8": 5.0e15, "fp32": 157.3e12}   # dense MFMA, published
 
@@ -48,6 +52,11 @@ def main() -> int:
     ap.add_argument("--no-peaks", action="store_true", help="skip the measurement of what this GPU's memory and matrix "
                     "cores deliver to a kernel that only reads and to the library's square product")
     ap.add_argument("--no-tune", action="store_true", help="do not let the GEMM library search its algorithms at start-up")
+    ap.add_argument("--mixed", type=int, default=0, metavar="REQUESTS",
+                    help="another workload instead: this many requests at once with prompt lengths drawn from 16 to "
+                         "4,096 and --mixed-decode tokens each, through the scheduler (portions of prompts beside "
+                         "decoded tokens); value = generated tokens per second from first arrival to last token")
+    ap.add_argument("--mixed-decode", type=int, default=256)
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this engine runs on one GPU; N > 1 is not measured")
@@ -70,6 +79,11 @@ def main() -> int:
     max_batch = max(max_batch, args.batch)
     per_req = -(-(args.prompt_len + args.steps + args.warmup + 32) // 16) * 16
     pool_tokens = max(max_batch * per_req, args.prefill_tokens + 64)
+    rs = np.random.RandomState(0)
+    if args.mixed:
+        mixed_lens = rs.randint(16, 4097, size=args.mixed)
+        pool_tokens = int(sum(-(-(int(n) + args.mixed_decode + 16) // 16) * 16 for n in mixed_lens))
+        max_batch, ctx_len = args.mixed, min(ctx_len, 8192)
     t0 = time.time()
     eng = Engine(config=cfg, random_weights_seed=0, dtype="bfloat16", page_size=16, num_pages=pool_tokens // 16,
                  max_running_reqs=max(max_batch, 1), max_seq_len=ctx_len, max_extend_tokens=8192, chunk_size=2048,
@@ -79,7 +93,26 @@ def main() -> int:
     if not args.no_tune and not args.no_prefill and not single_copy:
         print(f"[bench] GEMM library algorithm search at {args.prefill_tokens} rows: "
               f"{eng.tune_library_products(args.prefill_tokens):.1f} s", file=sys.stderr, flush=True)
-    rs = np.random.RandomState(0)
+
+    def mixed_run(reps: int = 2):
+        """All requests arrive at once; the scheduler cuts their prompts into portions under its token budget and
+        decodes beside them.  Best of `reps` runs: seconds, steps, prompt tokens."""
+        prompts = [rs.randint(0, cfg.vocab_size, size=int(n)).tolist() for n in mixed_lens]
+        sp = SamplingParams(max_tokens=args.mixed_decode, ignore_eos=True)
+        best = None
+        for rep in range(reps):
+            for p in prompts:
+                eng.add_request(p, sp)
+            torch.cuda.synchronize()
+            t, steps = time.perf_counter(), 0
+            while eng.has_work():
+                eng.step()
+                steps += 1
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t
+            print(f"[bench] mixed run {rep}: {dt:.3f} s, {steps} steps", file=sys.stderr, flush=True)
+            best = dt if best is None else min(best, dt)
+        return best, steps, int(mixed_lens.sum())
 
     def decode_run(batch: int, steps: int, warmup: int):
         """tokens/s and ms/step of `steps` decode steps at `batch` after prompts of --prompt-len tokens."""
@@ -156,6 +189,24 @@ def main() -> int:
     layer_params = qkv * H + qkv + cfg.num_attention_heads * cfg.head_dim * H + 3 * I * H + 2 * H
     weight_bytes = 2 * (L * layer_params + V * H + H)                  # every weight the step uses, once (bf16)
     kv_bytes_per_token = 2 * 2 * L * cfg.num_key_value_heads * cfg.head_dim
+
+    if args.mixed:
+        dt, steps, prompt_tokens = mixed_run()
+        gen = args.mixed * args.mixed_decode
+        print(json.dumps({
+            "metric": f"generated tok/s, {args.mixed} requests at once, prompts of 16 to 4,096 tokens, "
+                      f"{args.mixed_decode} decoded tokens each, {model_name} layer sizes",
+            "value": round(gen / dt, 1), "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": 0,
+            "ms_per_step": round(dt / steps * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "bf16", "data": "synthetic (random weights N(0,0.02), uniform random token ids)",
+            "config": {"model": f"{model_name} sizes", "layers": cfg.num_hidden_layers, "layers_full": FULL_LAYERS,
+                       "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
+                       "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
+                       "global_batch": args.mixed, "seq_len": int(mixed_lens.max()), "prompt_tokens": prompt_tokens,
+                       "decode_tokens": args.mixed_decode, "context_len": ctx_len, "kv_block": 16,
+                       "max_extend_tokens": 8192, "chunk_size": 2048, "parallelism": "1 GPU"},
+            "total_tokens_per_s": round((prompt_tokens + gen) / dt, 1), "seconds": round(dt, 3)}), flush=True)
+        return 0
 
     tps, ms, ctx_mid = decode_run(args.batch, args.steps, args.warmup)
     step_bytes = weight_bytes + args.batch * ctx_mid * kv_bytes_per_token
