@@ -145,9 +145,9 @@ def work_for(n, m, k):
 def test_linear_bf16_split_k_needs_and_uses_a_workspace():
     o = ops()
     g = torch.Generator().manual_seed(81)
-    n, m, k = 40, 256, 4096            # few rows of W, long k: the k range is split over blocks
+    n, m, k = 100, 256, 4096           # few rows of W, long k, more than 64 tokens: the k range is split over blocks
     assert o.linear_bf16_workspace(n, m, k) >= 2 * n * m
-    assert o.linear_bf16_workspace(8, m, k) == 0 or True
+    assert o.linear_bf16_workspace(8, m, k) == 0 and o.linear_bf16_workspace(24, m, k) == 0   # whole k in a block
     x = torch.randn(n, k, generator=g).to(torch.bfloat16)
     w = (torch.randn(m, k, generator=g) * 0.05).to(torch.bfloat16)
     b = torch.randn(m, generator=g)
@@ -156,6 +156,42 @@ def test_linear_bf16_split_k_needs_and_uses_a_workspace():
         o.linear_bf16(x.to(DEV), w.to(DEV), b.to(DEV), out)
     o.linear_bf16(x.to(DEV), w.to(DEV), b.to(DEV), out, work_for(n, m, k))
     assert rel_err(out, x.double() @ w.double().t() + b.double()) < 2e-5
+
+
+@pytest.mark.parametrize("n", [17, 31, 32, 33, 50, 64])
+@pytest.mark.parametrize("m,k", [(200, 200), (1030, 3584), (96, 18944 // 4), (3584, 512), (4608, 256), (4100, 128)])
+def test_linear_bf16_adds_to_a_residual_up_to_64_rows(n, m, k):
+    """17 to 64 rows: whole k in a block (two or four token tiles, one or two tile rows of W; 4,100 rows leave the
+    last block's second tile row beyond the matrix), the result added to a residual in place; shapes for which the
+    kernel that splits k over blocks is the faster one refuse a residual."""
+    g = torch.Generator().manual_seed(83)
+    x = torch.randn(n, k, generator=g).to(torch.bfloat16)
+    w = (torch.randn(m, k, generator=g) * 0.05).to(torch.bfloat16)
+    b = torch.randn(m, generator=g)
+    res = torch.randn(n, m, generator=g)
+    h = res.to(DEV)
+    if not ops().linear_bf16_adds_residual(n, m, k):
+        assert n > 32 and k > 3000
+        with pytest.raises(ops().KernelError, match="residual"):
+            ops().linear_bf16(x.to(DEV), w.to(DEV), b.to(DEV), h, residual=h)
+        return
+    out = ops().linear_bf16(x.to(DEV), w.to(DEV), b.to(DEV), h, residual=h)
+    assert out is h
+    assert rel_err(h, res.double() + x.double() @ w.double().t() + b.double()) < 2e-5
+    with pytest.raises(ops().KernelError, match="residual"):
+        big = torch.zeros(65, m, device=DEV)
+        ops().linear_bf16(torch.zeros(65, k, dtype=torch.bfloat16, device=DEV), w.to(DEV), None, big, residual=big)
+
+
+def test_linear_bf16_says_which_shapes_take_a_residual():
+    o = ops()
+    assert o.linear_bf16_adds_residual(16, 3584, 18944) and o.linear_bf16_adds_residual(1, 50, 64)
+    assert not o.linear_bf16_adds_residual(8, 50, 53)            # k no multiple of 8: the any-shape kernel
+    assert o.linear_bf16_adds_residual(64, 3584, 3584)           # 224 tile rows: one block each, whole k
+    assert o.linear_bf16_adds_residual(64, 4608, 3584)           # 288 tile rows: two per block
+    assert not o.linear_bf16_adds_residual(64, 3584, 18944)      # a long k at 64 rows: split over blocks is faster
+    assert not o.linear_bf16_adds_residual(64, 152064, 3584)     # many rows: nothing to split
+    assert not o.linear_bf16_adds_residual(65, 3584, 3584)
 
 
 def test_linear_bf16_odd_k_uses_plain_kernel():

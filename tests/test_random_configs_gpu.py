@@ -30,10 +30,21 @@ def draw_config(seed: int) -> dict:
 
 @pytest.mark.parametrize("seed", range(8))
 def test_random_configuration(seed, tmp_path):
+    check_configuration(draw_config(100 + seed), seed, tmp_path)
+
+
+@pytest.mark.parametrize("hidden,inter", [(100, 100), (104, 84), (76, 136)])
+def test_widths_that_are_no_multiple_of_eight(hidden, inter, tmp_path):
+    """The vectorised kernels (16-byte accesses, fused norm and residual) do not take these widths: the any-shape
+    kernels must, in every mode."""
+    cfg = dict(draw_config(3), hidden_size=hidden, intermediate_size=inter, num_hidden_layers=2, max_window_layers=1)
+    check_configuration(cfg, hidden, tmp_path)
+
+
+def check_configuration(cfg, seed, tmp_path):
     from vt_transformer_amd.config import config_from_dict
     from vt_transformer_amd.engine import StepEntry, load_model, make_runner
     from vt_transformer_amd.weights import write_random_model
-    cfg = draw_config(100 + seed)
     folder = str(tmp_path / "m")
     write_random_model(config_from_dict(cfg), folder, seed=seed)
     pcfg, w = plain_model.read_folder(folder)

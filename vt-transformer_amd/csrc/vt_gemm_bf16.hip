@@ -371,6 +371,132 @@ __global__ __launch_bounds__(WM * 64) void gemm_mid_kernel(const bf16_t* __restr
         }
 }
 
+// ---------------------------------------------------------------------------
+// 17 to 64 tokens, k not split over blocks: as in the few-row kernel a block owns one tile row of W (16 features)
+// and all of k, which its WPB waves split, and the waves' sums meet in LDS in wave order; each wave multiplies a
+// tile of W with NT token tiles of 16 rows, whose pieces it reads row by row (16 accesses of 64 bytes per tile) and
+// hands to their lanes through LDS of its own.  Every block reads all the tokens (64 x k values from the second-level
+// cache, four times the bytes of its share of W); in exchange nothing is left to add up afterwards, so the result can
+// take a residual with it, and a matrix of 224 tile rows fills the compute units without a split.
+// ---------------------------------------------------------------------------
+// slots (16 bytes) of one k tile of a wave's exchange buffer: NT token tiles of 4 pieces x 17 rows, and 8 more where
+// that is a multiple of 16, so that the two tiles of a pair, which a wave writes together, lie 32 banks apart
+template <int NT>
+__host__ __device__ constexpr int rows_tile_slots() { return NT * 4 * 17 + ((NT * 4 * 17) % 16 == 0 ? 8 : 0); }
+
+template <int WPB, int NT>
+__host__ __device__ constexpr int rows_lds_bytes() {
+    constexpr int exchange = WPB * 2 * rows_tile_slots<NT>() * 16, sums = WPB * NT * 256 * 4;
+    return exchange > sums ? exchange : sums;
+}
+
+template <int WPB, int NT, int R, typename TO>
+__global__ __launch_bounds__(WPB * 64) void gemm_rows_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wp,
+                                                            const float* __restrict__ bias, TO* __restrict__ y, int N,
+                                                            int Mout, int K, int KT, const float* resid) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char rows_lds[];
+    const int tid = threadIdx.x, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = tid & 63;
+    const int r = lane & 15, g = lane >> 4;
+    const int m_tiles = (Mout + 15) >> 4;
+    // the waves split k in pairs of tiles (KT is a multiple of 4): a token's 64 values of a pair are one cache line
+    const int KP = KT >> 1;
+    const int p_begin = (int)(((long long)wv * KP) / WPB), p_end = (int)(((long long)(wv + 1) * KP) / WPB);
+    // this block's R tile rows; beyond the matrix the last one again (its results are not stored)
+    const bf16_t* wbase[R];
+#pragma unroll
+    for (int j = 0; j < R; ++j) wbase[j] = wp + ((size_t)min((int)blockIdx.x * R + j, m_tiles - 1) * KT * 64 + lane) * 8;
+    // Lane l reads piece l % 8 (8 values) of rows l / 8 and l / 8 + 8 of each token tile: eight lanes read a whole
+    // cache line, a load is eight accesses (by 32 values, a tile at a time, it would be sixteen of half a line, and
+    // it is the number of accesses that the first-level cache limits).  Pieces 0..3 belong to the pair's first tile.
+    const bf16_t* xrow[NT][2];
+#pragma unroll
+    for (int i = 0; i < NT; ++i) {
+        xrow[i][0] = x + (size_t)min(16 * i + (lane >> 3), N - 1) * K;
+        xrow[i][1] = x + (size_t)min(16 * i + (lane >> 3) + 8, N - 1) * K;
+    }
+    const int xpiece = (lane & 7) * 8;
+    constexpr int TS = rows_tile_slots<NT>();
+    uint4* const xt = (uint4*)rows_lds + (size_t)wv * 2 * TS;      // this wave's [2 tiles][NT][4 * 17] slots
+    const int wslot = ((lane & 7) >> 2) * TS + (lane & 3) * 17 + (lane >> 3), rslot = g * 17 + r;
+    f32x4_t acc[R][NT];
+#pragma unroll
+    for (int j = 0; j < R; ++j)
+#pragma unroll
+        for (int i = 0; i < NT; ++i) acc[j][i] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+    // Blocks that start together would walk the tokens' lines in step and meet at the same channels of the
+    // second-level cache: every block starts at another pair of its waves' ranges.
+    const int p_len = p_end - p_begin;
+    int p = p_begin + (p_len > 0 ? (int)(blockIdx.x % (unsigned)p_len) : 0);
+    for (int q = 0; q < p_len; ++q, p = (p + 1 < p_end) ? p + 1 : p_begin) {
+        Frag wa[2][R], xa[NT][2];
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int j = 0; j < R; ++j) wa[u][j].u = *(const uint4*)(wbase[j] + (size_t)(2 * p + u) * PK_TILE);
+#pragma unroll
+        for (int i = 0; i < NT; ++i) {
+            xa[i][0].v = load_x(xrow[i][0], p * 64 + xpiece, K);
+            xa[i][1].v = load_x(xrow[i][1], p * 64 + xpiece, K);
+        }
+#pragma unroll
+        for (int i = 0; i < NT; ++i) {
+            xt[i * 4 * 17 + wslot] = xa[i][0].u;
+            xt[i * 4 * 17 + wslot + 8] = xa[i][1].u;
+        }
+        wave_lds_order();
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int i = 0; i < NT; ++i) {
+                Frag xf;
+                xf.u = xt[u * TS + i * 4 * 17 + rslot];
+#pragma unroll
+                for (int j = 0; j < R; ++j)
+                    acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[u][j].v, xf.v, acc[j][i], 0, 0, 0);
+            }
+        wave_lds_order();       // the next pair is written after these reads
+    }
+    // acc[j][i][e] is feature 16 (R blockIdx.x + j) + 4 g + e of token 16 i + r.  The waves' sums take the exchange
+    // buffers' place, one tile row at a time.
+    float* const red = (float*)rows_lds;            // [WPB][NT][256]
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < NT; ++i) *(f32x4_t*)&red[((size_t)wv * NT + i) * 256 + lane * 4] = acc[j][i];
+        __syncthreads();
+        const int mt = blockIdx.x * R + j;
+        for (int c = tid; c < NT * 256; c += WPB * 64) {
+            const int i = c >> 8, cc = c & 255, ln = cc >> 2, e = cc & 3;
+            const int m = mt * 16 + 4 * (ln >> 4) + e, n = 16 * i + (ln & 15);
+            float v = 0.f;
+            for (int q = 0; q < WPB; ++q) v += red[((size_t)q * NT + i) * 256 + cc];
+            if (m < Mout && n < N) {
+                if (bias) v += bias[m];
+                if (resid) v += resid[(size_t)n * Mout + m];
+                store_f32<TO>(y, (size_t)n * Mout + m, v);
+            }
+        }
+    }
+}
+
+template <int WPB, int NT, int R, typename TO>
+static int launch_rows(const bf16_t* x, const bf16_t* wp, const float* bias, TO* y, int N, int Mout, int K, int KT,
+                       const float* resid, hipStream_t stream) {
+    constexpr int lds = rows_lds_bytes<WPB, NT>();
+    static bool set = false;
+    if (!set) {
+        hipError_t e = hipFuncSetAttribute((const void*)gemm_rows_kernel<WPB, NT, R, TO>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        VT_REQUIRE(e == hipSuccess, "vt_linear_bf16: cannot get %d bytes of LDS: %s", lds, hipGetErrorString(e));
+        set = true;
+    }
+    const int m_tiles = (Mout + 15) / 16;
+    gemm_rows_kernel<WPB, NT, R, TO><<<(m_tiles + R - 1) / R, WPB * 64, lds, stream>>>(x, wp, bias, y, N, Mout, K, KT, resid);
+    VT_CHECK_LAUNCH("vt_linear_bf16(rows)");
+    return 0;
+}
+
 // y[i] = sum over splits of partial[s][i], added in split order
 template <typename TO>
 __global__ void sum_partials_kernel(const float* __restrict__ partial, TO* __restrict__ y, size_t n, int splits) {
@@ -413,6 +539,8 @@ __global__ void gemm_plain_kernel(const bf16_t* __restrict__ x, const bf16_t* __
     }
     store_f32<TO>(y, (size_t)n * Mout + m, v);
 }
+
+#define ROWS_MAX 64                 // rows up to which a plain product keeps k inside a block (gemm_rows_kernel)
 
 static int compute_units() {
     static int cus = 0;
@@ -458,22 +586,45 @@ static int mid_waves(int Mout, int rows_per_wave, int token_blocks) {
     return best;
 }
 
+// 17 to 64 rows: tile rows per block (1 or 2) if gemm_rows_kernel takes the product, 0 if the 64-token kernel does.
+// The first lasts about 4 us + 0.026 us per k tile and token tile (every block takes in all the tokens, and that
+// is what its time goes to, however many rows of W it has); the second about 14 us, the launch that adds its
+// partial sums included, + 0.21 us per MB of W (measured at 7B and 1.5B layer sizes).  From the shape of W and
+// whether the rows are more than 32 only.
+static int rows_tile_rows(int N, int Mout, int K) {
+    if (N <= 16 || N > ROWS_MAX || K % 8 != 0) return 0;
+    const int tiles = (Mout + 15) / 16, cus = compute_units();
+    const int rr = tiles <= cus ? 1 : 2;
+    if ((tiles + rr - 1) / rr > cus) return 0;      // many rows: the 64-token kernel needs no split there
+    const double rows_us = 4. + 0.026 * (pk_cols(K) / 32) * (N <= 32 ? 2 : 4);
+    const double mid_us = 14. + 0.21 * 2e-6 * Mout * K;
+    return rows_us < mid_us ? rr : 0;
+}
+
+// whether a plain product of N rows keeps all of k inside a block, so that it can add its result to a residual
+extern "C" int vt_linear_bf16_adds_residual(int N, int M, int K) {
+    if (N <= 0 || M <= 0 || K <= 0 || K % 8 != 0) return 0;
+    return N <= 16 || rows_tile_rows(N, M, K) > 0;
+}
+
 extern "C" long long vt_linear_bf16_workspace(int N, int M, int K, int gated) {
     // floats of workspace that vt_linear_bf16 / vt_gated_linear_bf16 need for this shape (0: none)
     if (N <= 16 || K % 8 != 0 || gated) return 0;
+    if (rows_tile_rows(N, M, K)) return 0;       // gemm_rows_kernel: nothing is split
     const int splits = mid_splits(M, K, 128);
     return splits > 1 ? (long long)splits * N * M : 0;
 }
 
-// gain != null: x is the fp32 residual stream and the RMSNorm (gain, eps) is part of the product; resid != null: the
-// result is added to it.  Both only with up to 16 tokens.
+// gain != null: x is the fp32 residual stream and the RMSNorm (gain, eps) is part of the product (up to 16 tokens);
+// resid != null: the result is added to it (up to 64 tokens).
 template <bool SWIGLU, typename TO>
 static int linear_bf16(const void* xv, const bf16_t* wp, const float* bias, TO* y, float* workspace, int N, int Mout,
                        int K, const float* gain, float eps, const float* resid, hipStream_t stream) {
     if (N == 0) return 0;
     const bf16_t* x = (const bf16_t*)xv;
-    VT_REQUIRE((!gain && !resid) || (N <= 16 && K % 8 == 0 && (((uintptr_t)xv) & 15) == 0),
-               "vt_linear_bf16: the fused norm and residual need at most 16 rows and k a multiple of 8 (N=%d K=%d)", N, K);
+    VT_REQUIRE(!gain || N <= 16, "vt_linear_bf16: the fused norm needs at most 16 rows (N=%d)", N);
+    VT_REQUIRE((!gain && !resid) || (K % 8 == 0 && (((uintptr_t)xv) & 15) == 0),
+               "vt_linear_bf16: the fused norm and residual need k a multiple of 8 and aligned tokens (K=%d)", K);
     VT_REQUIRE(!gain || (((uintptr_t)gain) & 15) == 0, "vt_linear_bf16: the norm's gains are not 16-byte aligned");
     const int KT = pk_cols(K) / 32, up_tiles = pk_rows(Mout) / 16;
     VT_REQUIRE((((uintptr_t)wp) & 15) == 0, "vt_linear_bf16: the packed matrix is not 16-byte aligned");
@@ -482,6 +633,16 @@ static int linear_bf16(const void* xv, const bf16_t* wp, const float* bias, TO* 
         gemm_plain_kernel<SWIGLU, TO><<<dim3((Mout + 255) / 256, N), 256, 0, stream>>>(x, wp, bias, y, N, Mout, K, KT, up_tiles);
         VT_CHECK_LAUNCH("vt_linear_bf16(plain)");
         return 0;
+    }
+    const int rows_rr = SWIGLU ? 0 : rows_tile_rows(N, Mout, K);
+    VT_REQUIRE(!resid || N <= 16 || rows_rr, "vt_linear_bf16: %d rows of [%d, %d] do not take a residual "
+               "(vt_linear_bf16_adds_residual)", N, Mout, K);
+    if constexpr (!SWIGLU) {
+        // whole k in a block of 8 waves (gemm_rows_kernel)
+#define VT_ROWS(NT, RR) launch_rows<8, NT, RR, TO>(x, wp, bias, y, N, Mout, K, KT, resid, stream)
+        if (rows_rr == 1) return N <= 32 ? VT_ROWS(2, 1) : VT_ROWS(4, 1);
+        if (rows_rr == 2) return N <= 32 ? VT_ROWS(2, 2) : VT_ROWS(4, 2);
+#undef VT_ROWS
     }
     if (N > 16) {
         // 64 tokens per block through LDS; two tile rows per wave (one for the gated product, which has two
@@ -528,7 +689,7 @@ extern "C" int vt_linear_bf16(const void* x, const void* wp, const float* bias, 
     return vt_fail("vt_linear_bf16: unknown out dtype %d", out_dtype);
 }
 
-// The same for up to 16 tokens with an RMSNorm in front and a residual addition behind, each optional:
+// The same with an RMSNorm in front (up to 16 tokens) and a residual addition behind (up to 64), each optional:
 // gain != null: h is the fp32 residual stream [N, K] and y = (rmsnorm(h; gain, eps) . W^T) + bias, else h is x in bf16;
 // resid != null (fp32 [N, M], may be y): y = resid + that.  y is fp32.
 extern "C" int vt_linear_bf16_fused(const void* h, const float* gain, float eps, const void* wp, const float* bias,

@@ -229,14 +229,28 @@ def linear_bf16_workspace(n: int, m: int, k: int) -> int:
     return int(lib.vt_linear_bf16_workspace(_i(n), _i(m), _i(k), _i(0)))
 
 
+NORM_MAX_ROWS = 16         # rows up to which the few-row product applies an RMSNorm in front
+_adds_residual = {}
+
+
+def linear_bf16_adds_residual(n: int, m: int, k: int) -> bool:
+    """Whether linear_bf16 takes `residual` for x [n, k] and W [m, k]: up to 16 rows always (k a multiple of 8), 17
+    to 64 rows where the kernel that keeps all of k inside a block is the faster one for this W."""
+    key = (n, m, k)
+    if key not in _adds_residual:
+        _adds_residual[key] = bool(load_lib("vt_gemm_bf16").vt_linear_bf16_adds_residual(_i(n), _i(m), _i(k)))
+    return _adds_residual[key]
+
+
 def linear_bf16(x: torch.Tensor, w, bias: Optional[torch.Tensor], out: torch.Tensor,
                 workspace: Optional[torch.Tensor] = None, norm_gain: Optional[torch.Tensor] = None,
                 norm_eps: float = 0.0, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Few rows (decoding, short portions): W is read once per 64 rows.  w: a PackedMatrix (a plain [m, k] tensor
     is packed on the spot, which costs more than the product).  Shapes whose k range is split over blocks need
     `workspace` (float32, at least linear_bf16_workspace(n, m, k) elements).
-    Up to 16 rows, float32 output: with norm_gain, x is the float32 residual stream and rmsnorm(x; gain, eps) is
-    what gets multiplied; with residual (float32 [n, m], may be `out`), out = residual + the product."""
+    float32 output: with norm_gain (up to 16 rows), x is the float32 residual stream and rmsnorm(x; gain, eps) is
+    what gets multiplied; with residual (where linear_bf16_adds_residual says so; float32 [n, m], may be `out`), out =
+    residual + the product."""
     n, k = x.shape
     if not isinstance(w, PackedMatrix):
         _chk(w, "linear_bf16.w", torch.bfloat16, (w.shape[0], k))
@@ -251,8 +265,11 @@ def linear_bf16(x: torch.Tensor, w, bias: Optional[torch.Tensor], out: torch.Ten
     if bias is not None:
         _chk(bias, "linear_bf16.bias", torch.float32, (m,))
     if fused:
-        if n > 16 or k % 8:
-            raise KernelError(f"linear_bf16: the fused norm and residual take at most 16 rows and k a multiple of 8 (n={n}, k={k})")
+        if k % 8 or (norm_gain is not None and n > NORM_MAX_ROWS):
+            raise KernelError(f"linear_bf16: the fused norm takes at most {NORM_MAX_ROWS} rows and k a multiple of 8 "
+                              f"(n={n}, k={k})")
+        if residual is not None and not linear_bf16_adds_residual(n, m, k):
+            raise KernelError(f"linear_bf16: {n} rows of [{m}, {k}] do not take a residual (linear_bf16_adds_residual)")
         if norm_gain is not None:
             _chk(norm_gain, "linear_bf16.norm_gain", torch.float32, (k,))
         if residual is not None:

@@ -21,7 +21,7 @@ import torch
 from ..config.base import PartSpec
 from ..kernels import ops
 from .base import MIXERS, POSITIONS, CacheNeed, Part, Runtime, StateNeed, TensorDecl
-from .linear import linear
+from .linear import can_add_residual, linear
 
 
 def decode_bucket(n_kv: int) -> int:
@@ -32,7 +32,10 @@ def decode_bucket(n_kv: int) -> int:
 @MIXERS.register("attention")
 class PagedAttention(Part):
     takes_normed_input = True     # the q/k/v product applies the norm in front of it when the rows are few
-    adds_residual = True          # the output product adds to the residual stream when the rows are few
+
+    def adds_residual(self, rows: int) -> bool:
+        """Whether the output product adds to the residual stream itself at this many rows."""
+        return can_add_residual(self.rt, rows, self.width, self.nh * self.d)
 
     def __init__(self, *, rt: Runtime, width: int, prefix: str, num_heads: int, num_kv_heads: int, head_dim: int,
                  qkv_bias: bool = False, out_bias: bool = False, window: int = 0,

@@ -9,7 +9,8 @@ With few rows in bfloat16 (decoding) the norms and additions are not kernels of
 their own: a mixer or feed-forward that says so takes the residual stream with
 the norm still to be applied (`NormedInput`: its first matrix product applies
 it) and adds its result to the stream itself (`residual=`: its last matrix
-product does).
+product does; `adds_residual(rows)` says for how many rows it can, which reaches
+up to 64 for matrices that fill the GPU without splitting k over blocks).
 """
 from __future__ import annotations
 
@@ -49,7 +50,8 @@ class PreNormBlock(Part):
             x = NormedInput(h, norm)
         else:
             x = norm.forward(h, delta)
-        if fuse and getattr(part, "adds_residual", False):
+        adds = getattr(part, "adds_residual", None)
+        if adds is not None and adds(h.shape[0]):
             part.forward(x, *args, residual=h)
             return None
         return part.forward(x, *args)

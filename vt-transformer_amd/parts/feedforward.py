@@ -17,7 +17,7 @@ import torch
 from ..kernels import ops
 from .base import FEED_FORWARDS, Part, Runtime, TensorDecl
 from .base import NormedInput
-from .linear import SKINNY_MAX_ROWS, can_fuse, linear
+from .linear import SKINNY_MAX_ROWS, can_add_residual, can_fuse, linear
 
 
 @FEED_FORWARDS.register("gated_mlp")
@@ -53,7 +53,10 @@ class GatedMLP(Part):
         self.w_gu, self.w_down = rt.row_major(self.w_gu, self.p_gu), rt.row_major(self.w_down, self.p_down)
 
     takes_normed_input = True     # the gate/up product applies the norm in front of it when the rows are few
-    adds_residual = True          # the down product adds to the residual stream when the rows are few
+
+    def adds_residual(self, rows: int) -> bool:
+        """Whether the down product adds to the residual stream itself at this many rows."""
+        return can_add_residual(self.rt, rows, self.width, self.inter)
 
     def forward(self, x, ctx=None, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
         rt = self.rt

@@ -29,12 +29,19 @@ def packed_kernel_rows(m: int, k: int) -> int:
     return LONG_K_MAX_ROWS if k >= 4 * m else SKINNY_MAX_ROWS
 
 
-# the few-row kernel applies an RMSNorm in front and adds a residual behind for up to this many rows
-FUSE_MAX_ROWS = 16
+# the few-row kernel applies an RMSNorm in front for up to this many rows
+FUSE_MAX_ROWS = ops.NORM_MAX_ROWS
 
 
 def can_fuse(rt: Runtime, n: int) -> bool:
+    """Whether a product of n rows can take the residual stream with its norm still to be applied."""
     return rt.dtype == torch.bfloat16 and n <= FUSE_MAX_ROWS
+
+
+def can_add_residual(rt: Runtime, n: int, m: int, k: int) -> bool:
+    """Whether the product of n rows with W [m, k] can add its result to the residual stream itself: it can where
+    no k range is split over blocks (up to 16 rows; 17 to 64 for matrices that the kernel for it suits)."""
+    return rt.dtype == torch.bfloat16 and ops.linear_bf16_adds_residual(n, m, k)
 
 
 def linear(rt: Runtime, x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], name: str,
@@ -46,19 +53,21 @@ def linear(rt: Runtime, x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.T
     packed: W as rt.pack(w) made it, for the few-row kernel (made on the spot if missing: slow).
     x may be a NormedInput (the norm then happens inside the few-row kernel, or before the product as a kernel of
     its own where that is not possible).  residual (float32 [N, M]): the product is added to it in place and
-    `residual` is returned; only callers that checked `can_fuse(rt, n)` may pass it."""
+    `residual` is returned (by the product's kernel where `can_add_residual` says so, else by a kernel after it)."""
     n, k = x.shape
     m = w.shape[0] if w is not None else packed.rows      # (no row-major copy: the runtime keeps the packed one only)
     if residual is not None or isinstance(x, NormedInput):
-        if can_fuse(rt, n) and k % 8 == 0:
+        if isinstance(x, NormedInput) and not (can_fuse(rt, n) and k % 8 == 0):
+            x = x.materialize()
+        if isinstance(x, NormedInput) or can_add_residual(rt, n, m, k):
             norm = x if isinstance(x, NormedInput) else None
             out = residual if residual is not None else rt.buffer(name, (n, m), torch.float32)
             return ops.linear_bf16(norm.h if norm else x, packed if packed is not None else w, bias, out,
                                    norm_gain=norm.gain if norm else None, norm_eps=norm.eps if norm else 0.0,
                                    residual=residual)
         if residual is not None:
-            raise ValueError("linear: a residual to add to needs the few-row kernel (see can_fuse)")
-        x = x.materialize()
+            # a shape the fused kernels do not take (k no multiple of 8): the product, then the addition
+            return ops.residual_add(residual, linear(rt, x, w, bias, name, out_dtype, bias_lowp, packed))
     if rt.dtype == torch.float32:
         out = rt.buffer(name, (n, m), torch.float32)
         return ops.linear_f32(x, w, bias, out)
