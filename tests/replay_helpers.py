@@ -107,10 +107,10 @@ def run_in_process(runner, steps: List[dict]) -> Dict[int, np.ndarray]:
 
 
 def run_trace_run(model_dir: str, dtype: str, steps: List[dict], out_dir: str, max_tokens: int, vocab: int,
-                  env=None) -> Dict[int, np.ndarray]:
+                  env=None, extra_args: Tuple[str, ...] = ()) -> Dict[int, np.ndarray]:
     """Drive bin/trace_run as a user would: steps on stdin, `done <step>` awaited after each."""
     cmd = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", model_dir, "--dtype", dtype,
-           "--out", out_dir, "--max-tokens", str(max_tokens)]
+           "--out", out_dir, "--max-tokens", str(max_tokens), *extra_args]
     proc = subprocess.Popen(cmd, stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True, env=env)
     try:
         for s in steps:

@@ -389,3 +389,42 @@ def test_toy_mixer_with_state_toy_position_encoding_and_toy_routing():
     got_c = runner.step([StepEntry("c", c, list(range(12)))]).cpu()
     assert rel(got_c, rc) < 2e-5
     assert not runner._stateless and not runner._replayable     # such a model is never replayed from a captured graph
+
+
+def test_a_plugin_file_brings_an_architecture_to_the_replay_program(tmp_path):
+    """A model folder of an architecture that the package does not know, written with random weights, replayed by
+    bin/trace_run through its loader, cache (pages and state slots), step function and kernels: all it takes is a
+    file that registers the architecture and its parts, named on the command line."""
+    import os
+    from replay_helpers import cut, max_live_tokens, random_requests, run_trace_run, trace_mixed
+    from vt_transformer_amd.config import config_from_dict, register_architecture
+    from vt_transformer_amd.weights import write_random_model
+    register_toy_parts()
+    register_architecture("ToyStateForCausalLM", ToyConfig)
+    d = {"architectures": ["ToyStateForCausalLM"], "n_layer": 4, "width": 48, "inter": 64, "vocab": 90, "eps": 1e-6,
+         "decay": 0.9, "slope": 0.01, "experts": 3}
+    folder = write_random_model(config_from_dict(d), str(tmp_path / "toy"), seed=4, dtype=torch.float32)
+    plugin = tmp_path / "toy_plugin.py"
+    plugin.write_text(
+        "import sys\n"
+        f"sys.path.insert(0, {os.path.dirname(os.path.abspath(__file__))!r})\n"
+        "import test_parts_gpu as toy\n"
+        "from vt_transformer_amd.config import register_architecture\n"
+        "toy.register_toy_parts()\n"
+        "register_architecture('ToyStateForCausalLM', toy.ToyConfig)\n")
+    reqs = random_requests(d["vocab"], [23, 9, 31, 14, 18], seed=5)
+    portions = {r: cut(t, [5, 2, 7, 1]) for r, t in reqs.items()}
+    steps = trace_mixed(reqs, portions, max_live=3, seed=6)
+    got = run_trace_run(folder, "float32", steps, str(tmp_path / "out"), max_live_tokens(steps), d["vocab"],
+                        extra_args=("--plugin", str(plugin)))
+    _, w = pm.read_folder(folder)
+    ref = {r: toy_plain(d, w, t) for r, t in reqs.items()}
+    pos = {r: 0 for r in reqs}
+    for s in steps:
+        row = 0
+        for e in s["entries"]:
+            for j in e["want"]:
+                want = ref[e["id"]][pos[e["id"]] + j]
+                assert rel(torch.from_numpy(got[s["step"]][row].copy()), want) < 2e-5, (s["step"], e["id"], j)
+                row += 1
+            pos[e["id"]] += len(e["tokens"])

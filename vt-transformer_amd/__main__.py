@@ -67,6 +67,8 @@ def build_parser() -> argparse.ArgumentParser:
     p.add_argument("--single-weight-copy", action="store_true",
                    help="keep the bfloat16 matrices once instead of twice (half the memory, slower prompts)")
     # random weights
+    p.add_argument("--plugin", action="append", default=[], metavar="FILE.py|MODULE",
+                   help="code that registers further architectures or parts (may be repeated; also $VT_TRANSFORMER_PLUGINS)")
     p.add_argument("--write-random-model", type=str, metavar="DIR", help="write config.json and model.safetensors with random weights")
     p.add_argument("--config", type=str, help="config.json for --write-random-model")
     return p
@@ -92,6 +94,8 @@ def _parse_ids(text: str) -> List[int]:
 
 def main(argv: Optional[List[str]] = None) -> int:
     args = build_parser().parse_args(argv)
+    from .plugins import load_plugins
+    load_plugins(args.plugin)
     if args.write_random_model:
         if not args.config:
             raise SystemExit("--write-random-model needs --config FILE")
