@@ -181,7 +181,10 @@ class Engine:
     # -- the whole loop --------------------------------------------------------
     def generate(self, prompts: Union[Sequence[int], Sequence[Sequence[int]]],
                  params: Union[None, SamplingParams, Sequence[SamplingParams]] = None) -> List[List[int]]:
-        """Token ids in, generated token ids out (one list per prompt, in order)."""
+        """Token ids in, generated token ids out (one list per prompt, in order).  The requests of this call stay
+        readable (`requests`, `finish_reason`) until the next call, which forgets every finished request."""
+        for u in [u for u, r in self.requests.items() if r.state == "finished"]:
+            del self.requests[u]
         single = len(prompts) > 0 and not isinstance(prompts[0], (list, tuple))
         plist = [prompts] if single else list(prompts)
         if params is None or isinstance(params, SamplingParams):
@@ -196,3 +199,11 @@ class Engine:
 
     def finish_reason(self, uid: Hashable) -> Optional[str]:
         return self.requests[uid].finish_reason
+
+    def forget(self, uid: Hashable) -> Request:
+        """Drop a finished request from the engine's books (a caller of add_request/step does this once it has
+        read the request's output, or the books grow for as long as the engine lives); returns the request."""
+        req = self.requests[uid]
+        if req.state != "finished":
+            raise ValueError(f"request {uid!r} has not finished (abort it first)")
+        return self.requests.pop(uid)

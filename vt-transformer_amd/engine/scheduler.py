@@ -139,12 +139,16 @@ class Scheduler:
             return self.config.max_seq_len
         return min(p.num_pages for p in self.cache.pools) * self.cache.page_size
 
-    def _fits(self, items: List[Tuple[Request, int]]) -> bool:
+    def _need(self, items: List[Tuple[Request, int]]) -> List[int]:
+        """Pages per group that these (request, new length) pairs would take together."""
         need = [0] * len(self.cache.pools)
         for r, new_len in items:
-            for gi, n in enumerate(self.cache.pages_needed(self.cache.get(r.uid), new_len)):
-                need[gi] += n
-        return all(n <= p.available for n, p in zip(need, self.cache.pools))
+            for gi, k in enumerate(self.cache.pages_needed(self.cache.get(r.uid), new_len)):
+                need[gi] += k
+        return need
+
+    def _fits(self, items: List[Tuple[Request, int]]) -> bool:
+        return all(n <= p.available for n, p in zip(self._need(items), self.cache.pools))
 
     def _preempt(self, r: Request) -> None:
         self.cache.release(r.uid)
@@ -240,13 +244,6 @@ class Scheduler:
             planned.append((r, n))
             budget -= n
         return plan
-
-    def _need(self, items: List[Tuple[Request, int]]) -> List[int]:
-        need = [0] * len(self.cache.pools)
-        for r, new_len in items:
-            for gi, k in enumerate(self.cache.pages_needed(self.cache.get(r.uid), new_len)):
-                need[gi] += k
-        return need
 
     # -- after the step ------------------------------------------------------
     def update(self, plan: List[Scheduled], sampled: Dict[Hashable, int]) -> List[ReqResult]:
