@@ -83,3 +83,50 @@ def check_configuration(cfg, seed, tmp_path):
         runner.decode_graphs = True
         check_against_plain(folder, reqs, steps, run_in_process(runner, steps), dtype)
         assert sum(runner.cache.held_pages()) == 0
+
+
+@pytest.mark.parametrize("name,hidden,heads,kv,inter", [("7B", 3584, 28, 4, 18944), ("1.5B", 1536, 12, 2, 8960)])
+def test_real_layer_sizes(name, hidden, heads, kv, inter, tmp_path):
+    """Two layers at Qwen2-7B and Qwen2-1.5B layer sizes (a small vocabulary): the kernels choose their launch shapes
+    by these sizes (waves per block, k ranges, which product kernel), so the tiny configurations do not reach them.
+    Whole, cut, decoded one by one (eagerly and through captured graphs), and 40 copies of the request decoding side
+    by side (the 17-to-64-row kernels)."""
+    from vt_transformer_amd.config import config_from_dict
+    from vt_transformer_amd.engine import StepEntry, load_model, make_runner
+    from vt_transformer_amd.weights import write_random_model
+    cfg = dict(architectures=["Qwen2ForCausalLM"], model_type="qwen2", vocab_size=4099, hidden_size=hidden,
+               intermediate_size=inter, num_hidden_layers=2, num_attention_heads=heads, num_key_value_heads=kv, head_dim=128,
+               rope_theta=1e6, rms_norm_eps=1e-6, tie_word_embeddings=name == "1.5B", max_position_embeddings=8192,
+               hidden_act="silu", use_sliding_window=False, torch_dtype="bfloat16")
+    folder = str(tmp_path / "m")
+    write_random_model(config_from_dict(cfg), folder, seed=1)
+    pcfg, w = plain_model.read_folder(folder)
+    n = 200
+    toks = np.random.RandomState(0).randint(0, 4099, size=n).tolist()
+    ref = plain_model.forward(pcfg, w, toks)
+    scale = ref.abs().max()
+    for dtype, tol in (("bfloat16", 4e-2), ("float32", 3e-5)):
+        model = load_model(folder, dtype)
+        for mode in ("whole", "cut", "decode", "graph", "batch"):
+            runner = make_runner(model, pool_tokens=10240, page_size=16, max_requests=48, max_seq_len=512)
+            runner.decode_graphs = mode == "graph"
+            if mode == "whole":
+                cuts = [(0, n)]
+            elif mode == "cut":
+                cuts = [(0, 70), (70, 87), (87, 150), (150, 152), (152, 200)]
+            else:
+                cuts = [(0, n - 32)] + [(i, i + 1) for i in range(n - 32, n)]
+            if mode == "batch":
+                ids = [f"r{i}" for i in range(40)]
+                for i in ids:
+                    runner.admit(i)
+                    runner.step([StepEntry(i, toks[:n - 32], [])])
+                got = torch.stack([runner.step([StepEntry(i, toks[a:b], [0]) for i in ids]).float().cpu()
+                                   for a, b in cuts[1:]]).double()          # [32, 40, vocab]
+                err = float((got - ref[n - 32:, None, :]).abs().max() / scale)
+            else:
+                runner.admit("r")
+                got = torch.cat([runner.step([StepEntry("r", toks[a:b], list(range(b - a)))]).float().cpu() for a, b in cuts])
+                err = float((got.double() - ref).abs().max() / scale)
+            assert err < tol, (name, dtype, mode, err)
+        del model
