@@ -85,9 +85,10 @@ def check_configuration(cfg, seed, tmp_path):
         assert sum(runner.cache.held_pages()) == 0
 
 
-@pytest.mark.parametrize("name,hidden,heads,kv,inter", [("7B", 3584, 28, 4, 18944), ("1.5B", 1536, 12, 2, 8960)])
+@pytest.mark.parametrize("name,hidden,heads,kv,inter", [("7B", 3584, 28, 4, 18944), ("1.5B", 1536, 12, 2, 8960),
+                                                        ("72B", 8192, 64, 8, 29568)])
 def test_real_layer_sizes(name, hidden, heads, kv, inter, tmp_path):
-    """Two layers at Qwen2-7B and Qwen2-1.5B layer sizes (a small vocabulary): the kernels choose their launch shapes
+    """Two layers at Qwen2-7B, 1.5B and 72B layer sizes (a small vocabulary): the kernels choose their launch shapes
     by these sizes (waves per block, k ranges, which product kernel), so the tiny configurations do not reach them.
     Whole, cut, decoded one by one (eagerly and through captured graphs), and 40 copies of the request decoding side
     by side (the 17-to-64-row kernels)."""
