@@ -43,7 +43,7 @@ def main() -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--prompt-len", type=int, default=1024)
     ap.add_argument("--sizes", choices=sorted(SIZES), default="7b",
-                    help="layer sizes; 72b keeps one copy of the weights (prompts then go through the few-row kernels)")
+                    help="layer sizes; 72b keeps one copy of the weights (long prompt portions unpack each matrix for the library)")
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the model has (named in config)")
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")

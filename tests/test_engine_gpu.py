@@ -439,25 +439,29 @@ def test_group_of_17_query_heads_is_not_replayed_and_right(tmp_path):
 
 
 def test_single_weight_copy_gives_the_same_logits(model_folders):
-    """With the matrices kept once (packed) instead of twice, long portions go through the few-row kernels 64 rows
-    at a time: the same logits to rounding as with the GEMM library, no row-major matrix left on the device."""
+    """With the matrices kept once (packed) instead of twice, portions of up to 255 rows go through the few-row kernels
+    64 rows at a time, longer ones unpack each matrix into scratch memory for the GEMM library: the same logits to
+    rounding as with two copies, no row-major matrix left on the device."""
     from vt_transformer_amd.engine import Engine, StepEntry
-    toks = random_requests(TINY["W"]["vocab_size"], [200], seed=31)["r0"]
+    toks = random_requests(TINY["W"]["vocab_size"], [480], seed=31)["r0"]
     logits = []
     for single in (False, True):
-        eng = Engine(model_folders["W"], dtype="bfloat16", num_pages=32, max_running_reqs=2, max_seq_len=256,
+        eng = Engine(model_folders["W"], dtype="bfloat16", num_pages=40, max_running_reqs=2, max_seq_len=512,
                      single_weight_copy=single)
         mixer = eng.model.layers[0].mixer
         assert (mixer.w_qkv is None) == single and mixer.p_qkv is not None
         assert (eng.model.layers[0].feed_forward.w_down is None) == single
         eng.runner.admit("x")
-        out = [eng.runner.step([StepEntry("x", toks[:150], list(range(150)))]).float().cpu()]
-        out += [eng.runner.step([StepEntry("x", toks[i:i + 1], [0])]).float().cpu() for i in range(150, 160)]
+        out = [eng.runner.step([StepEntry("x", toks[:150], list(range(150)))]).float().cpu()]               # few-row kernels
+        out += [eng.runner.step([StepEntry("x", toks[150:450], list(range(0, 300, 3)))]).float().cpu()]     # unpacked
+        out += [eng.runner.step([StepEntry("x", toks[i:i + 1], [0])]).float().cpu() for i in range(450, 460)]
         logits.append(torch.cat(out))
+        assert ("linear.unpacked" in eng.model.rt._buffers) == single
     assert float((logits[0] - logits[1]).abs().max() / logits[0].abs().max()) < 2e-2
     cfg, w = plain_model.read_folder(model_folders["W"])
-    ref = plain_model.forward(cfg, w, toks[:160])
-    assert float((logits[1].double() - ref).abs().max() / ref.abs().max()) < 3e-2
+    ref = plain_model.forward(cfg, w, toks[:460])
+    rows = list(range(150)) + list(range(150, 450, 3)) + list(range(450, 460))
+    assert float((logits[1].double() - ref[rows]).abs().max() / ref.abs().max()) < 3e-2
 
 
 def test_library_algorithm_search_keeps_results(model_folders):

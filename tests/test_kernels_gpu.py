@@ -194,6 +194,15 @@ def test_linear_bf16_says_which_shapes_take_a_residual():
     assert not o.linear_bf16_adds_residual(65, 3584, 3584)
 
 
+@pytest.mark.parametrize("m,k,halves", [(16, 128, 1), (70, 53, 1), (1030, 3584, 1), (200, 96, 2), (37, 264, 2)])
+def test_unpack_gives_back_what_was_packed(m, k, halves):
+    g = torch.Generator().manual_seed(84)
+    w = torch.randn(halves * m, k, generator=g).to(torch.bfloat16).to(DEV)
+    packed = ops().pack_matrix_bf16(w, halves)
+    out = torch.full_like(w, float("nan"))
+    assert torch.equal(ops().unpack_matrix_bf16(packed, out), w)
+
+
 def test_linear_bf16_odd_k_uses_plain_kernel():
     g = torch.Generator().manual_seed(8)
     n, m, k = 5, 70, 53

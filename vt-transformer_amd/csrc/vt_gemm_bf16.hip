@@ -76,6 +76,38 @@ extern "C" int vt_pack_matrix_bf16(const void* w, void* wp, int M, int K, hipStr
     return 0;
 }
 
+// The way back: one thread per 16-byte piece of the packed matrix writes its eight values into the row-major matrix.
+// (A model that is kept packed only gets the row-major form of a matrix back for as long as a long portion's product
+// through the GEMM library needs it.)
+__global__ void unpack_matrix_kernel(const bf16_t* __restrict__ wp, bf16_t* __restrict__ w, int M, int K, int KT, size_t pieces) {
+    const size_t p = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (p >= pieces) return;
+    const int lane = (int)(p & 63);
+    const size_t tile = p >> 6;
+    const int kt = (int)(tile % KT), mt = (int)(tile / KT);
+    const int m = mt * 16 + (lane & 15), k = kt * 32 + (lane >> 4) * 8;
+    if (m >= M || k >= K) return;
+    const uint4 v = *(const uint4*)(wp + p * 8);
+    bf16_t* dst = w + (size_t)m * K + k;
+    if (k + 8 <= K && (((uintptr_t)dst) & 15) == 0) {
+        *(uint4*)dst = v;
+    } else {
+        const uint32_t e[4] = {v.x, v.y, v.z, v.w};
+        for (int j = 0; j < 8 && k + j < K; ++j) dst[j] = (bf16_t)(e[j >> 1] >> (16 * (j & 1)));
+    }
+}
+
+// w [M, K] row-major from wp as vt_pack_matrix_bf16 made it
+extern "C" int vt_unpack_matrix_bf16(const void* wp, void* w, int M, int K, hipStream_t stream) {
+    VT_REQUIRE(M > 0 && K > 0, "vt_unpack_matrix_bf16: bad sizes M=%d K=%d", M, K);
+    VT_REQUIRE((((uintptr_t)wp) & 15) == 0, "vt_unpack_matrix_bf16: the packed matrix must be 16-byte aligned");
+    const int KT = pk_cols(K) / 32;
+    const size_t pieces = (size_t)(pk_rows(M) / 16) * KT * 64;
+    unpack_matrix_kernel<<<(unsigned)((pieces + 255) / 256), 256, 0, stream>>>((const bf16_t*)wp, (bf16_t*)w, M, K, KT, pieces);
+    VT_CHECK_LAUNCH("vt_unpack_matrix_bf16");
+    return 0;
+}
+
 typedef __attribute__((ext_vector_type(2))) float f32x2_t;
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
 // two floats to two bf16 (round to nearest even) in one instruction

@@ -33,7 +33,8 @@ class Engine:
         tune_gemm: let the GEMM library try its algorithms on this model's products at chunk_size rows (and at 128
         and 256 rows, if so many requests may run) once, at start-up (some seconds), and use the fastest from then on.
         single_weight_copy: keep the bfloat16 matrices once (in the few-row kernels' order) instead of twice; long
-        prompt portions are then several times slower.  For models that fit the GPU's memory once but not twice."""
+        prompt portions then unpack each matrix into scratch memory for the GEMM library (a fifth slower at 7B sizes).
+        For models that fit the GPU's memory once but not twice."""
         sc = scheduler_config or SchedulerConfig()
         for k, v in options.items():
             if not hasattr(sc, k):

@@ -222,6 +222,18 @@ def pack_matrix_bf16(w: torch.Tensor, halves: int = 1) -> PackedMatrix:
     return PackedMatrix(data, rows, cols, halves)
 
 
+def unpack_matrix_bf16(packed: PackedMatrix, out: torch.Tensor) -> torch.Tensor:
+    """The row-major matrix [halves * rows, cols] back from its packed form, into `out`."""
+    _chk(packed.data, "unpack_matrix_bf16.packed", torch.bfloat16)
+    _chk(out, "unpack_matrix_bf16.out", torch.bfloat16, (packed.halves * packed.rows, packed.cols))
+    lib = load_lib("vt_gemm_bf16")
+    per = packed.data.numel() // packed.halves
+    for h in range(packed.halves):
+        _run(lib, "vt_unpack_matrix_bf16", _ptr(packed.data[h * per:(h + 1) * per]),
+             _ptr(out[h * packed.rows:(h + 1) * packed.rows]), _i(packed.rows), _i(packed.cols), _stream())
+    return out
+
+
 def linear_bf16_workspace(n: int, m: int, k: int) -> int:
     """Floats of scratch memory that linear_bf16 needs for x [n, k], W [m, k] (0: none)."""
     lib = load_lib("vt_gemm_bf16")

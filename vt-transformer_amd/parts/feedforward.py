@@ -17,7 +17,7 @@ import torch
 from ..kernels import ops
 from .base import FEED_FORWARDS, Part, Runtime, TensorDecl
 from .base import NormedInput
-from .linear import SKINNY_MAX_ROWS, can_add_residual, can_fuse, linear
+from .linear import SKINNY_MAX_ROWS, UNPACK_MIN_ROWS, can_add_residual, can_fuse, linear
 
 
 @FEED_FORWARDS.register("gated_mlp")
@@ -65,13 +65,13 @@ class GatedMLP(Part):
         normed = isinstance(x, NormedInput)
         if normed and not (can_fuse(rt, n) and self.width % 8 == 0):
             x, normed = x.materialize(), False
-        if rt.dtype == torch.bfloat16 and (n <= SKINNY_MAX_ROWS or self.w_gu is None):
+        if rt.dtype == torch.bfloat16 and (n <= SKINNY_MAX_ROWS or (self.w_gu is None and (rt.keep_row_major or n < UNPACK_MIN_ROWS))):
             w = self.p_gu if self.p_gu is not None else self.w_gu
             if normed:
                 ops.gated_linear_bf16(x.h, w, act, norm_gain=x.gain, norm_eps=x.eps)
             else:
                 ops.gated_linear_bf16(x, w, act)
         else:
-            gu = linear(rt, x, self.w_gu, None, "mlp.gu")
+            gu = linear(rt, x, self.w_gu, None, "mlp.gu", packed=self.p_gu if self.w_gu is None else None)
             ops.silu_mul(gu, act)
         return linear(rt, act, self.w_down, None, "mlp.down", packed=self.p_down, residual=residual)

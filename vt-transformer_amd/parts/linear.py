@@ -24,6 +24,12 @@ SKINNY_MAX_ROWS = 64
 LONG_K_MAX_ROWS = 256
 
 
+# A model that keeps the packed copy only: from this many rows on, a product unpacks its matrix into scratch memory
+# and goes through the GEMM library (the unpacking costs about two passes over W, the few-row kernels one pass per 64
+# rows, and the library is the faster multiplier by far)
+UNPACK_MIN_ROWS = 256
+
+
 def packed_kernel_rows(m: int, k: int) -> int:
     """Rows up to which the hand-written kernel on the packed matrix multiplies [rows, k] by W[m, k]."""
     return LONG_K_MAX_ROWS if k >= 4 * m else SKINNY_MAX_ROWS
@@ -55,7 +61,7 @@ def linear(rt: Runtime, x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.T
     its own where that is not possible).  residual (float32 [N, M]): the product is added to it in place and
     `residual` is returned (by the product's kernel where `can_add_residual` says so, else by a kernel after it)."""
     n, k = x.shape
-    m = w.shape[0] if w is not None else packed.rows      # (no row-major copy: the runtime keeps the packed one only)
+    m = w.shape[0] if w is not None else packed.rows * packed.halves   # (no row-major copy: the runtime keeps the packed one only)
     if residual is not None or isinstance(x, NormedInput):
         if isinstance(x, NormedInput) and not (can_fuse(rt, n) and k % 8 == 0):
             x = x.materialize()
@@ -71,6 +77,9 @@ def linear(rt: Runtime, x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.T
     if rt.dtype == torch.float32:
         out = rt.buffer(name, (n, m), torch.float32)
         return ops.linear_f32(x, w, bias, out)
+    if w is None and not rt.keep_row_major and n >= UNPACK_MIN_ROWS:
+        # every product's matrix in turn in the same scratch memory (the largest one's size)
+        w = ops.unpack_matrix_bf16(packed, rt.buffer("linear.unpacked", (packed.halves * packed.rows, packed.cols), torch.bfloat16))
     if w is None or n <= (packed_kernel_rows(m, k) if packed is not None else SKINNY_MAX_ROWS):
         out = rt.buffer(name, (n, m), out_dtype or torch.float32)
         need = ops.linear_bf16_workspace(n, m, k) if n > 16 else 0
