@@ -341,13 +341,19 @@ def attention_case(dtype, nh, kvh, d, page_size, window, entries, seed, spike=Fa
                 first = out.clone()
             assert bool(torch.isfinite(out).all()), (target, rt)
             assert rel_err(out, first) < 1e-2, (target, rt)  # every way of cutting the work agrees to rounding
-        for rt in (1, 2):
-            items, _ = plan_tile_items(start, pos0, nh // kvh, window, kvh, np.arange(len(entries)), rt=rt)
+        # ... whole key ranges per item, and the longest items' keys cut into ranges that are merged afterwards
+        for rt, split in ((1, 0.), (2, 0.), (1, 0.3), (2, 0.3)):
+            items, _, citems, n_parts = plan_tile_items(start, pos0, nh // kvh, window, kvh, np.arange(len(entries)),
+                                                        rt=rt, split=split, head_dim=d)
+            part_o = torch.full((max(1, n_parts) * 4 * rt * kvh * 16 * d,), float("nan"), device=DEV)
+            part_ml = torch.full((max(1, n_parts) * 4 * rt * kvh * 32,), float("nan"), device=DEV)
             out.fill_(float("nan"))
             o.attention_bf16_tiles(q, kpd, vpd, btd, torch.from_numpy(items).to(DEV).reshape(-1), items.shape[0], out,
-                                   nh, kvh, d, window, scale, rt=rt)
-            assert bool(torch.isfinite(out).all()), ("tiles", rt)
-            assert rel_err(out, first) < 1e-2, ("tiles", rt)
+                                   nh, kvh, d, window, scale, rt=rt,
+                                   citems=torch.from_numpy(citems).to(DEV).reshape(-1) if len(citems) else None,
+                                   n_citems=len(citems), part_o=part_o, part_ml=part_ml, n_parts=n_parts)
+            assert bool(torch.isfinite(out).all()), ("tiles", rt, split)
+            assert rel_err(out, first) < 1e-2, ("tiles", rt, split)
     ref = torch.cat([ref_attention(qs[e][i], ks[e], vs[e], c + i, window, scale).reshape(1, -1)
                      for e, (c, n) in enumerate(entries) for i in range(n)])
     return out, ref

@@ -49,27 +49,57 @@ def test_every_row_gets_every_key_it_may_see_exactly_once(group, window, target,
 
 @pytest.mark.parametrize("group,window", [(1, 0), (7, 0), (5, 40)])
 @pytest.mark.parametrize("rt", [1, 2])
-def test_tile_items_cover_the_long_entries(group, window, rt):
+@pytest.mark.parametrize("split", [0., 0.5, 1.4, None])
+def test_tile_items_cover_the_long_entries(group, window, rt, split):
+    """Every row of a long entry meets every key it may see exactly once, whether or not the keys of the longest
+    items are cut into ranges; the ranges of an item have consecutive partial indices and one merge per 16-row tile."""
     lens = np.array([1, 300, 40, 2048, 260])
     pos0 = np.array([300, 0, 10, 77, 5000])
     start = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
     short, long = split_entries(start, group)
     assert sorted(list(short) + list(long)) == list(range(5))
     assert all(lens[e] * group >= 256 for e in long) and all(lens[e] * group < 256 for e in short)
-    items, got_rt = plan_tile_items(start, pos0.astype(np.int32), group, window, 4, long, rt=rt)
-    assert got_rt == rt
+    items, got_rt, citems, n_parts = plan_tile_items(start, pos0.astype(np.int32), group, window, 4, long,
+                                                     rt=rt if split is not None else None, split=split)
+    if split is not None:
+        assert got_rt == rt
+    rt = got_rt
     spans = [it[6] - it[5] for it in items.tolist()]
     assert spans == sorted(spans, reverse=True)                       # the longest first
-    seen = set()
+    if split == 0.:
+        assert n_parts == 0 and len(citems) == 0 and all(it[7] == -1 for it in items.tolist())
+    if split == 0.5 and window == 0:
+        assert n_parts > 0                      # (under a window of 40 no row sees keys enough to cut)
+    seen = {}            # (entry, row) -> key ranges
+    by_item = {}         # (entry, row0) -> [(lo, hi, part)]
     for entry, q_tok0, q_len, p0, row0, lo, hi, part in items.tolist():
-        assert part == -1 and lo % 16 == 0 and q_tok0 == start[entry]
-        for r_ in range(row0, min(row0 + 64 * rt, q_len * group)):
-            p = p0 + r_ // group
+        assert lo % 16 == 0 and q_tok0 == start[entry] and hi > lo and -1 <= part < n_parts
+        by_item.setdefault((entry, row0), []).append((lo, hi, part))
+    for (entry, row0), ranges in by_item.items():
+        ranges.sort()
+        assert all(a[1] == b[0] for a, b in zip(ranges, ranges[1:]))         # the ranges follow each other
+        if len(ranges) == 1:
+            assert ranges[0][2] == -1
+        else:
+            assert [r_[2] for r_ in ranges] == list(range(ranges[0][2], ranges[0][2] + len(ranges)))
+        lo, hi = ranges[0][0], ranges[-1][1]
+        for r_ in range(row0, min(row0 + 64 * rt, lens[entry] * group)):
+            p = pos0[entry] + r_ // group
             first = max(0, p - window + 1) if window else 0
             assert lo <= first and p < hi                               # all the keys the row may see are inside
             assert (entry, r_) not in seen
-            seen.add((entry, r_))
-    assert seen == {(e, r_) for e in long for r_ in range(lens[e] * group)}
+            seen[(entry, r_)] = True
+    assert set(seen) == {(e, r_) for e in long for r_ in range(lens[e] * group)}
+    # merges: one per existing 16-row tile of every cut item, naming its first partial index and number of ranges
+    want = set()
+    for (entry, row0), ranges in by_item.items():
+        if len(ranges) > 1:
+            for t in range(4 * rt):
+                if row0 + 16 * t < lens[entry] * group:
+                    want.add((int(start[entry]), int(lens[entry]), row0 + 16 * t, ranges[0][2], len(ranges), t))
+    assert {tuple(c) for c in citems.tolist()} == want and len(citems) == len(want)
+    used = sorted(p for rs in by_item.values() for _, _, p in rs if p >= 0)
+    assert len(set(used)) == len(used) and all(p < n_parts for p in used)
 
 
 def test_decode_chunk():

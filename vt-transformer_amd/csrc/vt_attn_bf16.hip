@@ -681,7 +681,7 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_tile_kernel(At
     const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int* it = a.items + (size_t)blockIdx.y * ITEM_INTS;
     const int entry = it[0], q_tok0 = it[1], q_len = it[2], pos0 = it[3], q_row0 = it[4];
-    const int key_lo = it[5], key_hi = it[6];
+    const int key_lo = it[5], key_hi = it[6], part = it[7];
     if (entry < 0) return;
     const int kvh = blockIdx.x;
     const int G = a.n_heads / a.n_kv;
@@ -890,6 +890,19 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_tile_kernel(At
     for (int rt = 0; rt < RT; ++rt) {
         if (!row_ok[rt]) continue;
         const float lt = ol[rt][0];
+        if (part >= 0) {
+            // one of several items over the keys of these rows: the unnormalised sums, for the merge (the item's
+            // 4 RT tiles of 16 rows lie one after the other, wave by wave)
+            const size_t slot = (((size_t)part * (4 * RT) + (wv * RT + rt)) * a.n_kv + kvh) * 16 + r;
+            float* po = a.part_o + slot * D;
+#pragma unroll
+            for (int t = 0; t < DT; ++t) *(f32x4_t*)(po + t * 16 + 4 * g) = o[rt][t];
+            if (g == 0) {
+                a.part_ml[slot * 2] = m[rt];
+                a.part_ml[slot * 2 + 1] = lt;
+            }
+            continue;
+        }
         const float inv = lt > 0.f ? 1.f / lt : 0.f;
         bf16_t* orow = a.out + ((size_t)(q_tok0 + ti[rt]) * a.n_heads + head[rt]) * D;
 #pragma unroll
@@ -995,17 +1008,21 @@ extern "C" int vt_attn_bf16(const void* q, const void* k_pages, const void* v_pa
     return 0;
 }
 
-// Long portions: items [n][8] as above, each 64 * rt rows (rt = 1 or 2) of one entry with all the keys they may
-// see (no split, the partial index is not used); one block of 4 waves per (item, kv head).
+// Long portions: items [n][8] as above, each 64 * rt rows (rt = 1 or 2) of one entry; one block of 4 waves per
+// (item, kv head).  An item holds all the keys its rows may see (partial index -1), or one of several ranges of them:
+// then it leaves its partial result in workspace slot (partial index * 4 rt + tile) and the combine items [m][6]
+// (one per 16-row tile, as above, with 4 rt tiles per item) merge the ranges.
 extern "C" int vt_attn_bf16_tiles(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
-                                  const int* items, int n_items, int rt, void* out, int n_heads, int n_kv, int page_size,
+                                  const int* items, int n_items, int rt, const int* citems, int n_citems, void* out,
+                                  float* part_o, float* part_ml, int n_heads, int n_kv, int page_size,
                                   int max_blocks, int num_pages, int window, float scale, hipStream_t stream) {
     if (check_common("vt_attn_bf16_tiles", n_heads, n_kv, page_size, max_blocks, num_pages)) return -1;
     VT_REQUIRE(rt == 1 || rt == 2, "vt_attn_bf16_tiles: %d row tiles per wave (1 or 2)", rt);
+    VT_REQUIRE(n_citems == 0 || (citems && part_o && part_ml), "vt_attn_bf16_tiles: split keys but no workspace");
     if (n_items <= 0) return 0;
     AttnArgs a;
     a.q = (const bf16_t*)q; a.k_pages = (const bf16_t*)k_pages; a.v_pages = (const bf16_t*)v_pages;
-    a.block_table = block_table; a.items = items; a.out = (bf16_t*)out; a.part_o = nullptr; a.part_ml = nullptr;
+    a.block_table = block_table; a.items = items; a.out = (bf16_t*)out; a.part_o = part_o; a.part_ml = part_ml;
     a.n_items = n_items; a.n_heads = n_heads; a.n_kv = n_kv; a.page_size = page_size; a.max_blocks = max_blocks;
     a.num_pages = num_pages; a.window = window; a.scale_log2 = scale * 1.4426950408889634f;
     a.entry_pos0 = nullptr; a.dec_params = nullptr; a.p_max = 0; a.ps_shift = shift_of(page_size);
@@ -1026,6 +1043,11 @@ extern "C" int vt_attn_bf16_tiles(const void* q, const void* k_pages, const void
     if (rt == 1) attn_bf16_tile_kernel<1><<<grid, 256, TILE_LDS_BYTES, stream>>>(a);
     else attn_bf16_tile_kernel<2><<<grid, 256, TILE_LDS_BYTES, stream>>>(a);
     VT_CHECK_LAUNCH("vt_attn_bf16_tiles");
+    if (n_citems > 0) {
+        attn_combine_kernel<false><<<dim3(n_citems, n_kv), 256, 0, stream>>>(citems, part_o, part_ml, (bf16_t*)out,
+                                                                            n_heads, n_kv, nullptr, nullptr, 0, window, 4 * rt);
+        VT_CHECK_LAUNCH("vt_attn_bf16_tiles(combine)");
+    }
     return 0;
 }
 

@@ -53,6 +53,11 @@ class AttentionPlan:
     tile_items: Optional[torch.Tensor] = None     # long entries: items of the LDS-tiled kernel
     n_tile_items: int = 0
     tile_rt: int = 1
+    tile_citems: Optional[torch.Tensor] = None    # ... and the merges of those whose keys were cut into ranges
+    n_tile_citems: int = 0
+    tile_part_o: Optional[torch.Tensor] = None
+    tile_part_ml: Optional[torch.Tensor] = None
+    n_tile_parts: int = 0
 
 
 MAX_PARTS = 128     # the merge kernel holds the weights of at most this many items per row tile
@@ -62,6 +67,16 @@ MAX_PARTS = 128     # the merge kernel holds the weights of at most this many it
 # with one and two row tiles per wave (measured on 512 to 4,096-token portions with and without earlier keys)
 TILE_SLOTS = 512
 TILE_STEP_US = {1: 2.1, 2: 2.45}
+# An item of the tiled kernel that is longer than TILE_CUT x the launch's balanced length (all items' steps shared
+# out over the slots) has its keys cut into ranges of about that length, each an item of its own, merged afterwards.
+# Measured with one and two row tiles and cuts at 0.7, 1, 1.4 and 2 (us, against no cut with the better of one and
+# two row tiles): a fresh 2,048-token portion with 28 query / 4 kv heads 74 (77), with 12 / 2 heads 50 (56), 4,096
+# tokens with 12 / 2 heads 104 (114); 2,048 tokens behind 2,048 earlier ones 148 (147), eight 1,024-token portions 102
+# (102), 64 / 8 heads 103 (103): no shorter cut helped anywhere, and cuts at 1 and below cost up to a fifth where the
+# items fill the GPU anyway.
+TILE_CUT = 1.4
+TILE_MIN_STEPS = 6      # no item's keys are cut into ranges of fewer steps than this
+TILE_MAX_PARTS = 8      # ... or into more ranges than this
 LONG_ENTRY_ROWS = 256   # entries with at least this many (token, head-of-group) rows go to the LDS-tiled kernel
 
 
@@ -74,25 +89,30 @@ def split_entries(entry_start: np.ndarray, group: int) -> Tuple[np.ndarray, np.n
 
 
 def plan_tile_items(entry_start: np.ndarray, entry_pos0: np.ndarray, group: int, window: int, n_kv: int,
-                    entries: np.ndarray, rt: Optional[int] = None, slots: int = TILE_SLOTS) -> Tuple[np.ndarray, int]:
-    """Items of the LDS-tiled kernel: 64 * rt rows of one entry and every key they may see, longest first so that
-    the blocks that finish last start first.  Returns (items [n, 8], rt).
+                    entries: np.ndarray, rt: Optional[int] = None, slots: int = TILE_SLOTS, head_dim: int = 128,
+                    split: Optional[float] = None) -> Tuple[np.ndarray, int, np.ndarray, int]:
+    """Items of the LDS-tiled kernel: 64 * rt rows of one entry and the keys they may see, longest first so that
+    the blocks that finish last start first.  Returns (items [n, 8], rt, combine items [m, 6], partial indices).
 
-    rt (row tiles per wave) is chosen by an estimate of the launch's length.  A block's step over 64 keys takes
-    about as long with two row tiles as with one (TILE_STEP_US), because a wave waits on its own chain of loads,
-    products and exponentials more than on the machine; `slots` blocks run at a time and the others follow as
-    blocks finish, so a launch lasts as long as its longest item or as all items' steps shared out over the
-    slots, whichever is more."""
+    A block's step over 64 keys takes about as long with two row tiles per wave as with one (TILE_STEP_US), because
+    a wave waits on its own chain of loads, products and exponentials more than on the machine; `slots` blocks run
+    at a time and the others follow as blocks finish, so a launch lasts as long as its longest item or as all items'
+    steps shared out over the slots, whichever is more.  The longest items of a fresh prompt (its last rows see
+    every key) are what a launch waits for when the items are few (few kv heads, one prompt): their keys are cut
+    into ranges, each an item of its own, whose partial results the merge kernel adds up (TILE_CUT).  `rt` (row
+    tiles per wave) and `split` (the length to cut to, in units of the balanced launch; 0: no cuts) override the
+    choice.  Heads above 128 keep whole items and choose rt by the estimate."""
     q_len = (entry_start[1:] - entry_start[:-1]).astype(np.int64)[entries]
     rows = q_len * group
     e_pos0_all = entry_pos0[entries].astype(np.int64)
+    none = (np.zeros((0, ATTN_ITEM_INTS), np.int32), rt or 1, np.zeros((0, ATTN_CITEM_INTS), np.int32), 0)
 
     def items_for(rt_: int):
         rpi = 64 * rt_
         n_tiles = (rows + rpi - 1) // rpi
         total = int(n_tiles.sum())
         if total == 0:
-            return np.zeros((0, ATTN_ITEM_INTS), np.int64), np.zeros((0,), np.int64)
+            return None
         which = np.repeat(np.arange(len(entries)), n_tiles)
         first = np.cumsum(n_tiles) - n_tiles
         row0 = (np.arange(total) - np.repeat(first, n_tiles)) * rpi
@@ -102,23 +122,60 @@ def plan_tile_items(entry_start: np.ndarray, entry_pos0: np.ndarray, group: int,
         min_p = e_pos0 + row0 // group
         max_p = e_pos0 + np.minimum(e_rows - 1, row0 + rpi - 1) // group
         lo = np.maximum(0, min_p - window + 1) if window > 0 else np.zeros_like(min_p)
-        key_lo, key_hi = (lo // 16) * 16, max_p + 1
-        return np.stack([ent, e_start, e_len, e_pos0, row0, key_lo, key_hi, np.full(total, -1)], axis=1), key_hi - key_lo
+        return dict(ent=ent, start=e_start, len=e_len, pos0=e_pos0, row0=row0, rows=e_rows, lo=(lo // 16) * 16, hi=max_p + 1)
 
-    def estimate(span: np.ndarray, rt_: int) -> float:
-        steps = (span + 63) // 64
+    def steps_of(it):
+        return (it["hi"] - it["lo"] + 63) // 64
+
+    def estimate(it, rt_: int) -> float:
+        steps = steps_of(it)
         return max(float(steps.max()), float(steps.sum()) * n_kv / slots) * TILE_STEP_US[rt_]
 
     if rt is None:
-        cands = [items_for(1), items_for(2)]
-        if cands[0][0].shape[0] == 0:
-            return cands[0][0].astype(np.int32), 1
-        rt = 1 if estimate(cands[0][1], 1) <= estimate(cands[1][1], 2) else 2
-        items, span = cands[rt - 1]
-    else:
-        items, span = items_for(rt)
-    order = np.argsort(-span, kind="stable")
-    return items[order].astype(np.int32), rt
+        if head_dim <= 128:
+            rt = 2          # (measured: with the longest items cut, two row tiles are as good as one or better)
+        else:
+            cands = [items_for(1), items_for(2)]
+            if cands[0] is None:
+                return none
+            rt = 1 if estimate(cands[0], 1) <= estimate(cands[1], 2) else 2
+    if split is None:
+        split = TILE_CUT if head_dim <= 128 else 0.
+    it = items_for(rt)
+    if it is None:
+        return none
+    steps = steps_of(it)
+    parts = np.ones_like(steps)
+    if split > 0:
+        balanced = float(steps.sum()) * n_kv / slots
+        target = max(TILE_MIN_STEPS, int(np.ceil(balanced * split)))
+        parts = np.minimum(np.where(steps > target, -(-steps // target), 1), TILE_MAX_PARTS)
+    total = len(parts)
+    n_all = int(parts.sum())
+    of = np.repeat(np.arange(total), parts)                   # item that each part belongs to
+    p_first = np.cumsum(parts) - parts
+    j = np.arange(n_all) - np.repeat(p_first, parts)          # index of the part within its item
+    per = (-(-steps // parts)) * 64                            # keys per part: whole steps
+    lo = it["lo"][of] + j * per[of]
+    hi = np.minimum(it["hi"][of], lo + per[of])
+    multi = parts > 1
+    part0 = np.cumsum(np.where(multi, parts, 0)) - np.where(multi, parts, 0)      # partial indices of split items
+    part_id = np.where(multi[of], part0[of] + j, -1)
+    items = np.stack([it["ent"][of], it["start"][of], it["len"][of], it["pos0"][of], it["row0"][of], lo, hi, part_id], axis=1)
+    keep = hi > lo                                            # (a last part can be empty when the steps do not divide)
+    order = np.argsort(-(hi - lo)[keep], kind="stable")
+    items = items[keep][order].astype(np.int32)
+    # an empty part still counts among its item's parts: its slot is never written, so it must not be merged.
+    n_real = np.bincount(of[keep], minlength=total)
+    cl = []
+    m = np.nonzero(multi)[0]
+    for t in range(4 * rt):
+        r0 = it["row0"][m] + 16 * t
+        ok = r0 < it["rows"][m]
+        mm = m[ok]
+        cl.append(np.stack([it["start"][mm], it["len"][mm], r0[ok], part0[mm], n_real[mm], np.full(len(mm), t)], axis=1))
+    citems = np.concatenate(cl).astype(np.int32) if cl else np.zeros((0, ATTN_CITEM_INTS), np.int32)
+    return items, rt, citems, int(np.where(multi, parts, 0).sum())
 
 
 def choose_row_tiles(entry_start: np.ndarray, group: int, n_kv: int, entries: np.ndarray, min_items: int = 768) -> int:
@@ -238,23 +295,29 @@ class StepContext:
         items, citems, n_parts = plan_attention_items(self.h_entry_start, self.h_entry_pos0, group, window, n_kv,
                                                       rt=row_tiles, entries=short)
         # (heads above 128: one block per compute unit at a time)
-        t_items, tile_rt = plan_tile_items(self.h_entry_start, self.h_entry_pos0, group, window, n_kv, long,
-                                           slots=TILE_SLOTS if head_dim <= 128 else TILE_SLOTS // 2)
+        t_items, tile_rt, t_citems, t_parts = plan_tile_items(
+            self.h_entry_start, self.h_entry_pos0, group, window, n_kv, long,
+            slots=TILE_SLOTS if head_dim <= 128 else TILE_SLOTS // 2, head_dim=head_dim)
         rt = self.rt
         tag = f"attnplan.{group}.{window}.{n_kv}.{head_dim}"
-        flat = np.concatenate([items.reshape(-1), citems.reshape(-1), t_items.reshape(-1)])
+        lists = [items, citems, t_items, t_citems]
+        flat = np.concatenate([x.reshape(-1) for x in lists])
         dev = rt.buffer(tag, (max(flat.size, 1),), torch.int32)
         if flat.size:
             dev[:flat.size].copy_(torch.from_numpy(flat))
-        d_items = dev[:items.size]
-        d_citems = dev[items.size:items.size + citems.size] if citems.size else None
-        d_tiles = dev[items.size + citems.size:flat.size] if t_items.size else None
-        part_o = part_ml = None
+        ends = np.cumsum([x.size for x in lists])
+        d_items, d_citems, d_tiles, d_tcitems = (dev[e - x.size:e] if x.size else None for x, e in zip(lists, ends))
+        if d_items is None:
+            d_items = dev[:0]
+        part_o = part_ml = t_part_o = t_part_ml = None
         if n_parts:
             part_o = rt.buffer("attn.part_o", (n_parts * row_tiles * n_kv * 16 * head_dim,), torch.float32)
             part_ml = rt.buffer("attn.part_ml", (n_parts * row_tiles * n_kv * 16 * 2,), torch.float32)
+        if t_parts:
+            t_part_o = rt.buffer("attn.tile_part_o", (t_parts * 4 * tile_rt * n_kv * 16 * head_dim,), torch.float32)
+            t_part_ml = rt.buffer("attn.tile_part_ml", (t_parts * 4 * tile_rt * n_kv * 16 * 2,), torch.float32)
         return AttentionPlan(d_items, items.shape[0], d_citems, citems.shape[0], part_o, part_ml, n_parts, row_tiles,
-                             d_tiles, t_items.shape[0], tile_rt)
+                             d_tiles, t_items.shape[0], tile_rt, d_tcitems, t_citems.shape[0], t_part_o, t_part_ml, t_parts)
 
 
 DECODE_BUCKETS = 8      # chunk lengths for 1, 2-3, 4-7, ... 128+ key/value heads

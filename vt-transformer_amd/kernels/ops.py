@@ -387,9 +387,14 @@ def attention_bf16(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor
 
 def attention_bf16_tiles(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
                          items: torch.Tensor, n_items: int, out: torch.Tensor, n_heads: int, n_kv: int, head_dim: int,
-                         window: int, scale: float, rt: int = 1) -> torch.Tensor:
+                         window: int, scale: float, rt: int = 1, citems: Optional[torch.Tensor] = None, n_citems: int = 0,
+                         part_o: Optional[torch.Tensor] = None, part_ml: Optional[torch.Tensor] = None,
+                         n_parts: int = 0) -> torch.Tensor:
     """Long portions: `items` as for attention_bf16, each 64 * rt rows of one entry against all the keys they may
-    see; key and value blocks go through LDS once per block of four waves."""
+    see, or (partial index >= 0) against one of several ranges of them; key and value blocks go through LDS once per
+    block of four waves.  `citems` [>=n_citems, 6] as for attention_bf16, one per 16-row tile of every item whose keys
+    were split (4 * rt tiles per item); part_o / part_ml: float32 workspaces of at least n_parts * 4 * rt * n_kv *
+    16 * head_dim and n_parts * 4 * rt * n_kv * 32 elements."""
     n = q.shape[0]
     num_pages, kvh, page_size, d = k_pages.shape
     if head_dim % 16 or not 16 <= head_dim <= 256:
@@ -404,9 +409,20 @@ def attention_bf16_tiles(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
     _chk(out, "attention_bf16_tiles.out", torch.bfloat16, (n, n_heads * head_dim))
     if items.numel() < n_items * ATTN_ITEM_INTS:
         raise KernelError("attention_bf16_tiles: item list shorter than n_items")
+    if n_citems or n_parts:
+        if citems is None or part_o is None or part_ml is None:
+            raise KernelError("attention_bf16_tiles: split keys need citems and the two workspaces")
+        _chk(citems, "attention_bf16_tiles.citems", torch.int32)
+        _chk(part_o, "attention_bf16_tiles.part_o", torch.float32)
+        _chk(part_ml, "attention_bf16_tiles.part_ml", torch.float32)
+        if citems.numel() < n_citems * ATTN_CITEM_INTS:
+            raise KernelError("attention_bf16_tiles: combine list shorter than n_citems")
+        if part_o.numel() < n_parts * 4 * rt * n_kv * 16 * head_dim or part_ml.numel() < n_parts * 4 * rt * n_kv * 32:
+            raise KernelError(f"attention_bf16_tiles: workspaces too small for {n_parts} partial results")
     _run(load_lib("vt_attn_bf16", head_dim), "vt_attn_bf16_tiles", _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
-         _ptr(items), _i(n_items), _i(rt), _ptr(out), _i(n_heads), _i(n_kv), _i(page_size), _i(block_table.shape[1]),
-         _i(num_pages), _i(window), _f(scale), _stream())
+         _ptr(items), _i(n_items), _i(rt), _ptr(citems if n_citems else None), _i(n_citems), _ptr(out),
+         _ptr(part_o if n_citems else None), _ptr(part_ml if n_citems else None), _i(n_heads), _i(n_kv), _i(page_size),
+         _i(block_table.shape[1]), _i(num_pages), _i(window), _f(scale), _stream())
     return out
 
 

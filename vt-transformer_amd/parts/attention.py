@@ -161,5 +161,7 @@ class PagedAttention(Part):
                                    max_part=plan.n_parts, rt=plan.rt)
             if plan.n_tile_items:   # long portions: key/value blocks through LDS, shared by four waves
                 ops.attention_bf16_tiles(q, cache.k, cache.v, cache.block_table, plan.tile_items, plan.n_tile_items,
-                                         out, nh, nkv, d, self.window, self.scale, rt=plan.tile_rt)
+                                         out, nh, nkv, d, self.window, self.scale, rt=plan.tile_rt,
+                                         citems=plan.tile_citems, n_citems=plan.n_tile_citems,
+                                         part_o=plan.tile_part_o, part_ml=plan.tile_part_ml, n_parts=plan.n_tile_parts)
         return linear(rt, out, self.w_o, self.b_o, "attn.o", packed=self.p_o, residual=residual)
