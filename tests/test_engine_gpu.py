@@ -476,3 +476,29 @@ def test_library_algorithm_search_keeps_results(model_folders):
         logits.append(eng.runner.step([StepEntry("x", toks, [149])]).float().cpu())
         assert sum(eng.runner.cache.held_pages()) == 10
     assert float((logits[0] - logits[1]).abs().max() / logits[0].abs().max()) < 2e-2
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_long_prompt_whole_and_in_two_portions(model_folders, dtype):
+    """1,800 tokens: in bfloat16 the last rows' keys are cut into ranges that are merged afterwards (whole: a fresh
+    portion; in two portions: the second one has 1,000 keys in the cache in front of it)."""
+    from vt_transformer_amd.engine import StepEntry, load_model
+    cfg = "B"
+    toks = random_requests(TINY[cfg]["vocab_size"], [1800], seed=41)["r0"]
+    pc, pw = plain_model.read_folder(model_folders[cfg])
+    rows = list(range(0, 1800, 37)) + [1799]
+    ref = plain_model.forward(pc, pw, toks)[rows]
+    model = load_model(model_folders[cfg], dtype)
+    tol = 3e-5 if dtype == "float32" else 4e-2
+    for cuts in ([(0, 1800)], [(0, 1000), (1000, 1800)]):
+        r = runner_for(model, 1856, max_requests=2)
+        r.admit("x")
+        got = torch.cat([r.step([StepEntry("x", toks[a:b], [i - a for i in rows if a <= i < b])]).float().cpu() for a, b in cuts])
+        err = float((got.double() - ref).abs().max() / ref.abs().max())
+        assert err < tol, (cuts, err)
+    # (the planner does cut this shape: three kv heads, one query head each, head size 32)
+    from vt_transformer_amd.engine.step import plan_tile_items
+    for pos0, n in ((0, 1800), (1000, 800)):
+        _, _, citems, n_parts = plan_tile_items(np.array([0, n], np.int32), np.array([pos0], np.int32), 1, 0, 3,
+                                                np.arange(1), head_dim=32)
+        assert n_parts > 0 and len(citems) > 0
