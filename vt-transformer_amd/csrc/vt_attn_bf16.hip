@@ -240,8 +240,9 @@ __device__ __forceinline__ void rot_apply(float (&x)[CH], const RotIn<CH>& r) {
 // Merge the partial results of a tile of 16 rows whose keys were split over n_parts items; all 256 threads of a
 // block.  sm and sl are [MAX_PARTS][16] floats of LDS.  Slot of (part pi, row r) = slot0 + pi * slot_step + r.
 #define MAX_PARTS 128
-__device__ __forceinline__ void merge_parts(float (*sm)[16], float (*sl)[16], const float* part_o, const float* part_ml,
-                                            bf16_t* out, size_t slot0, size_t slot_step, int n_parts, int n_valid,
+__device__ __forceinline__ void merge_parts(float (*sm)[16], float (*sl)[16], const float* __restrict__ part_o,
+                                            const float* __restrict__ part_ml, bf16_t* __restrict__ out, size_t slot0,
+                                            size_t slot_step, int n_parts, int n_valid,
                                             int q_tok0, int q_row0, int G, int kvh, int n_heads) {
     const int tid = threadIdx.x;
     // With few rows and parts (decoding) a thread's share of the partial outputs is on its way from memory while
@@ -292,15 +293,20 @@ __device__ __forceinline__ void merge_parts(float (*sm)[16], float (*sl)[16], co
         }
         return;
     }
-    for (int idx = tid; idx < n_valid * D; idx += 256) {
-        const int r = idx / D, d = idx - r * D;
+    // four elements of four dims per thread and turn, so that the loads of a turn are in flight together (one element
+    // per turn made a chain of as many round trips as the row tile has elements per thread)
+    for (int idx = tid * 4; idx < n_valid * D; idx += 256 * 4) {
+        const int r = idx / D, d = idx - r * D;           // D is a multiple of 16: the four dims are of one row
         const float* po = part_o + (slot0 + r) * D + d;
-        float acc = 0.f;
+        f32x4_t acc = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll 4
-        for (int pi = 0; pi < n_parts; ++pi) acc += sm[pi][r] * po[(size_t)pi * slot_step * D];
+        for (int pi = 0; pi < n_parts; ++pi) acc += sm[pi][r] * *(const f32x4_t*)(po + (size_t)pi * slot_step * D);
         const int row = q_row0 + r;
         const int ti = row / G, head = kvh * G + (row - ti * G);
-        out[((size_t)(q_tok0 + ti) * n_heads + head) * D + d] = f32_to_bf16(acc);
+        uint2 w;
+        w.x = pack2(acc[0], acc[1]);
+        w.y = pack2(acc[2], acc[3]);
+        *(uint2*)(out + ((size_t)(q_tok0 + ti) * n_heads + head) * D + d) = w;
     }
 }
 
