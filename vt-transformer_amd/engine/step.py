@@ -70,8 +70,8 @@ TILE_STEP_US = {1: 2.1, 2: 2.45}
 # An item of the tiled kernel that is longer than TILE_CUT x the launch's balanced length (all items' steps shared
 # out over the slots) has its keys cut into ranges of about that length, each an item of its own, merged afterwards.
 # Measured with one and two row tiles and cuts at 0.7, 1, 1.4 and 2 (us, against no cut with the better of one and
-# two row tiles): a fresh 2,048-token portion with 28 query / 4 kv heads 74 (77), with 12 / 2 heads 50 (56), 4,096
-# tokens with 12 / 2 heads 104 (114); 2,048 tokens behind 2,048 earlier ones 148 (147), eight 1,024-token portions 102
+# two row tiles): a fresh 2,048-token portion with 28 query / 4 kv heads 66 (77), with 12 / 2 heads 42 (56), 4,096
+# tokens with 12 / 2 heads 96 (114); 2,048 tokens behind 2,048 earlier ones 148 (147), eight 1,024-token portions 102
 # (102), 64 / 8 heads 103 (103): no shorter cut helped anywhere, and cuts at 1 and below cost up to a fifth where the
 # items fill the GPU anyway.
 TILE_CUT = 1.4
