@@ -426,7 +426,7 @@ def test_attention_fp32_one_key_is_value_row_and_zero_query_is_mean():
 
 # ---------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("nh,kvh,d,page_size", [(4, 2, 16, 16), (5, 1, 48, 32), (28, 4, 128, 16)])
+@pytest.mark.parametrize("nh,kvh,d,page_size", [(4, 2, 16, 16), (5, 1, 48, 32), (28, 4, 128, 16), (64, 8, 128, 16)])
 def test_rope_store(dtype, nh, kvh, d, page_size):
     from vt_transformer_amd.parts.rotary import rotary_table
     o = ops()
