@@ -56,3 +56,16 @@ def test_generate_and_shell(model_folders):
     outs = [ln.replace("$ ", "") for ln in r.stdout.splitlines() if ln.replace("$ ", "")[:1].isdigit()]
     assert outs == [",".join(map(str, want))] * 2
     assert "Exiting shell..." in r.stdout
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU: asked for more it says so in one line and exits with 2, before it touches a GPU."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    for extra_env, args in (({}, ["--gpus", "2"]), ({"WORLD_SIZE": "2"}, [])):
+        env = dict(os.environ, **extra_env)
+        p = subprocess.run([sys.executable, os.path.join(root, "bench.py"), *args], capture_output=True, text=True, env=env,
+                           timeout=120)
+        assert p.returncode == 2
+        assert len(p.stdout.strip().splitlines()) == 1 and "one GPU" in p.stdout
