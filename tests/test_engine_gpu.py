@@ -19,6 +19,7 @@ DTYPES = ["float32", "bfloat16"]
 CONFIGS = ["A", "B", "W"]
 _plain_cache = {}
 _models = {}
+TOL_BF16 = 1.5e-2
 
 
 def get_model(folders, name, dtype):
@@ -410,6 +411,58 @@ def test_decode_graph_replays_match_eager(model_folders):
     b = graph.step(e3).clone()
     assert torch.equal(a, b)
     assert len(graph._graphs) >= 1
+
+
+def test_a_request_name_used_again_does_not_decode_against_the_old_requests_pages(model_folders):
+    """A captured decoding step's metadata is patched from one step to the next when the same requests go on.  A
+    request that ended and a new one admitted under its name are not the same request, even if the new one is just
+    as long as the old one was: its pages are others (the pool hands them out last-in-first-out)."""
+    from vt_transformer_amd.engine import StepEntry
+    cfg = "B"
+    model = get_model(model_folders, cfg, "bfloat16")
+    pc, pw = plain_model.read_folder(model_folders[cfg])
+    runner = runner_for(model, 256, max_requests=2)
+    runner.decode_graphs = True
+    first = random_requests(TINY[cfg]["vocab_size"], [41], seed=51)["r0"]
+    second = random_requests(TINY[cfg]["vocab_size"], [42], seed=52)["r0"]
+    assert runner.admit("r")
+    runner.step([StepEntry("r", first[:40], [])])
+    got1 = runner.step([StepEntry("r", first[40:41], [0])]).float().cpu()
+    runner.release("r")
+    assert runner.admit("r")
+    runner.step([StepEntry("r", second[:41], [])])
+    assert runner.cache.get("r").tables[0] != [0, 1, 2]         # (other pages than the first request had)
+    got2 = runner.step([StepEntry("r", second[41:42], [0])]).float().cpu()
+    assert len(runner._graphs) == 1
+    for toks, got in ((first, got1), (second, got2)):
+        ref = plain_model.forward(pc, pw, toks)[-1]
+        assert float((got[0].double() - ref).abs().max() / ref.abs().max()) < TOL_BF16
+
+
+def test_prompts_that_fit_alone_but_not_together_finish_with_their_own_tokens(model_folders):
+    """Four pages of four tokens, portions of four, two prompts of twelve: admitted together they would hold every
+    page half-way through.  Both finish, with the tokens each gets alone."""
+    from vt_transformer_amd.engine import Engine
+    from vt_transformer_amd.sampling import SamplingParams
+    cfg = "B"
+    prompts = list(random_requests(TINY[cfg]["vocab_size"], [12, 12], seed=53).values())
+    sp = [SamplingParams(temperature=0.8, max_tokens=3, ignore_eos=True, seed=3000 + i) for i in range(2)]
+    alone = []
+    for i, p in enumerate(prompts):
+        eng = Engine(model_folders[cfg], dtype="float32", num_pages=4, page_size=4, max_running_reqs=1, max_seq_len=16)
+        alone.append(eng.generate([p], [sp[i]])[0])
+    eng = Engine(model_folders[cfg], dtype="float32", num_pages=4, page_size=4, chunk_size=4, max_extend_tokens=8,
+                 max_running_reqs=4, max_seq_len=16)
+    steps = 0
+    for p, s in zip(prompts, sp):
+        eng.add_request(p, s)
+    while eng.has_work():
+        eng.step()
+        steps += 1
+        assert steps < 100, "the engine does not finish"
+    assert [eng.requests[i].output for i in range(2)] == alone
+    assert [eng.requests[i].finish_reason for i in range(2)] == ["max_tokens"] * 2
+    assert sum(eng.runner.cache.held_pages()) == 0
 
 
 def test_group_of_17_query_heads_is_not_replayed_and_right(tmp_path):

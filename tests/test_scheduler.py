@@ -174,20 +174,117 @@ def test_a_lone_request_that_outgrows_the_pool_ends_with_an_error():
     assert e.cache.held_pages() == [0]
 
 
-@pytest.mark.parametrize("seed", range(6))
+def _alone(n_prompt, max_tokens, token, **cfg):
+    e = FakeEngine(token=token, **cfg)
+    r = e.add("x", n_prompt, max_tokens=max_tokens)
+    e.run()
+    return r.output
+
+
+@pytest.mark.parametrize("shape", [dict(num_pages=4, page_size=4, chunk_size=4, max_extend_tokens=8, n=12),
+                                   dict(num_pages=64, page_size=16, chunk_size=256, max_extend_tokens=8192, n=600)])
+def test_two_prompts_that_each_fit_alone_but_not_together_both_finish(shape):
+    """Two prompts cut into portions must not end up holding every page half-way through with neither able to go
+    on (the reference simply does not run a batch that gets no pages and tries again for ever,
+    vt-transformer/core/vt_scheduler.cpp:112-117, 365-371)."""
+    shape = dict(shape)
+    n = shape.pop("n")
+    token = lambda r: 1 + (len(r.output) * 7 + len(r.prompt)) % 5
+    e = FakeEngine(token=token, **shape)
+    a = e.add("a", n, max_tokens=3)
+    b = e.add("b", n, max_tokens=3)
+    e.run(limit=200)
+    assert (a.finish_reason, b.finish_reason) == ("max_tokens", "max_tokens")
+    alone = _alone(n, 3, token, **shape)
+    assert a.output == alone and b.output == alone
+    assert all(p for p in e.plans), "a step with running requests planned nothing"
+    assert e.cache.held_pages() == [0]
+
+
+def test_requests_inside_their_prompts_that_hold_every_page_do_not_stall():
+    """The state that admission now avoids, made by hand: two requests half-way through their prompts hold all four
+    pages.  The youngest gives way, the oldest goes on, and both finish."""
+    e = FakeEngine(num_pages=4, page_size=4, chunk_size=4, max_extend_tokens=8)
+    a = e.add("a", 12, max_tokens=2)
+    b = e.add("b", 12, max_tokens=2)
+    for r in (a, b):
+        e.sched.waiting.remove(r)
+        e.cache.admit(r.uid)
+        assert e.cache.reserve([(r.uid, 8)])
+        e.cache.commit(r.uid, 8)
+        r.state, r.computed = RUNNING, 8
+        e.sched.running.append(r)
+    assert e.cache.available_pages() == [0]
+    plan = e.sched.schedule()
+    assert [(s.request.uid, s.start, s.n_tokens) for s in plan] == [("a", 8, 4)]
+    assert b.state == WAITING and b.preemptions == 1 and e.sched.waiting[0] is b
+    e.sched.update([], {})
+    e.run(limit=100)
+    assert (a.finish_reason, b.finish_reason) == ("max_tokens", "max_tokens")
+    assert len(a.output) == 2 and len(b.output) == 2
+
+
+def test_a_lone_request_inside_its_prompt_that_cannot_go_on_ends_with_an_error():
+    e = FakeEngine(num_pages=2, page_size=4, chunk_size=4, max_seq_len=100)
+    a = e.add("a", 8, max_tokens=2)
+    e.sched.waiting.remove(a)
+    e.cache.admit(a.uid)
+    # another holder (not the scheduler's) has taken a page: the request's last portion can never get one
+    e.cache.admit("other")
+    assert e.cache.reserve([("other", 4), (a.uid, 4)])
+    e.cache.commit(a.uid, 4)
+    a.state, a.computed = RUNNING, 4
+    e.sched.running.append(a)
+    assert e.sched.schedule() == []
+    assert a.finish_reason == "out_of_pages" and not e.sched.running
+    assert [r.reason for r in e.sched.update([], {})] == ["out_of_pages"]
+
+
+def test_a_portion_is_cut_to_the_pages_that_are_left():
+    e = FakeEngine(num_pages=6, page_size=4, chunk_size=6, max_extend_tokens=64)
+    a = e.add("a", 3, max_tokens=30)
+    e.step()                                     # a holds one page
+    b = e.add("b", 14, max_tokens=2)             # needs 4 pages: fits beside a's one and one page of head-room
+    e.step()
+    assert e.plans[1] == [("a", 3, 1, True), ("b", 0, 6, False)]
+    e.cache.admit("other")                       # somebody else takes two of the three free pages
+    assert e.cache.reserve([("other", 8)])
+    e.step()                                     # a: its 5th token takes the last page; b: the 2 slots of its page
+    assert e.plans[2] == [("a", 4, 1, True), ("b", 6, 2, False)]
+    e.step()                                     # no page for b: it waits while a decodes
+    assert e.plans[3] == [("a", 5, 1, True)]
+    e.cache.release("other")
+    e.run()
+    assert b.finish_reason == "max_tokens" and b.preemptions == 0
+
+
+@pytest.mark.parametrize("seed", range(50))
 def test_random_load_always_drains(seed):
     rng = random.Random(seed)
-    e = FakeEngine(num_pages=rng.randint(8, 30), page_size=rng.choice([2, 4, 16]), windows=(0, rng.choice([0, 6])),
-                   max_running_reqs=rng.randint(1, 6), max_extend_tokens=rng.randint(4, 40), chunk_size=rng.randint(2, 16),
-                   max_seq_len=64, token=lambda r: rng.choice([1, 2, 3, EOS]))
+    tight = seed % 2 == 1       # chunk sizes below the prompt lengths, pools below the sum of the prompts
+    page_size = rng.choice([1, 2, 4, 16])
+    if tight:
+        max_len = 64
+        num_pages = -(-rng.randint(40, 70) // page_size) + 1
+        chunk, budget = rng.randint(2, 8), rng.randint(4, 16)
+        prompt = lambda: rng.randint(12, 38)
+    else:
+        max_len = 64
+        num_pages = rng.randint(8, 30)
+        chunk, budget = rng.randint(2, 16), rng.randint(4, 40)
+        prompt = lambda: rng.randint(1, 40)
+    e = FakeEngine(num_pages=num_pages, page_size=page_size, windows=(0, rng.choice([0, 6])),
+                   max_running_reqs=rng.randint(1, 6), max_extend_tokens=budget, chunk_size=chunk,
+                   max_seq_len=max_len, token=lambda r: rng.choice([1, 2, 3, EOS]))
     reqs = []
     for step in range(300):
         if rng.random() < 0.3:
-            reqs.append(e.add(len(reqs), rng.randint(1, 40), max_tokens=rng.randint(1, 12),
+            reqs.append(e.add(len(reqs), prompt(), max_tokens=rng.randint(1, 12),
                               ignore_eos=rng.random() < 0.3))
         if rng.random() < 0.05 and reqs:
             e.sched.abort_request(rng.choice(reqs).uid)
         e.step()
+        assert e.plans[-1] or not e.sched.running, "requests are running and the step planned nothing"
     e.run()
     assert all(r.state == FINISHED for r in reqs)
     assert all(r.finish_reason in ("eos", "max_tokens", "max_seq_len", "abort", "too_long", "out_of_pages") for r in reqs)

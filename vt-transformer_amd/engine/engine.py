@@ -131,7 +131,12 @@ class Engine:
         if cur is None:
             plan = self.scheduler.schedule()
             if not plan:
-                return self.scheduler.update(plan, {})
+                results = self.scheduler.update(plan, {})
+                if not results and (self.scheduler.running or self.scheduler.waiting):
+                    raise RuntimeError(
+                        f"the scheduler has {len(self.scheduler.running)} running and {len(self.scheduler.waiting)} "
+                        f"waiting requests and nothing to run: no slot, page or token budget lets any of them move")
+                return results
             cur = self._launch(plan, None)
         if self.pipeline_decode:
             nxt = self._plan_ahead(cur[0])
@@ -192,9 +197,7 @@ class Engine:
             params = [params] * len(plist)
         uids = [self.add_request(p, sp) for p, sp in zip(plist, params)]
         while self.has_work():
-            results = self.step()
-            if not results and not self.scheduler.running and self.scheduler.waiting:
-                raise RuntimeError("the scheduler cannot place the waiting requests (pool too small?)")
+            self.step()         # (raises if requests are left and none can move)
         outs = [self.requests[u].output for u in uids]
         return outs[0:1] if single else outs
 

@@ -18,8 +18,12 @@ cannot get a page it simply does not run and is tried again for ever
 portions of prompts; a prompt is cut to the budget; and when a decoding
 request cannot get a page the youngest running request is preempted: it
 gives everything back, returns to the head of the waiting line and is later
-recomputed from its prompt and the tokens it has produced.  A request that
-could never fit is finished with an error instead of waiting for ever.
+recomputed from its prompt and the tokens it has produced.  The same happens
+when requests inside their prompts hold every page among them and nothing
+can move: a plan is never empty while requests are running.  A request is
+admitted only if all it holds so far fits beside what the running requests
+still need for their prompts.  A request that could never fit is finished
+with an error instead of waiting for ever.
 """
 from __future__ import annotations
 
@@ -171,7 +175,34 @@ class Scheduler:
 
     def schedule(self) -> List[Scheduled]:
         """Choose the step's portions.  Pages are not taken here: the step function reserves them, and this
-        choice is made so that it will succeed."""
+        choice is made so that it will succeed.
+
+        A plan is never empty while requests are running: if nothing can move (requests inside their prompts hold
+        every page among them and none is decoding), the youngest running request is preempted and the choice is
+        made again, until something moves or the last one, which cannot go on even alone, ends with an error."""
+        while True:
+            plan = self._plan_once()
+            if plan or not self.running:
+                return plan
+            victim = max(self.running, key=lambda r: r.arrival)
+            if len(self.running) == 1:
+                self._finish(victim, "out_of_pages")
+                self.finished_early.append(ReqResult(victim.uid, None, True, "out_of_pages"))
+            else:
+                self._preempt(victim)
+
+    def _free_tokens_for(self, r: Request, planned: List[Tuple[Request, int]]) -> int:
+        """How many more tokens of r fit into its last page and the pages that `planned` leaves free."""
+        ps = self.cache.page_size
+        need = self._need(planned)
+        free_pages = min((p.available - n for p, n in zip(self.cache.pools, need)), default=None)
+        if free_pages is None:
+            return self.config.max_seq_len
+        rp = self.cache.get(r.uid)
+        slack = (-rp.length) % ps       # room left in the page that holds its newest keys
+        return max(0, free_pages) * ps + slack
+
+    def _plan_once(self) -> List[Scheduled]:
         cfg = self.config
         budget = cfg.max_extend_tokens
         plan: List[Scheduled] = []
@@ -196,18 +227,23 @@ class Scheduler:
             planned.append((r, r.computed + 1))
         budget -= len(plan)
 
-        # 2. running requests still inside their prompt (or being recomputed), oldest first
+        # 2. running requests still inside their prompt (or being recomputed), oldest first; a portion is cut to
+        #    the pages that are left, and a request that gets none waits for decoding requests to free some
         for r in sorted((r for r in self.running if not r.decoding), key=lambda r: r.arrival):
             if budget <= 0:
                 break
             n = min(r.total_len - r.computed, cfg.chunk_size, budget)
-            if n <= 0 or not self._fits(planned + [(r, r.computed + n)]):
-                continue   # it waits for pages; decoding requests will free some or be preempted
+            if n > 0 and not self._fits(planned + [(r, r.computed + n)]):
+                n = min(n, self._free_tokens_for(r, planned))
+            if n <= 0:
+                continue
             plan.append(Scheduled(r, r.computed, n, r.computed + n == r.total_len))
             planned.append((r, r.computed + n))
             budget -= n
 
-        # 3. admit from the waiting line, in order, while a slot, budget and pages for a first portion are there
+        # 3. admit from the waiting line, in order, while a slot, budget and pages are there: pages for the whole
+        #    of what the request holds so far (prompt and produced tokens), beside what the running requests still
+        #    need to finish their prompts, so that requests admitted together can all reach decoding
         while self.waiting and budget > 0 and len(self.running) < cfg.max_running_reqs:
             r = self.waiting[0]
             limit = min(cfg.max_seq_len, self._capacity_tokens())
@@ -218,16 +254,18 @@ class Scheduler:
             if self.cache.slots.available == 0:
                 break
             n = min(r.total_len - r.computed, cfg.chunk_size, budget)
-            rp = self.cache.admit(r.uid)
+            self.cache.admit(r.uid)
             # head-room: one page per running request, so that admission does not starve decoding at once
             reserve_pages = len(self.running)
-            ok = self._fits(planned + [(r, n)]) and all(
-                p.available - need >= reserve_pages for p, need in zip(
-                    self.cache.pools, self._need(planned + [(r, n)])))
+            promised = [(q, max(new_len, q.total_len)) for q, new_len in planned]
+            promised += [(q, q.total_len) for q in self.running if all(q is not p for p, _ in planned)]
+            need = self._need(promised + [(r, r.total_len)])
+            ok = all(p.available - k >= reserve_pages for p, k in zip(self.cache.pools, need))
             if not ok:
                 self.cache.release(r.uid)
                 if not self.running and not plan:
-                    # nothing else holds pages and it still does not fit: cut the portion to what fits
+                    # nothing else holds pages and it still does not fit (layers with a window give pages back as
+                    # the prompt goes on): cut the portion to what fits
                     n_fit = min(n, self.cache.available_tokens())
                     if n_fit <= 0:
                         self.waiting.popleft()

@@ -347,7 +347,8 @@ class _DecodeGraph:
         self.meta: Optional[torch.Tensor] = None
         self.logits: Optional[torch.Tensor] = None
         # what the next step through this graph needs to patch the metadata instead of building it anew
-        self.rids = None            # the requests of the last step, in order
+        self.rps = None             # what the requests of the last step hold (RequestPages), in order: the very
+                                    # objects, since a request that ended and one admitted later may share a name
         self.h = None               # its host arrays
         self.flat = None            # its metadata as one int32 array
         self.table_lens = None      # per group and entry, the block-table entries already written
@@ -527,8 +528,9 @@ class ModelRunner:
         n = len(entries)
         b = next(x for x in GRAPH_BATCHES if x >= n)
         g = self._graphs.get(b)
-        rids = tuple(e.rid for e in entries)
-        if g is not None and g.rids == rids and self._advance_decode_meta(g, entries):
+        rps = [self.cache.get(e.rid) for e in entries]
+        if (g is not None and g.rps is not None and len(g.rps) == n and all(a is b for a, b in zip(g.rps, rps))
+                and self._advance_decode_meta(g, entries, rps)):
             self._feed_ids(g, ids_dev, n)
             g.graph.replay()        # the same requests as in the last step, one token further: the metadata was patched
             return g.wanted
@@ -554,7 +556,7 @@ class ModelRunner:
             self._feed_ids(g, ids_dev, n)
             g.graph.replay()
         # what the next step can patch instead of building anew: the host copy of the metadata and where its parts lie
-        g.rids, g.h, g.flat = rids, h, self._last_flat
+        g.rps, g.h, g.flat = rps, h, self._last_flat
         g.table_lens = [[len(self.cache.get(e.rid).tables[gi]) for e in entries] for gi in range(self.storage.n_groups)]
         g.wants = [tuple(e.want) for e in entries]
         if len(h["rows"]) == 0:
@@ -563,18 +565,17 @@ class ModelRunner:
             g.wanted = g.logits[:len(h["rows"])]     # the first entries in order: a view, no copy
         else:
             g.wanted = None
-            g.rids = None                            # wanted rows that are no plain prefix: no patching next time
+            g.rps = None                             # wanted rows that are no plain prefix: no patching next time
             return g.logits.index_select(0, torch.from_numpy(h["rows"].astype(np.int64)).to(self.rt.device))
         return g.wanted
 
-    def _advance_decode_meta(self, g: "_DecodeGraph", entries: Sequence[StepEntry]) -> bool:
+    def _advance_decode_meta(self, g: "_DecodeGraph", entries: Sequence[StepEntry], rps) -> bool:
         """The last step through this graph had the same requests in the same order, and each has since grown by
         exactly its one token: patch token ids, positions, decode chunks and the block-table entries of pages that
         were added, in the host copy of the metadata, and send it.  False if anything else changed (the caller then
         builds the metadata anew)."""
-        cache, h, flat = self.cache, g.h, g.flat
+        h, flat = g.h, g.flat
         n = len(entries)
-        rps = [cache.get(e.rid) for e in entries]
         pos0 = h["pos0"]
         for i, (e, rp) in enumerate(zip(entries, rps)):
             if rp.length != pos0[i] + 1 or len(e.tokens) != 1 or tuple(e.want) != g.wants[i] or rp.fresh:
