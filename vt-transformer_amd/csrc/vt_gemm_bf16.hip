@@ -27,6 +27,8 @@
 // order.  How k is split depends on the shape of W only, never on the number
 // of rows, so a token's result does not change with the batch around it.
 #include "vt_common.h"
+#include "vt_gemm_bf16.h"
+#include <mutex>
 
 VT_DEFINE_LAST_ERROR()
 
@@ -733,6 +735,49 @@ extern "C" int vt_linear_bf16(const void* x, const void* wp, const float* bias, 
     if (out_dtype == VT_F32) return linear_bf16<false, float>(x, (const bf16_t*)wp, bias, (float*)y, workspace, N, M, K, nullptr, 0.f, nullptr, stream);
     if (out_dtype == VT_BF16) return linear_bf16<false, bf16_t>(x, (const bf16_t*)wp, bias, (bf16_t*)y, workspace, N, M, K, nullptr, 0.f, nullptr, stream);
     return vt_fail("vt_linear_bf16: unknown out dtype %d", out_dtype);
+}
+
+// ---------------------------------------------------------------------------
+// The product without a workspace argument and without any allocation: the partial sums of a split k range go into
+// an array that the code object itself brings, one copy per GPU.
+// ---------------------------------------------------------------------------
+static __device__ __align__(256) float vt_linear_scratch[VT_LINEAR_NOALLOC_MAX_FLOATS];
+
+#define VT_MAX_DEVICES 64
+// Where this GPU's copy of the array lies.  In host code the array's name is only a handle for the runtime, not an
+// address that a kernel could use: the address is asked for once per device, with that device current.
+static int noalloc_scratch(float** out) {
+    static float* ptrs[VT_MAX_DEVICES] = {nullptr};
+    static std::mutex lock;
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return vt_fail("vt_linear_bf16_noalloc: hipGetDevice: %s", hipGetErrorString(e));
+    VT_REQUIRE(dev >= 0 && dev < VT_MAX_DEVICES, "vt_linear_bf16_noalloc: device %d is beyond the %d that are kept track of",
+               dev, VT_MAX_DEVICES);
+    std::lock_guard<std::mutex> guard(lock);
+    if (!ptrs[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(vt_linear_scratch));
+        if (e != hipSuccess || !p)
+            return vt_fail("vt_linear_bf16_noalloc: hipGetSymbolAddress on device %d: %s", dev, hipGetErrorString(e));
+        ptrs[dev] = (float*)p;
+    }
+    *out = ptrs[dev];
+    return 0;
+}
+
+extern "C" int vt_linear_bf16_noalloc(const void* x, const void* wp, const float* bias, void* y, int out_dtype,
+                                      int N, int M, int K, hipStream_t stream) {
+    VT_REQUIRE(N >= 0 && M > 0 && K > 0, "vt_linear_bf16_noalloc: bad sizes N=%d M=%d K=%d", N, M, K);
+    const long long need = vt_linear_bf16_workspace(N, M, K, 0);
+    VT_REQUIRE(need <= (long long)VT_LINEAR_NOALLOC_MAX_FLOATS,
+               "vt_linear_bf16_noalloc: x [%d, %d] with W [%d, %d] needs %lld floats for its partial sums, the built-in "
+               "array holds %d: use vt_linear_bf16 with a workspace", N, K, M, K, need, VT_LINEAR_NOALLOC_MAX_FLOATS);
+    float* scratch = nullptr;
+    if (need > 0 && noalloc_scratch(&scratch) != 0) return -1;
+    if (out_dtype == VT_F32) return linear_bf16<false, float>(x, (const bf16_t*)wp, bias, (float*)y, scratch, N, M, K, nullptr, 0.f, nullptr, stream);
+    if (out_dtype == VT_BF16) return linear_bf16<false, bf16_t>(x, (const bf16_t*)wp, bias, (bf16_t*)y, scratch, N, M, K, nullptr, 0.f, nullptr, stream);
+    return vt_fail("vt_linear_bf16_noalloc: unknown out dtype %d", out_dtype);
 }
 
 // The same with an RMSNorm in front (up to 16 tokens) and a residual addition behind (up to 64), each optional:
