@@ -70,8 +70,8 @@ def linear(x: torch.Tensor, w: torch.Tensor, b: Optional[torch.Tensor] = None) -
 def rotary_angles(positions: torch.Tensor, dims: int, base: float) -> torch.Tensor:
     """v1/tensortype/common.cpp:6-24: inv_freq[i/2] = 1/base^(i/dims) for even i; angle = position * inv_freq.
     [T, dims/2]"""
-    i = torch.arange(0, dims, 2, dtype=DT)
-    inv = 1.0 / torch.pow(torch.tensor(base, dtype=DT), i / dims)
+    i = torch.arange(0, dims, 2, dtype=DT, device=positions.device)
+    inv = 1.0 / torch.pow(torch.tensor(base, dtype=DT, device=positions.device), i / dims)
     return positions.to(DT)[:, None] * inv[None, :]
 
 
@@ -99,18 +99,22 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, window: int = 0
     kvh = k.shape[1]
     rep = nh // kvh
     out = torch.zeros_like(q)
-    idx = torch.arange(t)
-    allowed = idx[None, :] <= idx[:, None]
-    if window > 0:
-        allowed &= idx[None, :] > idx[:, None] - window
-    for h in range(nh):
-        kh, vh = k[:, h // rep, :], v[:, h // rep, :]
-        s = (q[:, h, :] @ kh.t()) / math.sqrt(d)
-        s = torch.where(allowed, s, torch.tensor(float("-inf"), dtype=s.dtype))
-        s = s - s.max(dim=-1, keepdim=True).values
-        p = torch.exp(s)
-        p = p / p.sum(dim=-1, keepdim=True)
-        out[:, h, :] = p @ vh
+    cols = torch.arange(t, device=q.device)
+    # (rows in blocks of 2,048 so that a long sequence's score matrix need not exist all at once; every row still
+    # sees the whole sequence)
+    for r0 in range(0, t, 2048):
+        rows = torch.arange(r0, min(t, r0 + 2048), device=q.device)
+        allowed = cols[None, :] <= rows[:, None]
+        if window > 0:
+            allowed &= cols[None, :] > rows[:, None] - window
+        for h in range(nh):
+            kh, vh = k[:, h // rep, :], v[:, h // rep, :]
+            s = (q[rows, h, :] @ kh.t()) / math.sqrt(d)
+            s = torch.where(allowed, s, torch.tensor(float("-inf"), dtype=s.dtype, device=s.device))
+            s = s - s.max(dim=-1, keepdim=True).values
+            p = torch.exp(s)
+            p = p / p.sum(dim=-1, keepdim=True)
+            out[rows, h, :] = p @ vh
     return out
 
 
@@ -135,9 +139,14 @@ def layer_window(cfg: dict, i: int) -> int:
     return int(cfg["sliding_window"]) if i >= first else 0
 
 
-def forward(cfg: dict, w: Dict[str, torch.Tensor], ids: List[int], first_position: int = 0) -> torch.Tensor:
+def forward(cfg: dict, w: Dict[str, torch.Tensor], ids: List[int], first_position: int = 0,
+            device: Optional[str] = None) -> torch.Tensor:
     """Logits [T, V] of a whole sequence, float64.
-    Order of v1/models/qwen2-7b/inference_fp16.dag:287-345 (layer) and :368-388 (outer program)."""
+    Order of v1/models/qwen2-7b/inference_fp16.dag:287-345 (layer) and :368-388 (outer program).
+    device: where torch does the arithmetic (None: the tensors' own, the CPU; sequences of many thousands of
+    tokens are given a GPU, still in float64 and with these same functions); the logits come back on the CPU."""
+    if device is not None:
+        w = {k: v.to(device) for k, v in w.items()}
     nh = cfg["num_attention_heads"]
     kvh = cfg.get("num_key_value_heads", nh)
     hidden = cfg["hidden_size"]
@@ -145,8 +154,9 @@ def forward(cfg: dict, w: Dict[str, torch.Tensor], ids: List[int], first_positio
     eps = cfg.get("rms_norm_eps", 1e-6)
     base = cfg.get("rope_theta", 1000000.0)
     t = len(ids)
-    pos = torch.arange(first_position, first_position + t)
-    x = w["model.embed_tokens.weight"][torch.tensor(ids, dtype=torch.long)]          # dag :372-375
+    dev = w["model.embed_tokens.weight"].device
+    pos = torch.arange(first_position, first_position + t, device=dev)
+    x = w["model.embed_tokens.weight"][torch.tensor(ids, dtype=torch.long, device=dev)]   # dag :372-375
     for i in range(cfg["num_hidden_layers"]):
         p = f"model.layers.{i}."
         a = rmsnorm(x, w[p + "input_layernorm.weight"], eps)                              # :290
@@ -162,7 +172,7 @@ def forward(cfg: dict, w: Dict[str, torch.Tensor], ids: List[int], first_positio
                        w[p + "mlp.down_proj.weight"])
     x = rmsnorm(x, w["model.norm.weight"], eps)                                           # :383
     head = w["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings", False) else w["lm_head.weight"]
-    return linear(x, head)                                                                # :384-388
+    return linear(x, head).cpu()                                                          # :384-388
 
 
 def greedy(cfg: dict, w: Dict[str, torch.Tensor], prompt: List[int], n_new: int) -> List[int]:

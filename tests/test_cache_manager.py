@@ -188,3 +188,40 @@ def test_slot_pool():
     with pytest.raises(CacheError):
         s.free(a)
     assert s.alloc() == 0
+
+
+def test_a_byte_budget_is_shared_by_the_groups_of_layers():
+    """The reference sizes its one pool as budget // (block size x bytes per token)
+    (vt-transformer/models/qwen3-0.6b/init.vt:109-113).  With groups of layers that have pages of their own, a token
+    takes a slot in every group, so the budget is divided by the bytes of one page of each group together."""
+    from types import SimpleNamespace
+
+    import pytest
+    import torch
+
+    from vt_transformer_amd.cache.storage import CacheStorage
+    from vt_transformer_amd.config.base import ScheduleEntry
+    from vt_transformer_amd.parts.base import CacheNeed, Runtime
+
+    def mixer(kv, d, window):
+        return SimpleNamespace(cache_need=lambda: CacheNeed(kv, d, window), state_need=lambda: None)
+
+    # three layers keep every key of 2 heads x 16; two keep a window of 8 keys of 1 head x 32
+    mixers = [mixer(2, 16, 0), mixer(1, 32, 8), mixer(2, 16, 0), mixer(1, 32, 8), mixer(2, 16, 0)]
+    model = SimpleNamespace(schedule=[ScheduleEntry(i) for i in range(5)],
+                            layers=[SimpleNamespace(mixer=m) for m in mixers], spec=SimpleNamespace(vocab_size=10))
+    rt = Runtime(torch.device("cpu"), torch.float32)
+    page = 4
+    per_page = 2 * 4 * page * (3 * 2 * 16 + 2 * 1 * 32)          # keys and values, float32
+    st = CacheStorage(rt, model, page, None, 4, 64, kv_bytes=10 * per_page + per_page // 2)
+    assert st.num_pages == 10 and st.kv_bytes == 10 * per_page
+    assert [p.num_pages for p in st.manager.pools] == [10, 10]
+    held = sum(t.numel() * t.element_size() for t in st.k + st.v)
+    assert held == st.kv_bytes <= 10 * per_page + per_page // 2
+    assert st.page_bytes == [2 * 4 * page * 3 * 2 * 16, 2 * 4 * page * 2 * 1 * 32]
+    with pytest.raises(ValueError, match="does not hold one page"):
+        CacheStorage(rt, model, page, None, 4, 64, kv_bytes=per_page - 1)
+    with pytest.raises(ValueError, match="not both"):
+        CacheStorage(rt, model, page, 64, 4, 64, kv_bytes=per_page)
+    # the same pool given in tokens
+    assert CacheStorage(rt, model, page, 40, 4, 64).num_pages == 10

@@ -30,9 +30,9 @@ def get_model(folders, name, dtype):
     return _models[key]
 
 
-def runner_for(model, pool_tokens, max_requests=8):
+def runner_for(model, pool_tokens, max_requests=8, page_size=16):
     from vt_transformer_amd.engine import make_runner
-    return make_runner(model, pool_tokens=pool_tokens, page_size=16, max_requests=max_requests,
+    return make_runner(model, pool_tokens=pool_tokens, page_size=page_size, max_requests=max_requests,
                        max_seq_len=min(model.spec.max_positions, max(pool_tokens, 16)))
 
 
@@ -106,6 +106,66 @@ def test_mixed_batches_with_page_reuse(model_folders, cfg, dtype):
     worst = check_against_plain(model_folders[cfg], reqs, steps, got, dtype, _plain_cache)
     report(f"mixed {cfg} {dtype} pool={pool}", worst)
     assert sum(runner.cache.held_pages()) == 0
+
+
+@pytest.mark.parametrize("page_size", [1, 2, 4])
+@pytest.mark.parametrize("cfg", ["B", "W"])
+def test_small_pages_in_float32(model_folders, cfg, page_size):
+    """Pages of 4 tokens (the workload of the second tiny configuration), of 2 and of 1 (the reference's default,
+    vt-transformer/core/vt_scheduler.hpp:33; ids 0, 2 with pages of two, vt-transformer/test/vt_cache_test.cpp:108-116):
+    all four ways of cutting the work in float32, whose attention kernel takes any page size."""
+    dtype = "float32"
+    model = get_model(model_folders, cfg, dtype)
+    vocab = TINY[cfg]["vocab_size"]
+    reqs = random_requests(vocab, [5, 13, 70], seed=71)
+    steps = trace_alone(reqs, {r: [(0, len(t))] for r, t in reqs.items()})
+    worst = check_against_plain(model_folders[cfg], reqs, steps, run_in_process(runner_for(model, 192, page_size=page_size), steps),
+                                dtype, _plain_cache)
+    reqs = random_requests(vocab, [40, 97], seed=72)
+    steps = trace_alone(reqs, {r: [(0, len(t) - 32)] + [(i, i + 1) for i in range(len(t) - 32, len(t))] for r, t in reqs.items()})
+    worst = max(worst, check_against_plain(model_folders[cfg], reqs, steps,
+                                           run_in_process(runner_for(model, 128, page_size=page_size), steps), dtype, _plain_cache))
+    reqs = random_requests(vocab, [61, 47], seed=73)
+    sizes = {"r0": [7, 2, 5, 3, 2, 16, 2, 9], "r1": [15, 1, 16, 2, 13]}
+    steps = trace_alone(reqs, {r: cut(t, sizes[r]) for r, t in reqs.items()})
+    worst = max(worst, check_against_plain(model_folders[cfg], reqs, steps,
+                                           run_in_process(runner_for(model, 128, page_size=page_size), steps), dtype, _plain_cache))
+    reqs = random_requests(vocab, [31, 16, 7, 1, 50, 33, 20, 45], seed=74)
+    portions = {}
+    for i, (r, t) in enumerate(reqs.items()):
+        n_head = max(0, len(t) - 9)
+        portions[r] = (cut(t[:n_head], [8, 3, 2] if i % 2 == 0 else [5, 11]) if n_head else []) + \
+            [(j, j + 1) for j in range(n_head, len(t))]
+    steps = trace_mixed(reqs, portions, max_live=4, seed=75)
+    pool = max_live_tokens(steps, round_to=max(page_size, 4))       # as few pages as the trace can do with
+    runner = runner_for(model, pool, max_requests=4, page_size=page_size)
+    worst = max(worst, check_against_plain(model_folders[cfg], reqs, steps, run_in_process(runner, steps), dtype, _plain_cache))
+    assert sum(runner.cache.held_pages()) == 0
+    report(f"page size {page_size} {cfg} {dtype}", worst)
+
+
+def test_what_bfloat16_kernels_refuse_is_said_when_the_model_or_engine_is_built(model_folders, tmp_path):
+    """Pages that are no multiple of 16 tokens and head sizes that are no multiple of 16: refused in bfloat16 before
+    anything runs (and before weights are read), taken in float32."""
+    from vt_transformer_amd.config import config_from_dict
+    from vt_transformer_amd.engine import Engine, build_model, make_runner
+    from vt_transformer_amd.weights import write_random_model
+    (tmp_path / "cfg_only").mkdir()
+    config_from_dict(dict(TINY["A"])).save(str(tmp_path / "cfg_only"))          # (no tensors: they are never asked for)
+    with pytest.raises(ValueError, match="page size 4.*multiple of 16"):
+        Engine(str(tmp_path / "cfg_only"), dtype="bfloat16", page_size=4)
+    with pytest.raises(ValueError, match="page size 24"):
+        make_runner(get_model(model_folders, "A", "bfloat16"), pool_tokens=96, page_size=24)
+    odd = config_from_dict(dict(TINY["A"], head_dim=24, num_attention_heads=2, num_key_value_heads=1))
+    with pytest.raises(ValueError, match="head size 24"):
+        build_model(odd, "bfloat16")
+    # float32 takes both: pages of 24 tokens, heads of 24
+    folder = write_random_model(odd, str(tmp_path / "odd"), seed=3)
+    reqs = random_requests(TINY["A"]["vocab_size"], [50], seed=76)
+    steps = trace_alone(reqs, {r: cut(t, [20, 1, 1, 11, 2]) for r, t in reqs.items()})
+    from vt_transformer_amd.engine import load_model
+    runner = runner_for(load_model(folder, "float32"), 96, page_size=24)
+    check_against_plain(folder, reqs, steps, run_in_process(runner, steps), "float32", {})
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -188,16 +248,37 @@ def test_trace_run_program(model_folders, dtype, tmp_path):
     report(f"trace_run decode {cfg} {dtype}", worst)
 
 
-def test_random_weights_on_device_match_written_folder(model_folders):
-    """random_model draws on the device; a written folder draws on the host.  Both must be proper models of the
-    configuration (their values differ: the generators do)."""
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_random_weights_drawn_on_the_device_are_the_written_folders_model(dtype, tmp_path):
+    """`random_model(config, seed)` draws its tensors on the device, the only way a model of 145 GB can be made;
+    `write_random_model(config, folder, seed)` draws them on the host.  Both use one counter-based generator, so
+    they are the same model: the device's one, under all four ways of cutting the work, against the plain
+    implementation reading the written folder."""
     from vt_transformer_amd.config import config_from_dict
-    from vt_transformer_amd.engine import StepEntry, random_model
-    model = random_model(config_from_dict(dict(TINY["A"])), seed=3, dtype="bfloat16")
-    r = runner_for(model, 64)
-    r.admit(0)
-    logits = r.step([StepEntry(0, [1, 2, 3, 4, 5], [4])])
-    assert logits.shape == (1, TINY["A"]["vocab_size"]) and bool(torch.isfinite(logits).all())
+    from vt_transformer_amd.engine import random_model
+    from vt_transformer_amd.weights import write_random_model
+    cfg = "B"
+    folder = write_random_model(config_from_dict(dict(TINY[cfg])), str(tmp_path / "m"), seed=77)
+    model = random_model(config_from_dict(dict(TINY[cfg])), seed=77, dtype=dtype)
+    vocab = TINY[cfg]["vocab_size"]
+    cache = {}
+    # whole; last 32 one by one; portions of changing size; mixed with page reuse
+    reqs = random_requests(vocab, [9, 70], seed=61)
+    steps = trace_alone(reqs, {r: [(0, len(t))] for r, t in reqs.items()})
+    worst = check_against_plain(folder, reqs, steps, run_in_process(runner_for(model, 128), steps), dtype, cache)
+    reqs = random_requests(vocab, [50], seed=62)
+    steps = trace_alone(reqs, {r: [(0, len(t) - 32)] + [(i, i + 1) for i in range(len(t) - 32, len(t))] for r, t in reqs.items()})
+    worst = max(worst, check_against_plain(folder, reqs, steps, run_in_process(runner_for(model, 64), steps), dtype, cache))
+    reqs = random_requests(vocab, [61], seed=63)
+    steps = trace_alone(reqs, {r: cut(t, [7, 2, 5, 3, 2, 16, 2, 9]) for r, t in reqs.items()})
+    worst = max(worst, check_against_plain(folder, reqs, steps, run_in_process(runner_for(model, 64), steps), dtype, cache))
+    reqs = random_requests(vocab, [31, 16, 7, 50, 33, 20], seed=64)
+    portions = {r: cut(t[:max(0, len(t) - 6)], [8, 3, 2]) + [(j, j + 1) for j in range(max(0, len(t) - 6), len(t))]
+                for r, t in reqs.items()}
+    steps = trace_mixed(reqs, portions, max_live=4, seed=65)
+    runner = runner_for(model, max_live_tokens(steps), max_requests=4)
+    worst = max(worst, check_against_plain(folder, reqs, steps, run_in_process(runner, steps), dtype, cache))
+    report(f"random_model {cfg} {dtype}", worst)
 
 
 # ---------------------------------------------------------------------------
@@ -221,7 +302,7 @@ def test_greedy_generation_through_entry_point(model_folders):
         logits = plain_model.forward(pc, pw, p + g)
         for i, tok in enumerate(g):
             row = logits[len(p) - 1 + i]
-            assert float(row.max() - row[tok]) <= 3e-2 * float(row.abs().max())
+            assert float(row.max() - row[tok]) <= TOL_BF16 * float(row.abs().max())
 
 
 def test_chunked_prompts_mixed_with_decoding_and_temperature(model_folders):
@@ -480,7 +561,7 @@ def test_group_of_17_query_heads_is_not_replayed_and_right(tmp_path):
     cfg, w = plain_model.read_folder(folder)
     toks = random_requests(d["vocab_size"], [40], seed=3)["r0"]
     ref = plain_model.forward(cfg, w, toks)
-    for dtype, tol in (("float32", 2e-5), ("bfloat16", 3e-2)):
+    for dtype, tol in (("float32", 2e-5), ("bfloat16", TOL_BF16)):
         runner = runner_for(load_model(folder, dtype), 128)
         runner.decode_graphs = True
         assert not runner._replayable
@@ -516,21 +597,23 @@ def test_single_weight_copy_gives_the_same_logits(model_folders):
     cfg, w = plain_model.read_folder(model_folders["W"])
     ref = plain_model.forward(cfg, w, toks[:460])
     rows = list(range(150)) + list(range(150, 450, 3)) + list(range(450, 460))
-    assert float((logits[1].double() - ref[rows]).abs().max() / ref.abs().max()) < 3e-2
+    assert float((logits[1].double() - ref[rows]).abs().max() / ref.abs().max()) < TOL_BF16
 
 
 def test_library_algorithm_search_keeps_results(model_folders):
-    """With the GEMM library's algorithm search on, a long portion gives the same logits to rounding."""
+    """With the GEMM library's algorithm search on, a long portion gives the plain implementation's logits, as
+    without it."""
     from vt_transformer_amd.engine import Engine, StepEntry
     toks = random_requests(TINY["B"]["vocab_size"], [150], seed=30)["r0"]
-    logits = []
+    pc, pw = plain_model.read_folder(model_folders["B"])
+    ref = plain_model.forward(pc, pw, toks)[[149, 70]]
     for tune in (False, True):
         eng = Engine(model_folders["B"], dtype="bfloat16", num_pages=32, max_running_reqs=2, max_seq_len=256,
                      chunk_size=128, tune_gemm=tune)
         eng.runner.admit("x")
-        logits.append(eng.runner.step([StepEntry("x", toks, [149])]).float().cpu())
+        got = eng.runner.step([StepEntry("x", toks, [149, 70])]).float().cpu().double()
         assert sum(eng.runner.cache.held_pages()) == 10
-    assert float((logits[0] - logits[1]).abs().max() / logits[0].abs().max()) < 2e-2
+        assert float((got - ref).abs().max() / ref.abs().max()) < TOL_BF16, tune
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -544,7 +627,7 @@ def test_a_long_prompt_whole_and_in_two_portions(model_folders, dtype):
     rows = list(range(0, 1800, 37)) + [1799]
     ref = plain_model.forward(pc, pw, toks)[rows]
     model = load_model(model_folders[cfg], dtype)
-    tol = 3e-5 if dtype == "float32" else 4e-2
+    tol = 3e-5 if dtype == "float32" else TOL_BF16
     for cuts in ([(0, 1800)], [(0, 1000), (1000, 1800)]):
         r = runner_for(model, 1856, max_requests=2)
         r.admit("x")
@@ -552,7 +635,7 @@ def test_a_long_prompt_whole_and_in_two_portions(model_folders, dtype):
         err = float((got.double() - ref).abs().max() / ref.abs().max())
         assert err < tol, (cuts, err)
     # (the planner does cut this shape: three kv heads, one query head each, head size 32)
-    from vt_transformer_amd.engine.step import plan_tile_items
+    from vt_transformer_amd.parts.attention_plan import plan_tile_items
     for pos0, n in ((0, 1800), (1000, 800)):
         _, _, citems, n_parts = plan_tile_items(np.array([0, n], np.int32), np.array([pos0], np.int32), 1, 0, 3,
                                                 np.arange(1), head_dim=32)

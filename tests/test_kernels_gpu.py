@@ -319,10 +319,10 @@ def attention_case(dtype, nh, kvh, d, page_size, window, entries, seed, spike=Fa
         o.attention_f32(q, kp.to(DEV), vp.to(DEV), positions.to(DEV), tok_entry.to(DEV), bt.to(DEV), out, nh, kvh, d,
                         window, scale)
     else:
-        from vt_transformer_amd.engine.step import plan_attention_items
+        from vt_transformer_amd.parts.attention_plan import plan_attention_items
         start = np.cumsum([0] + [n for _, n in entries]).astype(np.int32)
         pos0 = np.array([c for c, _ in entries], dtype=np.int32)
-        from vt_transformer_amd.engine.step import plan_tile_items
+        from vt_transformer_amd.parts.attention_plan import plan_tile_items
         first = None
         kpd, vpd, btd = kp.to(DEV), vp.to(DEV), bt.to(DEV)
         # 16-row items with keys unsplit and split, one and two row tiles; then the LDS-tiled kernel on all entries
@@ -674,3 +674,16 @@ def test_stream_read_reads_every_word_once(nbytes, blocks):
     assert got == np.bitwise_xor.reduce(host.view(np.uint32))
     with pytest.raises(o.KernelError):
         o.stream_read(buf.view(torch.int16)[:4], sums, blocks)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n,first", [(1, 0), (1000, 0), (70001, 12345), (3 * 257 * 129, 2 ** 33 + 5)])
+def test_random_normal_kernel_makes_the_hosts_bits(dtype, n, first):
+    """The device's counter-based generator against its numpy twin: equal to the bit, for matrices (mean 0) and
+    gains (mean 1), at an offset beyond 32 bits too."""
+    from vt_transformer_amd.weights.random_init import counter_normal, normal_scale
+    for key, mean in ((0x0123456789ABCDEF, 0.0), (2 ** 64 - 3, 1.0)):
+        out = torch.empty(n, dtype=dtype, device=DEV)
+        ops().random_normal(out, key, normal_scale(0.02), mean, first=first)
+        want = torch.from_numpy(counter_normal(key, first, n, 0.02, mean)).to(dtype)
+        assert torch.equal(out.cpu(), want), (key, mean)

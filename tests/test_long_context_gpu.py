@@ -1,0 +1,127 @@
+"""Contexts of many thousands of tokens, checked: 8,192 (the context that the bench times, four portions of 2,048
+and then token by token) and beyond 20,000 (block tables of more than a thousand entries, decoding with every
+entry's keys cut into sixteen ranges, 2,048-token portions behind tens of thousands of cached keys), in float32 and
+bfloat16, against the plain implementation run in float64 on the GPU.
+
+The reference stops at 4,096 (MAX_CONTEXT, v1/models/qwen2-7b/inference_fp16.dag:14; its softmax kernel takes
+fewer than 8,192 keys, v1/tensortype/hip_kernels/softmax.cpp:111).
+
+With N(0, 0.02) weights the scores of a small model are nearly equal, every key gets 1/T of the weight, and a block
+of keys that went missing or was read from the wrong page would change the result by less than bfloat16 rounds
+away.  The query and key projections are therefore scaled up so that scores spread over several units: each row's
+weight then sits on a few keys that lie anywhere in the context."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import plain_model
+from replay_helpers import random_requests
+
+pytestmark = pytest.mark.gpu
+
+LONG = dict(architectures=["Qwen2ForCausalLM"], model_type="qwen2", vocab_size=320, hidden_size=128,
+            intermediate_size=256, num_hidden_layers=2, num_attention_heads=4, num_key_value_heads=2, head_dim=128,
+            rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=32768,
+            hidden_act="silu", use_sliding_window=False, torch_dtype="bfloat16")
+QK_SCALE = 6.0
+# about twice the worst error seen (relative to a row's largest logit): 1.1e-6 in float32, 7.3e-3 in bfloat16
+TOL = {"float32": 3e-6, "bfloat16": 1.5e-2}
+
+
+@pytest.fixture(scope="module")
+def long_folder(tmp_path_factory):
+    from vt_transformer_amd.config import config_from_dict
+    from vt_transformer_amd.weights.random_init import declared_tensors, random_tensor
+    from vt_transformer_amd.weights.safetensors_io import write_safetensors
+    cfg = config_from_dict(dict(LONG))
+    folder = str(tmp_path_factory.mktemp("long") / "m")
+    os.makedirs(folder)
+    cfg.save(folder)
+
+    def tensors():
+        for name, decl in declared_tensors(cfg).items():
+            if decl.optional:
+                continue
+            t = random_tensor(name, decl, 11, torch.device("cpu"), torch.bfloat16)
+            if "q_proj" in name or "k_proj" in name:
+                t = (t.float() * QK_SCALE).to(torch.bfloat16)
+            yield name, t
+    write_safetensors(os.path.join(folder, "model.safetensors"), tensors(), metadata={"format": "pt"})
+    return folder
+
+
+_ref = {}
+
+
+def reference(folder, toks):
+    key = (folder, len(toks), toks[0], toks[-1])
+    if key not in _ref:
+        cfg, w = plain_model.read_folder(folder)
+        _ref[key] = plain_model.forward(cfg, w, toks, device="cuda").numpy()
+    return _ref[key]
+
+
+def test_the_long_model_spreads_its_weight_over_far_keys(long_folder):
+    """What makes the comparisons below mean something: in the plain model the last row's logits change by far more
+    than the tolerance when 64 tokens in the middle of its context are replaced by others (positions stay: what
+    changes is only what the later rows read from those keys and values)."""
+    cfg, w = plain_model.read_folder(long_folder)
+    toks = random_requests(LONG["vocab_size"], [6000], seed=5)["r0"]
+    other = list(toks)
+    other[3000:3064] = [(t + 1) % LONG["vocab_size"] for t in toks[3000:3064]]
+    full = plain_model.forward(cfg, w, toks, device="cuda")[-1]
+    changed = plain_model.forward(cfg, w, other, device="cuda")[-1]
+    effect = float((full - changed).abs().max() / full.abs().max())
+    print(f"effect of 64 far tokens among 6,000 on the last row: {effect:.3e}")
+    assert effect > 2.5 * TOL["bfloat16"], effect
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("n_long", [8192, 20480])
+def test_long_context_in_portions_then_token_by_token_beside_another_prompt(long_folder, dtype, n_long):
+    from vt_transformer_amd.engine import StepEntry, load_model, make_runner
+    vocab = LONG["vocab_size"]
+    a = random_requests(vocab, [n_long + 32], seed=n_long)["r0"]
+    b = random_requests(vocab, [2048 + 6], seed=n_long + 1)["r0"]
+    ref_a, ref_b = reference(long_folder, a), reference(long_folder, b)
+    model = load_model(long_folder, dtype)
+    runner = make_runner(model, pool_tokens=n_long + 64 + 2112, page_size=16, max_requests=4, max_seq_len=32768)
+    runner.decode_graphs = True
+    worst = [0.0]
+
+    def check(logits, rows):
+        got = logits.float().cpu().numpy().astype(np.float64)
+        assert np.isfinite(got).all()
+        for g, (name, ref, pos) in zip(got, rows):
+            err = float(np.abs(g - ref[pos]).max() / np.abs(ref[pos]).max())
+            assert err < TOL[dtype], f"request {name} position {pos}: error {err:.3e}"
+            worst[0] = max(worst[0], err)
+
+    assert runner.admit("a") and runner.admit("b")
+    sample = [0, 1, 777, 1023, 1024, 2047]
+    for p0 in range(0, n_long, 2048):
+        logits = runner.step([StepEntry("a", a[p0:p0 + 2048], sample)])
+        check(logits, [("a", ref_a, p0 + i) for i in sample])
+    for i in range(n_long, n_long + 32):
+        entries, rows = [StepEntry("a", a[i:i + 1], [0])], [("a", ref_a, i)]
+        j = i - n_long - 10
+        if j == 0:        # a decoded token of the long request beside a whole 2,048-token portion of another one
+            entries.append(StepEntry("b", b[:2048], [0, 2047]))
+            rows += [("b", ref_b, 0), ("b", ref_b, 2047)]
+        elif 0 < j <= 6:  # ... and then the two decode side by side, 20,000 keys beside 2,000
+            entries.insert(0, StepEntry("b", b[2047 + j:2048 + j], [0]))
+            rows.insert(0, ("b", ref_b, 2047 + j))
+        check(runner.step(entries), rows)
+    assert len(runner.cache.get("a").tables[0]) == (n_long + 32 + 15) // 16
+    if dtype == "bfloat16":
+        assert runner._graphs, "decoding did not go through captured steps"
+    runner.release("a"); runner.release("b")
+    assert sum(runner.cache.held_pages()) == 0
+    print(f"long context {n_long} {dtype}: worst relative error {worst[0]:.3e}")
+    folder = os.environ.get("VT_TEST_REPORT_DIR")
+    if folder:
+        os.makedirs(folder, exist_ok=True)
+        with open(os.path.join(folder, "engine_errors.txt"), "a") as f:
+            f.write(f"long context {n_long} {dtype}: worst relative error {worst[0]:.3e}\n")

@@ -200,7 +200,7 @@ def test_run_order_is_data(dtype):
     for a, b in [(0, 17), (17, 18), (18, 41)]:
         got.append(runner.step([StepEntry("r", ids[a:b], list(range(b - a)))]).cpu())
     ref = plain_scheduled(dict(TINY_A), {n: t.double() for n, t in w.items()}, ids, schedule)
-    assert rel(torch.cat(got), ref) < (2e-5 if dtype == "float32" else 3e-2)
+    assert rel(torch.cat(got), ref) < (2e-5 if dtype == "float32" else 1.5e-2)
 
 
 # ---------------------------------------------------------------------------

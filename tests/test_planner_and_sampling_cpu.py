@@ -2,7 +2,7 @@
 import numpy as np
 import pytest
 
-from vt_transformer_amd.engine.step import decode_chunk, plan_attention_items, plan_tile_items, split_entries
+from vt_transformer_amd.parts.attention_plan import decode_chunk, plan_attention_items, plan_tile_items, split_entries
 from vt_transformer_amd.sampling import SamplingParams, request_seed, uniform
 
 
@@ -103,16 +103,29 @@ def test_tile_items_cover_the_long_entries(group, window, rt, split):
 
 
 def test_decode_chunk():
-    from vt_transformer_amd.engine.step import decode_bucket
-    from vt_transformer_amd.parts.attention import decode_bucket as part_bucket
+    from vt_transformer_amd.parts.attention_plan import decode_parts_max
     assert decode_chunk(np.array([1]), 16) == 64
     c = decode_chunk(np.array([8192]), 16, n_kv=4)             # one entry: cut into as many items as allowed
     assert c % 64 == 0 and -(-8192 // c) <= 16
     assert decode_chunk(np.full(256, 1024), 16, n_kv=4) == 1024  # many entries: one item each
     c = decode_chunk(np.full(8, 1040), 16, n_kv=4)
     assert c % 64 == 0 and -(-1040 // c) * 8 * 4 >= 64
-    assert [decode_bucket(n) for n in (1, 2, 3, 4, 7, 8, 64, 1000)] == [0, 1, 1, 2, 2, 3, 6, 7]
-    assert all(decode_bucket(n) == part_bucket(n) for n in range(1, 300))
+    assert [decode_parts_max(n) for n in (1, 64, 65, 1000, 1024, 100000)] == [1, 1, 2, 16, 16, 16]
+
+
+def test_the_step_function_knows_no_kernel():
+    """The step function builds tokens, positions, entries, slots and block tables; what a mixer's kernels need
+    beyond that is the mixer's to plan (prepare_step)."""
+    import ast
+    import os
+    import vt_transformer_amd.engine.step as step
+    tree = ast.parse(open(step.__file__).read())
+    imported = set()
+    for node in ast.walk(tree):
+        if isinstance(node, ast.ImportFrom) and node.module:
+            imported.add(node.module)
+    assert not any("kernels" in m or "attention" in m for m in imported), imported
+    assert os.path.basename(step.__file__) == "step.py"
 
 
 def test_uniform_numbers_depend_only_on_seed_and_counter():

@@ -52,7 +52,8 @@ def check_configuration(cfg, seed, tmp_path):
     n = int(rs.randint(70, 200))
     toks = rs.randint(0, cfg["vocab_size"], size=n).tolist()
     ref = plain_model.forward(pcfg, w, toks)
-    for dtype, tol in (("float32", 3e-5), ("bfloat16", 4e-2)):
+    worst = {}
+    for dtype, tol in (("float32", 3e-5), ("bfloat16", 1.5e-2)):
         model = load_model(folder, dtype)
         for mode in ("whole", "cut", "decode", "graph"):
             runner = make_runner(model, pool_tokens=-(-n // 16) * 16 + 32, page_size=16, max_requests=2, max_seq_len=512)
@@ -71,6 +72,7 @@ def check_configuration(cfg, seed, tmp_path):
             got = torch.cat([runner.step([StepEntry("r", toks[a:b], list(range(b - a)))]).float().cpu() for a, b in cuts])
             err = float((got.double() - ref).abs().max() / ref.abs().max())
             assert err < tol, (cfg, dtype, mode, err)
+            worst[dtype] = max(worst.get(dtype, 0.), err)
         # several requests at a time, portions of some beside decoded tokens of others, pages used again
         reqs = random_requests(cfg["vocab_size"], [int(x) for x in rs.randint(1, 70, size=7)], seed=seed)
         portions = {}
@@ -81,8 +83,9 @@ def check_configuration(cfg, seed, tmp_path):
         steps = trace_mixed(reqs, portions, max_live=4, seed=seed)
         runner = make_runner(model, pool_tokens=max_live_tokens(steps), page_size=16, max_requests=4, max_seq_len=512)
         runner.decode_graphs = True
-        check_against_plain(folder, reqs, steps, run_in_process(runner, steps), dtype)
+        worst[dtype] = max(worst[dtype], check_against_plain(folder, reqs, steps, run_in_process(runner, steps), dtype))
         assert sum(runner.cache.held_pages()) == 0
+    print(f"random configuration {seed}: worst relative error {worst}")
 
 
 @pytest.mark.parametrize("name,hidden,heads,kv,inter", [("7B", 3584, 28, 4, 18944), ("1.5B", 1536, 12, 2, 8960),
@@ -106,7 +109,7 @@ def test_real_layer_sizes(name, hidden, heads, kv, inter, tmp_path):
     toks = np.random.RandomState(0).randint(0, 4099, size=n).tolist()
     ref = plain_model.forward(pcfg, w, toks)
     scale = ref.abs().max()
-    for dtype, tol in (("bfloat16", 4e-2), ("float32", 3e-5)):
+    for dtype, tol in (("bfloat16", 2e-2), ("float32", 3e-5)):
         model = load_model(folder, dtype)
         for mode in ("whole", "cut", "decode", "graph", "batch"):
             runner = make_runner(model, pool_tokens=10240, page_size=16, max_requests=48, max_seq_len=512)
@@ -130,4 +133,48 @@ def test_real_layer_sizes(name, hidden, heads, kv, inter, tmp_path):
                 got = torch.cat([runner.step([StepEntry("r", toks[a:b], list(range(b - a)))]).float().cpu() for a, b in cuts])
                 err = float((got.double() - ref).abs().max() / scale)
             assert err < tol, (name, dtype, mode, err)
+            print(f"layer sizes {name} {dtype} {mode}: relative error {err:.3e}")
         del model
+
+
+def test_96_requests_decoding_side_by_side_at_7b_layer_sizes(tmp_path):
+    """More decoding requests than the few-row kernels and the captured steps take (64): the step is launched kernel
+    by kernel and its products of 65 to 255 rows go to the GEMM library (the down projection to the packed kernel).
+    96 requests with prompts of their own, of different lengths, decode eight tokens side by side; every row against
+    the plain implementation (in float64 on the GPU: 96 sequences at these sizes take the CPU minutes)."""
+    from vt_transformer_amd.config import config_from_dict
+    from vt_transformer_amd.engine import StepEntry, load_model, make_runner
+    from vt_transformer_amd.weights import write_random_model
+    cfg = dict(architectures=["Qwen2ForCausalLM"], model_type="qwen2", vocab_size=4099, hidden_size=3584,
+               intermediate_size=18944, num_hidden_layers=2, num_attention_heads=28, num_key_value_heads=4, head_dim=128,
+               rope_theta=1e6, rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=8192,
+               hidden_act="silu", use_sliding_window=False, torch_dtype="bfloat16")
+    folder = str(tmp_path / "m")
+    write_random_model(config_from_dict(cfg), folder, seed=2)
+    pcfg, w = plain_model.read_folder(folder)
+    w = {k: v.to("cuda") for k, v in w.items()}
+    rs = np.random.RandomState(1)
+    n_req, n_dec = 96, 8
+    reqs = [rs.randint(0, 4099, size=int(rs.randint(20, 120)) + n_dec).tolist() for _ in range(n_req)]
+    refs = [plain_model.forward(pcfg, w, t)[-n_dec:] for t in reqs]            # [n_dec, vocab] each
+    del w
+    torch.cuda.empty_cache()
+    for dtype, tol in (("bfloat16", 2e-2), ("float32", 3e-5)):
+        model = load_model(folder, dtype)
+        runner = make_runner(model, pool_tokens=n_req * 144, page_size=16, max_requests=n_req, max_seq_len=512)
+        runner.decode_graphs = True
+        for i, t in enumerate(reqs):
+            runner.admit(i)
+        # the prompts in steps of 24 requests, then all 96 decode together
+        for i0 in range(0, n_req, 24):
+            runner.step([StepEntry(i, reqs[i][:-n_dec], []) for i in range(i0, i0 + 24)])
+        worst = 0.0
+        for j in range(n_dec):
+            got = runner.step([StepEntry(i, [reqs[i][len(reqs[i]) - n_dec + j]], [0]) for i in range(n_req)]).float().cpu().double()
+            for i in range(n_req):
+                err = float((got[i] - refs[i][j]).abs().max() / refs[i][j].abs().max())
+                assert err < tol, (dtype, "request", i, "token", j, err)
+                worst = max(worst, err)
+        assert not runner._graphs          # (no captured step takes 96 entries)
+        print(f"96 decoding requests {dtype}: worst relative error {worst:.3e}")
+        del model, runner

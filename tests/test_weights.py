@@ -113,6 +113,34 @@ def test_random_weights(tmp_path):
     assert torch.equal(alone, a.get("model.layers.2.self_attn.v_proj.weight"))
 
 
+def test_counter_based_generator_is_a_function_of_key_and_index():
+    """Pinned values (so that the device's twin and any later rewrite must make these very bits), independence of
+    how the elements are cut into pieces, and the distribution: close to normal with the asked deviation."""
+    import numpy as np
+    from vt_transformer_amd.weights.random_init import counter_normal, normal_scale, tensor_key
+    assert tensor_key(5, "model.norm.weight") == tensor_key(5, "model.norm.weight") != tensor_key(6, "model.norm.weight")
+    x = counter_normal(12345, 0, 200000, 0.02, 0.0)
+    assert x.dtype == np.float32
+    # the sum of the twelve 16-bit fields of three SplitMix64 words, by hand for element 7
+    def mix(z):
+        z &= (1 << 64) - 1
+        z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & ((1 << 64) - 1)
+        z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & ((1 << 64) - 1)
+        return z ^ (z >> 31)
+    total = 0
+    for j in (1, 2, 3):
+        w = mix(12345 + (3 * 7 + j) * 0x9E3779B97F4A7C15)
+        total += sum((w >> s) & 0xFFFF for s in (0, 16, 32, 48))
+    assert x[7] == np.float32(total - 393210) * np.float32(normal_scale(0.02))
+    pieces = np.concatenate([counter_normal(12345, a, b - a, 0.02, 0.0) for a, b in ((0, 7), (7, 1000), (1000, 200000))])
+    assert np.array_equal(pieces, x)
+    assert abs(float(x.mean())) < 2e-4 and abs(float(x.std()) - 0.02) < 2e-4
+    z = x / x.std()
+    assert abs(float((z ** 3).mean())) < 0.03 and 2.8 < float((z ** 4).mean()) < 3.0      # a sum of twelve: kurtosis 2.9
+    assert np.array_equal(counter_normal(12345, 0, 1000, 0.02, 1.0), x[:1000] + np.float32(1.0))
+    assert not np.array_equal(counter_normal(12346, 0, 1000, 0.02, 0.0), x[:1000])
+
+
 def test_a_tensor_stored_in_32_bit_stays_so():
     from vt_transformer_amd.parts.base import Runtime
     rt = Runtime(torch.device("cpu"), torch.bfloat16)

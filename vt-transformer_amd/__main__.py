@@ -57,6 +57,8 @@ def build_parser() -> argparse.ArgumentParser:
     # scheduler (vt_scheduler.hpp)
     p.add_argument("--max-running-reqs", type=int, default=128)
     p.add_argument("--num-pages", type=int, default=None, help="cache pages per group of layers (default: for max-running-reqs/4 full sequences)")
+    p.add_argument("--kv-bytes", type=int, default=None,
+                   help="size of the cache in bytes, shared by all groups of layers (instead of --num-pages)")
     p.add_argument("--max-seq-len", type=int, default=4096)
     p.add_argument("--page-size", type=int, default=16)
     p.add_argument("--max-extend-tokens", type=int, default=8192)
@@ -117,9 +119,11 @@ def main(argv: Optional[List[str]] = None) -> int:
     temperature = args.temperature if args.temperature is not None else (_env("SHELL_TEMPERATURE", 0.6, float) if shell else 0.0)
     top_k = args.top_k if args.top_k is not None else (_env("SHELL_TOP_K", -1, int) if shell else -1)
     top_p = args.top_p if args.top_p is not None else (_env("SHELL_TOP_P", 1.0, float) if shell else 1.0)
+    if args.kv_bytes is not None and args.num_pages is not None:
+        raise SystemExit("give --num-pages or --kv-bytes, not both")
     num_pages = args.num_pages or max(64, (args.max_seq_len // args.page_size) * max(1, args.max_running_reqs // 4))
     eng = Engine(args.model, dtype=args.dtype, seed=args.seed, max_running_reqs=args.max_running_reqs,
-                 num_pages=num_pages, max_seq_len=args.max_seq_len, page_size=args.page_size,
+                 num_pages=num_pages, kv_bytes=args.kv_bytes, max_seq_len=args.max_seq_len, page_size=args.page_size,
                  max_extend_tokens=args.max_extend_tokens, default_max_output=args.default_max_output,
                  chunk_size=args.chunk_size, decode_graphs=not args.no_decode_graphs, tune_gemm=args.tune_gemm,
                  single_weight_copy=args.single_weight_copy)

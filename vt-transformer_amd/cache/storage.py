@@ -31,8 +31,13 @@ class LayerCache:
 
 
 class CacheStorage:
-    def __init__(self, rt: Runtime, model, page_size: int, pool_tokens: int, max_requests: int, max_seq_len: int):
-        """`pool_tokens`: how many tokens the pages of each group hold together."""
+    def __init__(self, rt: Runtime, model, page_size: int, pool_tokens: Optional[int], max_requests: int,
+                 max_seq_len: int, kv_bytes: Optional[int] = None):
+        """`pool_tokens`: how many tokens the pages of each group hold together.  Or `kv_bytes`: a budget in bytes
+        for all keys and values, shared by the groups: a token takes a slot of a page in every group, so every
+        group gets the same number of pages, budget // (bytes of one page of each group together), as the
+        reference sizes its one pool (vt-transformer/models/qwen3-0.6b/init.vt:109-113:
+        num_blocks = budget // (block_size * per_token_bytes))."""
         self.rt = rt
         self.page_size = int(page_size)
         schedule = model.schedule
@@ -67,8 +72,25 @@ class CacheStorage:
             if e.cache_from is not None:
                 self.entry_group[i] = self.entry_group[e.cache_from]
                 self.entry_index[i] = self.entry_index[e.cache_from]
-        num_pages = max(1, -(-int(pool_tokens) // self.page_size))
         self.group_needs = [CacheNeed(*k) for k in keys]
+        elem = torch.empty((), dtype=rt.dtype).element_size()
+        # bytes of one page of every layer of a group: keys and values
+        self.page_bytes = [2 * members[g] * need.kv_heads * need.head_dim * self.page_size * elem
+                           for g, need in enumerate(self.group_needs)]
+        if kv_bytes is not None:
+            if pool_tokens is not None:
+                raise ValueError("give the cache's size in tokens or in bytes, not both")
+            per_page = sum(self.page_bytes)
+            num_pages = int(kv_bytes) // per_page if per_page else 1
+            if num_pages < 1 and per_page:
+                raise ValueError(f"a cache of {kv_bytes} bytes does not hold one page of {self.page_size} tokens "
+                                 f"({per_page} bytes over {len(keys)} group(s) of layers)")
+            num_pages = max(1, num_pages)
+        else:
+            if pool_tokens is None:
+                raise ValueError("the cache needs a size: pool_tokens or kv_bytes")
+            num_pages = max(1, -(-int(pool_tokens) // self.page_size))
+        self.num_pages = num_pages
         self.manager = CacheManager([GroupSpec(k, k[2], num_pages) for k in keys], self.page_size, max_requests,
                                     max_seq_len)
         self.k: List[torch.Tensor] = []
@@ -84,6 +106,11 @@ class CacheStorage:
         for need in state_needs:
             self.state.append(None if need is None else
                               torch.zeros((max_requests,) + tuple(need.shape), dtype=need.dtype, device=rt.device))
+
+    @property
+    def kv_bytes(self) -> int:
+        """Bytes that the pages of all groups take."""
+        return self.num_pages * sum(self.page_bytes)
 
     @property
     def n_groups(self) -> int:

@@ -554,3 +554,56 @@ extern "C" int vt_stream_read(const void* p, long long bytes, unsigned* sums, in
     VT_CHECK_LAUNCH("vt_stream_read");
     return 0;
 }
+
+// ---------------------------------------------------------------------------
+// Random weights whose bits do not depend on where they are made.  Element i of a tensor is a function of
+// (key, i) alone: three words of the SplitMix64 stream that starts at `key` (counters 3 i + 1 .. 3 i + 3), cut
+// into twelve 16-bit integers whose sum is close to normally distributed (mean 393,210, variance 2^32 - 1).  The
+// sum is exact in integers; one float multiplication and one addition, each rounded on its own, make the value,
+// so the host's twin of this kernel (weights/random_init.py) produces the same bits.  The reference has no such
+// mode (nearest: the fixed mt19937(1979) of v1/tensortype/context.cpp:45).
+__device__ __forceinline__ unsigned long long splitmix64_at(unsigned long long key, unsigned long long counter) {
+    unsigned long long z = key + counter * 0x9E3779B97F4A7C15ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
+
+template <typename TO>
+__global__ void random_normal_kernel(TO* __restrict__ out, unsigned long long n, unsigned long long first,
+                                     unsigned long long key, float scale, float mean) {
+    const unsigned long long stride = (unsigned long long)gridDim.x * blockDim.x;
+    for (unsigned long long i = (unsigned long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        const unsigned long long e = first + i;
+        int s = 0;
+#pragma unroll
+        for (int j = 1; j <= 3; ++j) {
+            const unsigned long long w = splitmix64_at(key, 3ull * e + j);
+            s += (int)(w & 0xffffu) + (int)((w >> 16) & 0xffffu) + (int)((w >> 32) & 0xffffu) + (int)(w >> 48);
+        }
+        float v;
+        {
+            // the product and the sum each rounded on its own, as the host's twin does: never one fused operation
+#pragma clang fp contract(off)
+            const float prod = (float)(s - 393210) * scale;
+            v = prod + mean;
+        }
+        store_f32<TO>(out, i, v);
+    }
+}
+
+// out[i] = mean + scale * (sum of twelve 16-bit integers of element first + i  -  393,210), i < n
+extern "C" int vt_random_normal(void* out, int out_dtype, long long n, long long first, unsigned long long key,
+                                float scale, float mean, hipStream_t stream) {
+    VT_REQUIRE(n >= 0 && first >= 0, "vt_random_normal: n=%lld first=%lld", n, first);
+    if (n == 0) return 0;
+    const unsigned blocks = (unsigned)((n + 255) / 256 < 16384 ? (n + 255) / 256 : 16384);
+    if (out_dtype == VT_F32)
+        random_normal_kernel<float><<<blocks, 256, 0, stream>>>((float*)out, (unsigned long long)n, (unsigned long long)first, key, scale, mean);
+    else if (out_dtype == VT_BF16)
+        random_normal_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)out, (unsigned long long)n, (unsigned long long)first, key, scale, mean);
+    else
+        return vt_fail("vt_random_normal: unknown out dtype %d", out_dtype);
+    VT_CHECK_LAUNCH("vt_random_normal");
+    return 0;
+}

@@ -29,7 +29,8 @@ class Engine:
                  tune_gemm: bool = False, single_weight_copy: bool = False, **options):
         """model: a folder with config.json and model.safetensors.  Or `config` with `random_weights_seed`
         for random weights drawn on the device.  `options` override fields of SchedulerConfig
-        (max_running_reqs, num_pages, max_seq_len, page_size, max_extend_tokens, default_max_output, chunk_size).
+        (max_running_reqs, num_pages or kv_bytes, max_seq_len, page_size, max_extend_tokens, default_max_output,
+        chunk_size).
         tune_gemm: let the GEMM library try its algorithms on this model's products at chunk_size rows (and at 128
         and 256 rows, if so many requests may run) once, at start-up (some seconds), and use the fastest from then on.
         single_weight_copy: keep the bfloat16 matrices once (in the few-row kernels' order) instead of twice; long
@@ -41,17 +42,19 @@ class Engine:
                 raise TypeError(f"unknown engine option '{k}'")
             setattr(sc, k, v)
         if model is not None:
-            self.model = load_model(model, dtype, keep_row_major=not single_weight_copy)
+            self.model = load_model(model, dtype, keep_row_major=not single_weight_copy, page_size=sc.page_size)
         elif config is not None and random_weights_seed is not None:
-            self.model = random_model(config, random_weights_seed, dtype, keep_row_major=not single_weight_copy)
+            self.model = random_model(config, random_weights_seed, dtype, keep_row_major=not single_weight_copy,
+                                      page_size=sc.page_size)
         else:
             raise ValueError("give a model folder, or a config and random_weights_seed")
         spec = self.model.spec
         sc.max_seq_len = min(sc.max_seq_len, spec.max_positions)
         self.config = sc
-        self.runner: ModelRunner = make_runner(self.model, pool_tokens=sc.num_pages * sc.page_size,
-                                               page_size=sc.page_size, max_requests=sc.max_running_reqs,
-                                               max_seq_len=sc.max_seq_len)
+        self.runner: ModelRunner = make_runner(
+            self.model, pool_tokens=None if sc.kv_bytes is not None else sc.num_pages * sc.page_size,
+            kv_bytes=sc.kv_bytes, page_size=sc.page_size, max_requests=sc.max_running_reqs, max_seq_len=sc.max_seq_len)
+        sc.num_pages = self.runner.storage.num_pages
         self.runner.decode_graphs = bool(decode_graphs)
         self.scheduler = Scheduler(sc, self.runner.cache, spec.eos_token_ids)
         self.sampler = Sampler(self.model.rt)

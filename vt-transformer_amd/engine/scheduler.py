@@ -46,6 +46,8 @@ class SchedulerConfig:
     max_extend_tokens: int = 8192   # new tokens per step, prompts and decoding together
     default_max_output: int = 1024  # output limit of a request that names none
     chunk_size: int = 2048          # longest portion of one prompt in a step
+    kv_bytes: Optional[int] = None  # the cache's size in bytes, shared by the groups of layers; sets num_pages
+                                    # (num_blocks = budget // bytes of a block, vt-transformer/models/qwen3-0.6b/init.vt:109-113)
 
 
 WAITING, RUNNING, FINISHED = "waiting", "running", "finished"

@@ -138,6 +138,15 @@ def stream_read(buf: torch.Tensor, sums: torch.Tensor, blocks: int = 256) -> tor
     return sums
 
 
+def random_normal(out: torch.Tensor, key: int, scale: float, mean: float, first: int = 0) -> torch.Tensor:
+    """out.flat[i] = mean + scale * (twelve 16-bit integers of element first + i, summed and centred): close to
+    N(mean, (65536 scale)^2), and the same bits as weights.random_init.counter_normal makes on the host."""
+    _chk(out, "random_normal.out")
+    _run(load_lib("vt_elementwise"), "vt_random_normal", _ptr(out), _i(_code(out)), ctypes.c_longlong(out.numel()),
+         ctypes.c_longlong(int(first)), ctypes.c_ulonglong(int(key) & 0xFFFFFFFFFFFFFFFF), _f(scale), _f(mean), _stream())
+    return out
+
+
 def rope_store(qkv: torch.Tensor, cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], positions: torch.Tensor,
                tok_entry: torch.Tensor, block_table: Optional[torch.Tensor], q_out: torch.Tensor,
                k_pages: Optional[torch.Tensor], v_pages: Optional[torch.Tensor], n_heads: int, n_kv: int, head_dim: int,

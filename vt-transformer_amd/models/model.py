@@ -67,13 +67,12 @@ class DecoderModel:
             for p in layer.parts():
                 p.load(get, self.rt)
         self.final_norm.load(get, self.rt)
+        # a head's loader takes `shared`: tensors by name that other parts have already placed on the device (the
+        # embedding's table, which a tied head multiplies by)
         shared = {}
         if getattr(self.embedding, "table", None) is not None:
             shared[self.embedding.name] = self.embedding.table
-        try:
-            self.head.load(get, self.rt, shared=shared)
-        except TypeError:
-            self.head.load(get, self.rt)
+        self.head.load(get, self.rt, shared=shared)
 
     # ------------------------------------------------------------------
     def forward(self, ctx, caches, states) -> Optional[torch.Tensor]:

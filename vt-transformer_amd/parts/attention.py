@@ -19,14 +19,15 @@ from typing import Callable, Dict, Optional
 import torch
 
 from ..config.base import PartSpec
+import numpy as np
+
 from ..kernels import ops
+from .attention_plan import decode_chunk, decode_parts_max, device_plan, plan_step
 from .base import MIXERS, POSITIONS, CacheNeed, Part, Runtime, StateNeed, TensorDecl
 from .linear import can_add_residual, linear
 
-
-def decode_bucket(n_kv: int) -> int:
-    """Which of the step's decode chunk lengths is meant for this many key/value heads."""
-    return min(7, max(1, int(n_kv)).bit_length() - 1)
+# the decoding kernels take the (token, head-of-group) rows of one entry as one tile of 16
+DECODE_MAX_GROUP = 16
 
 
 @MIXERS.register("attention")
@@ -46,6 +47,9 @@ class PagedAttention(Part):
         self.rt = rt
         self.width = int(width)
         self.nh, self.nkv, self.d = int(num_heads), int(num_kv_heads), int(head_dim)
+        if rt.dtype == torch.bfloat16 and (self.d % 16 or not 16 <= self.d <= 256):
+            raise ValueError(f"head size {self.d}: the bfloat16 attention kernels take multiples of 16 from 16 to 256 "
+                             f"(float32 takes any)")
         self.qkv_bias, self.out_bias = bool(qkv_bias), bool(out_bias)
         self.window = int(window)
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.d)
@@ -66,11 +70,12 @@ class PagedAttention(Part):
     def replayable(self) -> bool:
         # the decoding kernels cut the keys from positions in device memory; a group of more than 16 query heads
         # takes the kernel whose work items the host plans anew every step
-        return self.nh // self.nkv <= 16 and bool(getattr(self.position, "replayable", False))
+        return self.nh // self.nkv <= DECODE_MAX_GROUP and bool(getattr(self.position, "replayable", False))
 
     # -- what the cache manager must hold for this mixer --------------------
     def cache_need(self) -> Optional[CacheNeed]:
-        return CacheNeed(self.nkv, self.d, self.window)
+        # the bfloat16 kernels read keys 16 at a time, from one page
+        return CacheNeed(self.nkv, self.d, self.window, page_multiple=16 if self.rt.dtype == torch.bfloat16 else 1)
 
     def state_need(self) -> Optional[StateNeed]:
         return None
@@ -105,6 +110,43 @@ class PagedAttention(Part):
         self.w_qkv, self.w_o = rt.row_major(self.w_qkv, self.p_qkv), rt.row_major(self.w_o, self.p_o)
 
     # -- one step --------------------------------------------------------------
+    def _decode_key(self):
+        return ("attention.decode_chunk", self.nkv)
+
+    def _items_key(self):
+        return ("attention.items", self.nh // self.nkv, self.window, self.nkv, self.d)
+
+    def prepare_step(self, ctx) -> Optional[Dict[tuple, np.ndarray]]:
+        """The integers that this step's bfloat16 attention launches read from device memory.  A decoding step
+        (one token per entry): the number of keys per work item, one integer, so that a captured step can be
+        replayed with another one.  Any other step: the work items of the planned kernels.  Layers of the same
+        shape share one plan."""
+        if self.rt.dtype != torch.bfloat16:
+            return None
+        if ctx.single_token and self.nh // self.nkv <= DECODE_MAX_GROUP:
+            key = self._decode_key()
+            if key in ctx.extra_host:
+                return None
+            chunk = decode_chunk(ctx.h_kv_lens, decode_parts_max(ctx.n_positions), n_kv=self.nkv)
+            return {key: np.array([chunk], np.int32)}
+        key = self._items_key()
+        if key in ctx.extra_host:
+            return None
+        host = plan_step(ctx.h_entry_start, ctx.h_entry_pos0, self.nh // self.nkv, self.window, self.nkv, self.d)
+        ctx.memo[key] = host
+        return {key: host.flat()}
+
+    def _plan(self, ctx):
+        """The step's plan on the device (made once per step and shape of layer)."""
+        key = self._items_key()
+        plan = ctx.memo.get(("device",) + key)
+        if plan is None:
+            if key not in ctx.extra:
+                raise RuntimeError("the attention mixer was not asked to prepare this step (prepare_step)")
+            plan = device_plan(ctx.memo[key], ctx.extra[key], self.rt, self.nkv, self.d)
+            ctx.memo[("device",) + key] = plan
+        return plan
+
     def forward(self, x, ctx, cache, state=None, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
         rt, nh, nkv, d = self.rt, self.nh, self.nkv, self.d
         n = x.shape[0]
@@ -128,16 +170,16 @@ class PagedAttention(Part):
                 qkv[:, nq:nq + nkv * d] = k2.reshape(n, nkv * d).to(qkv.dtype)
         cos, sin = tables if tables is not None else (None, None)
         plain_positions = tables is not None or getattr(self.position, "dim", 0) == 0
-        if (rt.dtype == torch.bfloat16 and ctx.decode_params is not None and cache.writes and qkv.dtype == torch.float32
-                and plain_positions and nh // nkv <= 16 and (cos is None or cos.shape[1] % 8 == 0)):
+        chunk = ctx.extra.get(self._decode_key()) if rt.dtype == torch.bfloat16 and ctx.single_token else None
+        p_max = decode_parts_max(ctx.n_positions)
+        if (chunk is not None and cache.writes and qkv.dtype == torch.float32
+                and plain_positions and (cos is None or cos.shape[1] % 8 == 0)):
             # one token per entry, straight from the projection: the attention kernel rotates and writes the pages
             out = rt.buffer("attn.out", (n, nq), rt.dtype)
-            part_o = rt.buffer("attn.dec_part_o", (n * ctx.decode_p_max * nkv * 16 * d,), torch.float32)
-            part_ml = rt.buffer("attn.dec_part_ml", (n * ctx.decode_p_max * nkv * 32,), torch.float32)
-            b = decode_bucket(nkv)
+            part_o = rt.buffer("attn.dec_part_o", (n * p_max * nkv * 16 * d,), torch.float32)
+            part_ml = rt.buffer("attn.dec_part_ml", (n * p_max * nkv * 32,), torch.float32)
             ops.attention_bf16_decode_fused(qkv, cos, sin, cache.k, cache.v, cache.block_table, ctx.entry_pos0,
-                                            ctx.decode_params[b:b + 1], ctx.decode_p_max, out, part_o, part_ml, nh, nkv, d,
-                                            self.window, self.scale)
+                                            chunk, p_max, out, part_o, part_ml, nh, nkv, d, self.window, self.scale)
             return linear(rt, out, self.w_o, self.b_o, "attn.o", packed=self.p_o, residual=residual)
         q = rt.buffer("attn.q", (n, nq), rt.dtype)
         ops.rope_store(qkv, cos, sin, ctx.positions, ctx.tok_entry, cache.block_table, q, cache.k, cache.v, nh, nkv, d,
@@ -146,15 +188,14 @@ class PagedAttention(Part):
         if rt.dtype == torch.float32:
             ops.attention_f32(q, cache.k, cache.v, ctx.positions, ctx.tok_entry, cache.block_table, out, nh, nkv, d,
                               self.window, self.scale)
-        elif ctx.decode_params is not None and nh // nkv <= 16:
+        elif chunk is not None:
             # one token per entry: the kernel cuts the keys itself from the positions on the device
-            part_o = rt.buffer("attn.dec_part_o", (n * ctx.decode_p_max * nkv * 16 * d,), torch.float32)
-            part_ml = rt.buffer("attn.dec_part_ml", (n * ctx.decode_p_max * nkv * 32,), torch.float32)
-            b = decode_bucket(nkv)
-            ops.attention_bf16_decode(q, cache.k, cache.v, cache.block_table, ctx.entry_pos0, ctx.decode_params[b:b + 1],
-                                      ctx.decode_p_max, out, part_o, part_ml, nh, nkv, d, self.window, self.scale)
+            part_o = rt.buffer("attn.dec_part_o", (n * p_max * nkv * 16 * d,), torch.float32)
+            part_ml = rt.buffer("attn.dec_part_ml", (n * p_max * nkv * 32,), torch.float32)
+            ops.attention_bf16_decode(q, cache.k, cache.v, cache.block_table, ctx.entry_pos0, chunk, p_max, out,
+                                      part_o, part_ml, nh, nkv, d, self.window, self.scale)
         else:
-            plan = ctx.attention_plan(nh // nkv, self.window, nkv, d)
+            plan = self._plan(ctx)
             if plan.n_items:        # decoded tokens and short portions: 16-row items, keys split where that helps
                 ops.attention_bf16(q, cache.k, cache.v, cache.block_table, plan.items, plan.n_items, plan.citems,
                                    plan.n_citems, out, plan.part_o, plan.part_ml, nh, nkv, d, self.window, self.scale,

@@ -16,7 +16,14 @@ Interfaces (N = tokens of the step, H = model width):
                   apply(q, k, positions) -> (q, k) otherwise.
   Mixer           forward(x[N,H], ctx, cache, state) -> [N,H]; cache_need() / state_need() say what the cache
                   manager has to hold for it (keys and values in pages; fixed-size state per request).
+                  Optional: prepare_step(ctx) -> {key: int32 array} or None, called on the host once per step
+                  before the step's metadata goes to the device; what it returns is found in ctx.extra[key] on
+                  the device when the part runs (work items of its kernels, lengths they read from memory).
   FeedForward     forward(x[N,H], ctx) -> [N,H]
+  Embedding       forward(ids[N] int32) -> h[N,H] fp32; `name` and `table` say what it has loaded.
+  Head            load(get, rt, shared) where `shared` maps tensor names to tensors that other parts have placed
+                  on the device already (a tied head finds the embedding's table there); forward(x[R,H]) -> fp32
+                  logits [R,V].
   Block           forward(h, delta, ctx, cache, state) -> (h, delta): arranges two norms, a mixer and a
                   feed-forward around the fp32 residual stream h.  `delta` is a layer output that has
                   not been added to h yet, so that the next norm can fuse the addition.
@@ -55,6 +62,7 @@ class CacheNeed:
     kv_heads: int
     head_dim: int
     window: int = 0  # 0: every key stays; W: a key is dead once W later tokens exist
+    page_multiple: int = 1  # the mixer's kernels take pages whose size is a multiple of this many tokens
 
     def group_key(self):
         return (self.kv_heads, self.head_dim, self.window)
