@@ -6,8 +6,9 @@
 Prints one JSON line.  `value` is decoded tokens per second at batch 8 after 1,024-token prompts (a step is one
 decode step of the whole batch through scheduler, step function and sampler).  The line also carries the
 prefill of one 2,048-token prompt, the decode step's achieved HBM bandwidth against the bytes it has to read,
-decode at batch 1 and 64, and what this GPU's memory and matrix cores were measured to deliver (a kernel that only
-reads; the library's square product), beside the published peaks that the fractions are taken against.  The reference publishes no number to compare with (vs_baseline is null).
+decode at batch 1 and 64 (`points`, and `points_frac`: their fractions of the same roofline), and what this GPU's
+memory and matrix cores were measured to deliver (a kernel that only reads; the library's square product), beside
+the published peaks that the fractions are taken against (`vs_measured_peaks`: the same fractions against those).  The reference publishes no number to compare with (vs_baseline is null).
 """
 import argparse
 import json
@@ -218,11 +219,15 @@ def main() -> int:
     attn_flops = L * 4.0 * cfg.num_attention_heads * cfg.head_dim * (T * (T + 1) / 2)   # causal: QK^T and PV
     p_flops = mm_flops + attn_flops
 
-    points = {}
+    points, points_frac = {}, {}
     if not args.no_points:
         for b in point_batches:
             k = max(16, args.steps // 2)
-            points[f"decode_b{b}"] = round(decode_run(b, k, 8)[0], 1)
+            b_tps, b_ms, b_ctx = decode_run(b, k, 8)
+            points[f"decode_b{b}"] = round(b_tps, 1)
+            # the same roofline as the headline's: the weights once and the live requests' keys and values
+            points_frac[f"decode_b{b}"] = round((weight_bytes + b * b_ctx * kv_bytes_per_token) / (b_ms * 1e-3) / 1e9
+                                                / HBM_GBPS, 4)
 
     line = {
         "metric": f"decode tok/s at batch {args.batch}, {model_name} layer sizes, {args.prompt_len:,}-token prompts",
@@ -240,9 +245,18 @@ def main() -> int:
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_GBPS, 4)},
         "points": points,
+        "points_frac": points_frac,
     }
     if not args.no_peaks:
-        line["measured_peaks"] = measured_peaks()
+        peaks = measured_peaks()
+        line["measured_peaks"] = peaks
+        # the same fractions against what this machine was measured to deliver
+        vs = {"decode": round(achieved / peaks["hbm_read_GBps"], 4)}
+        if p_dt is not None:
+            vs["prefill"] = round(p_flops / p_dt / (peaks["gemm_bf16_TFLOPs"] * 1e12), 4)
+        for k_, f in points_frac.items():
+            vs[k_] = round(f * HBM_GBPS / peaks["hbm_read_GBps"], 4)
+        line["vs_measured_peaks"] = vs
     print(json.dumps(line), flush=True)
     return 0
 

@@ -687,3 +687,64 @@ def test_random_normal_kernel_makes_the_hosts_bits(dtype, n, first):
         ops().random_normal(out, key, normal_scale(0.02), mean, first=first)
         want = torch.from_numpy(counter_normal(key, first, n, 0.02, mean)).to(dtype)
         assert torch.equal(out.cpu(), want), (key, mean)
+
+
+@pytest.mark.parametrize("n", [1, 5, 8, 16])
+@pytest.mark.parametrize("h,k1,m2,gated", [(3584, 3584, 4608, False), (3584, 18944, 1184, True), (200, 96, 320, False),
+                                           (1536, 8960, 2048, False), (8192, 512, 640, True), (72, 40, 56, True)])
+def test_rmsnorm_handed_from_one_product_to_the_next(n, h, k1, m2, gated):
+    """A product that adds to the residual stream prepares the norm behind it (the stream times the gains in
+    bfloat16, its blocks' shares of the rows' sums of squares); the product behind the norm takes those as its
+    tokens and divides by the root.  Against the plain chain: add, RMSNorm, product."""
+    o = ops()
+    g = torch.Generator().manual_seed(n * 1000 + h)
+    x = (torch.randn(n, k1, generator=g) * 0.5).to(torch.bfloat16)
+    w1 = (torch.randn(h, k1, generator=g) * 0.05).to(torch.bfloat16)
+    bias1 = torch.randn(h, generator=g) * 0.1
+    resid = torch.randn(n, h, generator=g)
+    gain = 1.0 + 0.1 * torch.randn(h, generator=g)
+    w2 = (torch.randn((2 if gated else 1) * m2, h, generator=g) * 0.05).to(torch.bfloat16)
+    eps = 1e-5
+    shares = o.linear_bf16_link_shares(n, h, k1)
+    assert shares == (h + 15) // 16
+    hbuf = resid.clone().to(DEV)
+    xn = torch.full((n, h), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ssq = torch.full((shares, 16), float("nan"), dtype=torch.float32, device=DEV)
+    o.linear_bf16_link(x.to(DEV), o.pack_matrix_bf16(w1.to(DEV)), bias1.to(DEV), hbuf, residual=hbuf, xn_out=xn,
+                       gain_next=gain.to(DEV), ssq_out=ssq)
+    h_ref = resid.double() + x.double() @ w1.double().t() + bias1.double()
+    assert rel_err(hbuf, h_ref) < 1e-5
+    assert rel_err(ssq[:, :n].sum(dim=0), (h_ref * h_ref).sum(dim=1)) < 1e-5
+    assert bool((ssq[:, n:] == 0).all())
+    # what the consumer reads: exactly bf16(h * gain) of the stream as the producer left it
+    assert torch.equal(xn.cpu(), (hbuf.cpu() * gain).to(torch.bfloat16))
+    normed = bf16_round(hbuf.cpu() * gain) / torch.sqrt((h_ref * h_ref).mean(dim=1, keepdim=True) + eps)
+    if gated:
+        out = torch.empty(n, m2, dtype=torch.float32, device=DEV)
+        o.gated_linear_bf16_link(xn, o.pack_matrix_bf16(w2.to(DEV), halves=2), out, ssq, eps)
+        gate, up = normed @ w2[:m2].double().t(), normed @ w2[m2:].double().t()
+        ref = gate / (1 + torch.exp(-gate)) * up
+    else:
+        bias2 = torch.randn(m2, generator=g) * 0.1
+        out = torch.empty(n, m2, dtype=torch.float32, device=DEV)
+        o.linear_bf16_link(xn, o.pack_matrix_bf16(w2.to(DEV)), bias2.to(DEV), out, ssq_in=ssq, eps_in=eps)
+        ref = normed @ w2.double().t() + bias2.double()
+    assert rel_err(out, ref) < 3e-5
+    # and the same bits as the product that applies the norm itself from the float32 stream
+    if gated:
+        same = torch.empty(n, m2, dtype=torch.float32, device=DEV)
+        o.gated_linear_bf16(hbuf, o.pack_matrix_bf16(w2.to(DEV), halves=2), same, norm_gain=gain.to(DEV), norm_eps=eps)
+        assert rel_err(out, same) < 2e-6
+
+
+def test_rmsnorm_hand_over_is_refused_where_it_cannot_work():
+    o = ops()
+    assert o.linear_bf16_link_shares(17, 3584, 3584) == 0        # more than 16 rows
+    assert o.linear_bf16_link_shares(8, 3584, 100) == 0          # k no multiple of 8
+    assert o.linear_bf16_link_shares(8, 100, 64) == 0            # a width that the next product could not read by 16 bytes
+    x = torch.zeros(17, 64, dtype=torch.bfloat16, device=DEV)
+    w = o.pack_matrix_bf16(torch.zeros(32, 64, dtype=torch.bfloat16, device=DEV))
+    out = torch.zeros(17, 32, device=DEV)
+    ssq = torch.zeros(4, 16, device=DEV)
+    with pytest.raises(Exception, match="up to 16 rows"):
+        o.linear_bf16_link(x, w, None, out, ssq_in=ssq, eps_in=1e-6)

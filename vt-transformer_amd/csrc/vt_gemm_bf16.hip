@@ -126,6 +126,25 @@ __device__ __forceinline__ bf16x8_t load_x(const bf16_t* row, int k, int K) {
 }
 
 // ---------------------------------------------------------------------------
+// An RMSNorm handed from the product in front of it to the product behind it, so that it is no kernel of its own
+// and the product behind it reads its tokens in bf16 like any other.
+// The product in front (one that adds its result to the residual stream h) is the producer: beside h it writes
+// xn = bf16(h * gain) for the norm's gains, and each of its blocks writes its features' share of every row's sum
+// of h^2 to ssq_out[block][row].  The product behind is the consumer: its tokens are xn, it adds up the shares in
+// block order and multiplies its sums by 1/sqrt(sum / width + eps), which is where the norm's division belongs
+// since it is the same for a whole row.  The shares are added in a fixed order: the result does not depend on
+// which block finished first.  Rows of ssq are SSQ_STRIDE(N) floats apart.
+struct NormLink {
+    bf16_t* xn_out;            // producer: [N][Mout], or null
+    const float* gain_next;    //           [Mout]
+    float* ssq_out;            //           [blocks][stride]
+    const float* ssq_in;       // consumer: [n_ssq][stride], or null
+    int n_ssq;
+    float eps;
+};
+#define SSQ_STRIDE(N) ((N) <= 16 ? 16 : 64)
+
+// ---------------------------------------------------------------------------
 // Up to 16 tokens: a block owns one tile row of W (16 features; two for the gated product) and all of k, which
 // its WPB waves split; the tokens are the B operand.  U tiles are in flight per wave and matrix.
 //
@@ -145,15 +164,26 @@ __global__ __launch_bounds__(WPB * 64) void gemm_skinny_kernel(const void* __res
                                                               const float* __restrict__ bias, TO* __restrict__ y, int N,
                                                               int Mout, int K, int KT, int up_tiles,
                                                               const float* __restrict__ gain, float eps,
-                                                              const float* resid) {
+                                                              const float* resid, NormLink link) {
     constexpr int NW = SWIGLU ? 2 : 1;
     constexpr int U = NORM ? 2 : 4;     // tiles in flight (fp32 tokens take three times the registers: measured)
     __shared__ float red[NW][WPB][256];
     __shared__ uint4 xt[WPB][2][4 * 17];
     __shared__ float ssq[NORM ? WPB : 1][16];
+    __shared__ float4 ssq_part[WPB][4];                       // consumer of a NormLink: the waves' sums of shares
     const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63;
     const int r = lane & 15, g = lane >> 4;
     const int mt = blockIdx.x;
+    // Consumer of a NormLink: thread t adds up rows 4 (t % 4) .. + 3 of shares t / 4, t / 4 + threads / 4, ...; the
+    // first two loads are asked for here, ahead of everything, and used at the end.
+    float4 sh0 = make_float4(0.f, 0.f, 0.f, 0.f), sh1 = sh0;
+    if constexpr (!NORM) {
+        if (link.ssq_in) {
+            const int b0 = tid >> 2, b1 = b0 + WPB * 16;
+            if (b0 < link.n_ssq) sh0 = *(const float4*)(link.ssq_in + (size_t)b0 * 16 + (tid & 3) * 4);
+            if (b1 < link.n_ssq) sh1 = *(const float4*)(link.ssq_in + (size_t)b1 * 16 + (tid & 3) * 4);
+        }
+    }
     const int t_begin = (int)(((long long)wv * KT) / WPB), t_end = (int)(((long long)(wv + 1) * KT) / WPB);
     const bf16_t* wbase[NW];
     wbase[0] = wp + ((size_t)mt * KT * 64 + lane) * 8;
@@ -264,6 +294,23 @@ __global__ __launch_bounds__(WPB * 64) void gemm_skinny_kernel(const void* __res
     for (int a = 0; a < NW; ++a)
 #pragma unroll
         for (int e = 0; e < 4; ++e) red[a][wv][lane * 4 + e] = acc[a][e];
+    const bool consumes = !NORM && link.ssq_in != nullptr;
+    if constexpr (!NORM) {
+        if (consumes) {
+            float4 sh = make_float4(sh0.x + sh1.x, sh0.y + sh1.y, sh0.z + sh1.z, sh0.w + sh1.w);
+            for (int b = (tid >> 2) + 2 * WPB * 16; b < link.n_ssq; b += WPB * 16) {      // (more than 2 x threads / 4 shares)
+                const float4 t4 = *(const float4*)(link.ssq_in + (size_t)b * 16 + (tid & 3) * 4);
+                sh.x += t4.x; sh.y += t4.y; sh.z += t4.z; sh.w += t4.w;
+            }
+            // the 16 lanes of a wave that hold the same four rows; every lane ends with the same sum
+#pragma unroll
+            for (int o = 4; o < 64; o <<= 1) {
+                sh.x += __shfl_xor(sh.x, o, 64); sh.y += __shfl_xor(sh.y, o, 64);
+                sh.z += __shfl_xor(sh.z, o, 64); sh.w += __shfl_xor(sh.w, o, 64);
+            }
+            if (lane < 4) ssq_part[wv][lane] = sh;
+        }
+    }
     __syncthreads();
     for (int c = tid; c < 256; c += WPB * 64) {
         const int ln = c >> 2, e = c & 3;
@@ -272,6 +319,7 @@ __global__ __launch_bounds__(WPB * 64) void gemm_skinny_kernel(const void* __res
         for (int q = 0; q < WPB; ++q) v += red[0][q][c];
         if (SWIGLU)
             for (int q = 0; q < WPB; ++q) u += red[NW - 1][q][c];
+        float sq = 0.f;
         if (m < Mout && n < N) {
             if constexpr (NORM) {
                 float tot = 0.f;
@@ -279,11 +327,33 @@ __global__ __launch_bounds__(WPB * 64) void gemm_skinny_kernel(const void* __res
                 const float rinv = 1.0f / sqrtf(tot / (float)K + eps);
                 v *= rinv;
                 u *= rinv;
+            } else if (consumes) {
+                float tot = 0.f;
+                const float* col = (const float*)&ssq_part[0][0] + n;       // [waves][16 rows]
+                for (int q = 0; q < WPB; ++q) tot += col[q * 16];
+                const float rinv = 1.0f / sqrtf(tot / (float)K + link.eps);
+                v *= rinv;
+                u *= rinv;
             }
             if (SWIGLU) v = v / (1.f + expf(-v)) * u;
             else if (bias) v += bias[m];
             if (resid) v += resid[(size_t)n * Mout + m];
             store_f32<TO>(y, (size_t)n * Mout + m, v);
+            if (link.xn_out) {
+                link.xn_out[(size_t)n * Mout + m] = f32_to_bf16(v * link.gain_next[m]);
+                sq = v * v;
+            }
+        }
+        if (link.xn_out) red[0][0][c] = sq;       // (this thread alone has read slot c)
+    }
+    if (link.xn_out) {
+        // this block's share of the rows' sums of squares: 16 features per row, added in feature order
+        __syncthreads();
+        if (tid < 16) {
+            float tot = 0.f;
+            for (int gg = 0; gg < 4; ++gg)
+                for (int e = 0; e < 4; ++e) tot += red[0][0][((gg * 16 + tid) << 2) + e];
+            link.ssq_out[(size_t)blockIdx.x * 16 + tid] = tot;
         }
     }
 }
@@ -665,10 +735,26 @@ extern "C" long long vt_linear_bf16_workspace(int N, int M, int K, int gated) {
 
 // gain != null: x is the fp32 residual stream and the RMSNorm (gain, eps) is part of the product (up to 16 tokens);
 // resid != null: the result is added to it (up to 64 tokens).
+static const NormLink NO_LINK = {nullptr, nullptr, nullptr, nullptr, 0, 0.f};
+
+// shares of the rows' sums of squares that a producing product of this shape writes (0: it cannot produce)
+extern "C" int vt_linear_bf16_link_shares(int N, int M, int K) {
+    if (N <= 0 || N > 16 || M <= 0 || K <= 0 || K % 8 != 0 || M % 8 != 0) return 0;
+    return (M + 15) / 16;
+}
+
 template <bool SWIGLU, typename TO>
 static int linear_bf16(const void* xv, const bf16_t* wp, const float* bias, TO* y, float* workspace, int N, int Mout,
-                       int K, const float* gain, float eps, const float* resid, hipStream_t stream) {
+                       int K, const float* gain, float eps, const float* resid, hipStream_t stream,
+                       const NormLink& link = NO_LINK) {
     if (N == 0) return 0;
+    const bool linked = link.xn_out || link.ssq_in;
+    VT_REQUIRE(!linked || (N <= 16 && K % 8 == 0 && (((uintptr_t)xv) & 15) == 0 && !gain),
+               "vt_linear_bf16: a norm is handed over between products of up to 16 rows with k a multiple of 8 (N=%d, K=%d)", N, K);
+    VT_REQUIRE(!link.xn_out || (resid && vt_linear_bf16_link_shares(N, Mout, K) > 0 && link.gain_next && link.ssq_out),
+               "vt_linear_bf16: a product that hands a norm on adds to a residual and has gains and room for the sums");
+    VT_REQUIRE(!link.ssq_in || (link.n_ssq > 0 && (((uintptr_t)link.ssq_in) & 15) == 0),
+               "vt_linear_bf16: the shares of the sums of squares are missing or not 16-byte aligned");
     const bf16_t* x = (const bf16_t*)xv;
     VT_REQUIRE(!gain || N <= 16, "vt_linear_bf16: the fused norm needs at most 16 rows (N=%d)", N);
     VT_REQUIRE((!gain && !resid) || (K % 8 == 0 && (((uintptr_t)xv) & 15) == 0),
@@ -720,7 +806,7 @@ static int linear_bf16(const void* xv, const bf16_t* wp, const float* bias, TO* 
     // in the same order whatever the number of rows: 8 waves, 16 for matrices with few rows and a long k.
     const int tiles16 = (Mout + 15) / 16;
     const bool wide = tiles16 >= 512 || KT < 256;
-#define VT_SKINNY(W, NRM) gemm_skinny_kernel<W, SWIGLU, NRM, TO><<<tiles16, W * 64, 0, stream>>>(x, wp, bias, y, N, Mout, K, KT, up_tiles, gain, eps, resid)
+#define VT_SKINNY(W, NRM) gemm_skinny_kernel<W, SWIGLU, NRM, TO><<<tiles16, W * 64, 0, stream>>>(x, wp, bias, y, N, Mout, K, KT, up_tiles, gain, eps, resid, link)
     if (gain) { if (wide) VT_SKINNY(8, true); else VT_SKINNY(16, true); }
     else { if (wide) VT_SKINNY(8, false); else VT_SKINNY(16, false); }
 #undef VT_SKINNY
@@ -788,6 +874,31 @@ extern "C" int vt_linear_bf16_fused(const void* h, const float* gain, float eps,
     VT_REQUIRE(N >= 0 && M > 0 && K > 0, "vt_linear_bf16_fused: bad sizes N=%d M=%d K=%d", N, M, K);
     VT_REQUIRE(gain || resid, "vt_linear_bf16_fused: neither a norm nor a residual: use vt_linear_bf16");
     return linear_bf16<false, float>(h, (const bf16_t*)wp, bias, y, nullptr, N, M, K, gain, eps, resid, stream);
+}
+
+// The product between two RMSNorms that are no kernels of their own (up to 16 rows):
+// ssq_in != null: x is xn = bf16(h * gain) as a producing product left it, ssq_in [n_ssq][16] its blocks' shares of the
+// rows' sums of h^2, and the result is multiplied by 1/sqrt(sum / K + eps_in);
+// xn_out != null (needs resid): beside y = resid + product, xn_out [N][M] = bf16(y * gain_next) and this product's
+// shares ssq_out [vt_linear_bf16_link_shares(N, M, K)][16] are written for the product behind the next norm.
+extern "C" int vt_linear_bf16_link(const void* x, const void* wp, const float* bias, const float* resid, float* y,
+                                   int N, int M, int K, const float* ssq_in, int n_ssq, float eps_in, void* xn_out,
+                                   const float* gain_next, float* ssq_out, hipStream_t stream) {
+    VT_REQUIRE(N >= 0 && M > 0 && K > 0, "vt_linear_bf16_link: bad sizes N=%d M=%d K=%d", N, M, K);
+    VT_REQUIRE(ssq_in || xn_out, "vt_linear_bf16_link: neither end of a norm: use vt_linear_bf16");
+    const NormLink link = {(bf16_t*)xn_out, gain_next, ssq_out, ssq_in, n_ssq, eps_in};
+    return linear_bf16<false, float>(x, (const bf16_t*)wp, bias, y, nullptr, N, M, K, nullptr, 0.f, resid, stream, link);
+}
+
+// the gated product behind a norm that the product in front has prepared (x = xn, ssq_in, n_ssq, eps_in as above)
+extern "C" int vt_gated_linear_bf16_link(const void* x, const void* wp, void* y, int out_dtype, int N, int I, int K,
+                                         const float* ssq_in, int n_ssq, float eps_in, hipStream_t stream) {
+    VT_REQUIRE(N >= 0 && I > 0 && K > 0, "vt_gated_linear_bf16_link: bad sizes N=%d I=%d K=%d", N, I, K);
+    VT_REQUIRE(ssq_in, "vt_gated_linear_bf16_link: no sums of squares: use vt_gated_linear_bf16");
+    const NormLink link = {nullptr, nullptr, nullptr, ssq_in, n_ssq, eps_in};
+    if (out_dtype == VT_F32) return linear_bf16<true, float>(x, (const bf16_t*)wp, nullptr, (float*)y, nullptr, N, I, K, nullptr, 0.f, nullptr, stream, link);
+    if (out_dtype == VT_BF16) return linear_bf16<true, bf16_t>(x, (const bf16_t*)wp, nullptr, (bf16_t*)y, nullptr, N, I, K, nullptr, 0.f, nullptr, stream, link);
+    return vt_fail("vt_gated_linear_bf16_link: unknown out dtype %d", out_dtype);
 }
 
 // y[N, I] = silu(x . Wg^T) * (x . Wu^T); wp = Wg [I, K] packed, followed by Wu [I, K] packed.

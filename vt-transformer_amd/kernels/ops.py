@@ -310,6 +310,74 @@ def linear_bf16(x: torch.Tensor, w, bias: Optional[torch.Tensor], out: torch.Ten
     return out
 
 
+_link_shares = {}
+
+
+def linear_bf16_link_shares(n: int, m: int, k: int) -> int:
+    """Blocks' shares of the rows' sums of squares that a product of this shape writes when it hands an RMSNorm on to
+    the product behind it (linear_bf16_link with xn_out); 0: this shape cannot."""
+    key = (n, m, k)
+    if key not in _link_shares:
+        _link_shares[key] = int(load_lib("vt_gemm_bf16").vt_linear_bf16_link_shares(_i(n), _i(m), _i(k)))
+    return _link_shares[key]
+
+
+def linear_bf16_link(x: torch.Tensor, w: PackedMatrix, bias: Optional[torch.Tensor], out: torch.Tensor,
+                     residual: Optional[torch.Tensor] = None, ssq_in: Optional[torch.Tensor] = None, eps_in: float = 0.0,
+                     xn_out: Optional[torch.Tensor] = None, gain_next: Optional[torch.Tensor] = None,
+                     ssq_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The few-row product between RMSNorms that are no kernels of their own (up to 16 rows).
+    ssq_in (float32 [shares, 16]): x is bf16(h * gain) as the product in front left it, and the result is divided by
+    the norm's root, which the shares of the rows' sums of squares give (eps_in: the norm's eps).
+    xn_out (bfloat16 [n, m]; needs residual): beside out = residual + product, xn_out = bf16(out * gain_next) and this
+    product's own shares ssq_out (float32 [linear_bf16_link_shares(n, m, k), 16]) for the product behind the next norm."""
+    n, k = x.shape
+    m = w.rows
+    if w.cols != k or w.halves != 1:
+        raise KernelError(f"linear_bf16_link: x [{n}, {k}] does not fit a packed matrix [{w.rows}, {w.cols}] x {w.halves}")
+    _chk(x, "linear_bf16_link.x", torch.bfloat16)
+    _chk(w.data, "linear_bf16_link.w", torch.bfloat16)
+    _chk(out, "linear_bf16_link.out", torch.float32, (n, m))
+    if bias is not None:
+        _chk(bias, "linear_bf16_link.bias", torch.float32, (m,))
+    if residual is not None:
+        _chk(residual, "linear_bf16_link.residual", torch.float32, (n, m))
+    n_ssq = 0
+    if ssq_in is not None:
+        _chk(ssq_in, "linear_bf16_link.ssq_in", torch.float32)
+        if ssq_in.dim() != 2 or ssq_in.shape[1] != 16:
+            raise KernelError(f"linear_bf16_link.ssq_in: shape {tuple(ssq_in.shape)}, expected [shares, 16]")
+        n_ssq = ssq_in.shape[0]
+    if xn_out is not None:
+        shares = linear_bf16_link_shares(n, m, k)
+        if residual is None or shares == 0:
+            raise KernelError(f"linear_bf16_link: {n} rows of [{m}, {k}] cannot hand a norm on (linear_bf16_link_shares)")
+        _chk(xn_out, "linear_bf16_link.xn_out", torch.bfloat16, (n, m))
+        _chk(gain_next, "linear_bf16_link.gain_next", torch.float32, (m,))
+        _chk(ssq_out, "linear_bf16_link.ssq_out", torch.float32, (shares, 16))
+    _run(load_lib("vt_gemm_bf16"), "vt_linear_bf16_link", _ptr(x), _ptr(w.data), _ptr(bias), _ptr(residual), _ptr(out),
+         _i(n), _i(m), _i(k), _ptr(ssq_in), _i(n_ssq), _f(eps_in), _ptr(xn_out), _ptr(gain_next), _ptr(ssq_out), _stream())
+    return out
+
+
+def gated_linear_bf16_link(x: torch.Tensor, w: PackedMatrix, out: torch.Tensor, ssq_in: torch.Tensor,
+                           eps_in: float) -> torch.Tensor:
+    """gated_linear_bf16 behind an RMSNorm that the product in front has prepared: x = bf16(h * gain), ssq_in its
+    shares of the rows' sums of squares (up to 16 rows)."""
+    n, k = x.shape
+    if w.cols != k or w.halves != 2:
+        raise KernelError(f"gated_linear_bf16_link: x [{n}, {k}] does not fit a packed matrix [{w.rows}, {w.cols}] x {w.halves}")
+    _chk(x, "gated_linear_bf16_link.x", torch.bfloat16)
+    _chk(w.data, "gated_linear_bf16_link.w", torch.bfloat16)
+    _chk(out, "gated_linear_bf16_link.out", None, (n, w.rows))
+    _chk(ssq_in, "gated_linear_bf16_link.ssq_in", torch.float32)
+    if ssq_in.dim() != 2 or ssq_in.shape[1] != 16:
+        raise KernelError(f"gated_linear_bf16_link.ssq_in: shape {tuple(ssq_in.shape)}, expected [shares, 16]")
+    _run(load_lib("vt_gemm_bf16"), "vt_gated_linear_bf16_link", _ptr(x), _ptr(w.data), _ptr(out), _i(_code(out)), _i(n),
+         _i(w.rows), _i(k), _ptr(ssq_in), _i(ssq_in.shape[0]), _f(eps_in), _stream())
+    return out
+
+
 def gated_linear_bf16(x: torch.Tensor, w_gate_up, out: torch.Tensor, norm_gain: Optional[torch.Tensor] = None,
                       norm_eps: float = 0.0) -> torch.Tensor:
     """out = silu(x Wg^T) * (x Wu^T).  w_gate_up: a PackedMatrix of two halves (pack_matrix_bf16(w, halves=2)), or

@@ -13,8 +13,8 @@ from typing import Callable, Dict, List, Optional
 import torch
 
 from ..config.base import LayerSpec, ModelSpec, PartSpec
-from ..parts.base import (BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, Part, Registry, Runtime,
-                          TensorDecl)
+from ..parts.base import (BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, NormedInput, Part, Registry,
+                          Runtime, TensorDecl)
 
 
 def build_part(registry: Registry, spec: PartSpec, prefix: str, **context):
@@ -80,9 +80,20 @@ class DecoderModel:
         Returns fp32 logits [rows wanted, vocab], or None if no row is wanted."""
         h = self.embedding.forward(ctx.token_ids)
         delta = None
+        last = len(self.schedule) - 1
         for i, entry in enumerate(self.schedule):
-            h, delta = self.layers[entry.layer].forward(h, delta, ctx, caches[i], states[i])
+            block = self.layers[entry.layer]
+            if getattr(block, "takes_next_norm", False):
+                # the norm that the layer behind starts with, which this layer's last product may prepare
+                nxt = getattr(self.layers[self.schedule[i + 1].layer], "first_norm", None) if i < last else None
+                h, delta = block.forward(h, delta, ctx, caches[i], states[i], next_norm=nxt)
+            else:
+                if isinstance(delta, NormedInput):
+                    delta = None            # (its addition is done; this block applies its own norm)
+                h, delta = block.forward(h, delta, ctx, caches[i], states[i])
         if ctx.n_logit_rows == 0:
             return None
+        if isinstance(delta, NormedInput):
+            delta = None
         x = self.final_norm.forward(h, delta, rows=ctx.logit_rows)
         return self.head.forward(x)

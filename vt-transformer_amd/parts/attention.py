@@ -33,6 +33,7 @@ DECODE_MAX_GROUP = 16
 @MIXERS.register("attention")
 class PagedAttention(Part):
     takes_normed_input = True     # the q/k/v product applies the norm in front of it when the rows are few
+    hands_norm_on = True          # ... and the output product prepares the norm behind it
 
     def adds_residual(self, rows: int) -> bool:
         """Whether the output product adds to the residual stream itself at this many rows."""
@@ -147,7 +148,7 @@ class PagedAttention(Part):
             ctx.memo[("device",) + key] = plan
         return plan
 
-    def forward(self, x, ctx, cache, state=None, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+    def forward(self, x, ctx, cache, state=None, residual: Optional[torch.Tensor] = None, hand_on=None):
         rt, nh, nkv, d = self.rt, self.nh, self.nkv, self.d
         n = x.shape[0]
         nq = nh * d
@@ -180,7 +181,7 @@ class PagedAttention(Part):
             part_ml = rt.buffer("attn.dec_part_ml", (n * p_max * nkv * 32,), torch.float32)
             ops.attention_bf16_decode_fused(qkv, cos, sin, cache.k, cache.v, cache.block_table, ctx.entry_pos0,
                                             chunk, p_max, out, part_o, part_ml, nh, nkv, d, self.window, self.scale)
-            return linear(rt, out, self.w_o, self.b_o, "attn.o", packed=self.p_o, residual=residual)
+            return linear(rt, out, self.w_o, self.b_o, "attn.o", packed=self.p_o, residual=residual, hand_on=hand_on)
         q = rt.buffer("attn.q", (n, nq), rt.dtype)
         ops.rope_store(qkv, cos, sin, ctx.positions, ctx.tok_entry, cache.block_table, q, cache.k, cache.v, nh, nkv, d,
                        write_kv=cache.writes)
@@ -205,4 +206,4 @@ class PagedAttention(Part):
                                          out, nh, nkv, d, self.window, self.scale, rt=plan.tile_rt,
                                          citems=plan.tile_citems, n_citems=plan.n_tile_citems,
                                          part_o=plan.tile_part_o, part_ml=plan.tile_part_ml, n_parts=plan.n_tile_parts)
-        return linear(rt, out, self.w_o, self.b_o, "attn.o", packed=self.p_o, residual=residual)
+        return linear(rt, out, self.w_o, self.b_o, "attn.o", packed=self.p_o, residual=residual, hand_on=hand_on)

@@ -150,10 +150,18 @@ class Runtime:
 class NormedInput:
     """What a block hands to a mixer or feed-forward that says it `takes_normed_input`: the residual stream and the
     norm that is to be applied to it, not yet applied, so that the part's first matrix product can do it on the way
-    (few rows in bfloat16).  `materialize()` is the norm as a kernel of its own, for whoever cannot."""
+    (few rows in bfloat16).  `materialize()` is the norm as a kernel of its own, for whoever cannot.
 
-    def __init__(self, h: torch.Tensor, norm):
-        self.h, self.norm = h, norm
+    The product in front of the norm may have `prepared` it (a part that `hands_norm_on`): beside adding its result
+    to the stream it has written `xn` = bfloat16(h * gain) and `ssq`, its blocks' shares of the rows' sums of squares,
+    so that the product behind the norm reads bfloat16 tokens and only divides its sums by the norm's root."""
+
+    def __init__(self, h: torch.Tensor, norm, xn: Optional[torch.Tensor] = None, ssq: Optional[torch.Tensor] = None):
+        self.h, self.norm, self.xn, self.ssq = h, norm, xn, ssq
+
+    @property
+    def prepared(self) -> bool:
+        return self.xn is not None
 
     @property
     def shape(self):

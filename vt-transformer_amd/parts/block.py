@@ -10,7 +10,10 @@ their own: a mixer or feed-forward that says so takes the residual stream with
 the norm still to be applied (`NormedInput`: its first matrix product applies
 it) and adds its result to the stream itself (`residual=`: its last matrix
 product does; `adds_residual(rows)` says for how many rows it can, which reaches
-up to 64 for matrices that fill the GPU without splitting k over blocks).
+up to 64 for matrices that fill the GPU without splitting k over blocks).  A part
+that `hands_norm_on` is also told which norm comes behind it (`hand_on=`) and
+may return that norm prepared (a NormedInput with `xn` and `ssq`), which the
+part behind the norm then takes as its input.
 """
 from __future__ import annotations
 
@@ -20,13 +23,13 @@ import torch
 
 from .base import BLOCKS, NormedInput, Part, Runtime
 from .linear import can_fuse
-from .norm import RMSNorm
 
 
 @BLOCKS.register("prenorm")
 class PreNormBlock(Part):
     norm_roles = ("input", "post_mixer")
     replayable = True
+    takes_next_norm = True      # forward(..., next_norm=): the norm that the layer behind this one starts with
 
     def __init__(self, *, rt: Runtime, norms, mixer, feed_forward):
         self.rt = rt
@@ -38,20 +41,34 @@ class PreNormBlock(Part):
     def parts(self):
         return [self.norm_in, self.mixer, self.norm_post, self.feed_forward]
 
-    def forward(self, h: torch.Tensor, delta: Optional[torch.Tensor], ctx, cache, state) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    @property
+    def first_norm(self):
+        """The norm that this layer applies to the stream it is given (what the layer in front may prepare)."""
+        return self.norm_in
+
+    def forward(self, h: torch.Tensor, delta, ctx, cache, state, next_norm=None) -> Tuple[torch.Tensor, object]:
+        """delta: what is still to be added to h (a tensor), None, or this layer's first norm as the layer in front
+        has prepared it (a NormedInput; its addition is done).  Returns (h, delta) in the same terms."""
         fuse = can_fuse(self.rt, h.shape[0]) and h.shape[1] % 8 == 0
-        y = self._run(self.mixer, self.norm_in, h, delta, fuse, ctx, cache, state)
-        z = self._run(self.feed_forward, self.norm_post, h, y, fuse, ctx)
+        y = self._run(self.mixer, self.norm_in, h, delta, fuse, self.norm_post, ctx, cache, state)
+        z = self._run(self.feed_forward, self.norm_post, h, y, fuse, next_norm, ctx)
         return h, z
 
-    def _run(self, part, norm, h, delta, fuse, *args):
-        """norm (of h + delta), then the part; returns what is still to be added to h (None: the part added it)."""
-        if fuse and delta is None and isinstance(norm, RMSNorm) and getattr(part, "takes_normed_input", False):
+    def _run(self, part, norm, h, delta, fuse, norm_behind, *args):
+        """norm (of h + delta), then the part; returns what is still to be added to h (None: the part added it; a
+        NormedInput: it added it and prepared `norm_behind`)."""
+        takes = getattr(part, "takes_normed_input", False)
+        if isinstance(delta, NormedInput):
+            x = delta if (delta.norm is norm and takes) else norm.forward(h, None)
+        elif fuse and delta is None and getattr(norm, "rms_fusable", False) and takes:
             x = NormedInput(h, norm)
         else:
             x = norm.forward(h, delta)
         adds = getattr(part, "adds_residual", None)
         if adds is not None and adds(h.shape[0]):
+            if norm_behind is not None and getattr(part, "hands_norm_on", False):
+                r = part.forward(x, *args, residual=h, hand_on=norm_behind)
+                return r if isinstance(r, NormedInput) else None
             part.forward(x, *args, residual=h)
             return None
         return part.forward(x, *args)

@@ -53,25 +53,28 @@ class GatedMLP(Part):
         self.w_gu, self.w_down = rt.row_major(self.w_gu, self.p_gu), rt.row_major(self.w_down, self.p_down)
 
     takes_normed_input = True     # the gate/up product applies the norm in front of it when the rows are few
+    hands_norm_on = True          # ... and the down product prepares the norm behind it
 
     def adds_residual(self, rows: int) -> bool:
         """Whether the down product adds to the residual stream itself at this many rows."""
         return can_add_residual(self.rt, rows, self.width, self.inter)
 
-    def forward(self, x, ctx=None, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+    def forward(self, x, ctx=None, residual: Optional[torch.Tensor] = None, hand_on=None):
         rt = self.rt
         n = x.shape[0]
         act = rt.buffer("mlp.act", (n, self.inter), rt.dtype)
         normed = isinstance(x, NormedInput)
-        if normed and not (can_fuse(rt, n) and self.width % 8 == 0):
+        if normed and not (can_fuse(rt, n) and self.width % 8 == 0 and (self.p_gu is not None or not x.prepared)):
             x, normed = x.materialize(), False
         if rt.dtype == torch.bfloat16 and (n <= SKINNY_MAX_ROWS or (self.w_gu is None and (rt.keep_row_major or n < UNPACK_MIN_ROWS))):
             w = self.p_gu if self.p_gu is not None else self.w_gu
-            if normed:
+            if normed and x.prepared:
+                ops.gated_linear_bf16_link(x.xn, w, act, x.ssq, x.eps)
+            elif normed:
                 ops.gated_linear_bf16(x.h, w, act, norm_gain=x.gain, norm_eps=x.eps)
             else:
                 ops.gated_linear_bf16(x, w, act)
         else:
             gu = linear(rt, x, self.w_gu, None, "mlp.gu", packed=self.p_gu if self.w_gu is None else None)
             ops.silu_mul(gu, act)
-        return linear(rt, act, self.w_down, None, "mlp.down", packed=self.p_down, residual=residual)
+        return linear(rt, act, self.w_down, None, "mlp.down", packed=self.p_down, residual=residual, hand_on=hand_on)

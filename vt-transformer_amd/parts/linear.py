@@ -50,16 +50,23 @@ def can_add_residual(rt: Runtime, n: int, m: int, k: int) -> bool:
     return rt.dtype == torch.bfloat16 and ops.linear_bf16_adds_residual(n, m, k)
 
 
+def can_hand_norm_on(rt: Runtime, n: int, m: int, k: int) -> bool:
+    """Whether the product of n rows with W [m, k], adding to the residual stream, can prepare the norm behind it."""
+    return rt.dtype == torch.bfloat16 and n <= FUSE_MAX_ROWS and ops.linear_bf16_link_shares(n, m, k) > 0
+
+
 def linear(rt: Runtime, x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], name: str,
            out_dtype: Optional[torch.dtype] = None, bias_lowp: Optional[torch.Tensor] = None,
-           packed=None, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+           packed=None, residual: Optional[torch.Tensor] = None, hand_on=None):
     """x [N, K] in the runtime's dtype -> [N, M].  `name` keys the output's scratch buffer.
     Output dtype: float32 from the hand-written kernels unless `out_dtype` says otherwise; the
     library path returns bfloat16 (its bias, if any, is `bias_lowp`, the same values in bfloat16).
     packed: W as rt.pack(w) made it, for the few-row kernel (made on the spot if missing: slow).
     x may be a NormedInput (the norm then happens inside the few-row kernel, or before the product as a kernel of
     its own where that is not possible).  residual (float32 [N, M]): the product is added to it in place and
-    `residual` is returned (by the product's kernel where `can_add_residual` says so, else by a kernel after it)."""
+    `residual` is returned (by the product's kernel where `can_add_residual` says so, else by a kernel after it).
+    hand_on (with residual): the norm that comes behind this product (`rms_fusable`); where the kernel can, it
+    prepares that norm on its way and a prepared NormedInput is returned instead of `residual`."""
     n, k = x.shape
     m = w.shape[0] if w is not None else packed.rows * packed.halves   # (no row-major copy: the runtime keeps the packed one only)
     if residual is not None or isinstance(x, NormedInput):
@@ -68,7 +75,25 @@ def linear(rt: Runtime, x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.T
         if isinstance(x, NormedInput) or can_add_residual(rt, n, m, k):
             norm = x if isinstance(x, NormedInput) else None
             out = residual if residual is not None else rt.buffer(name, (n, m), torch.float32)
-            return ops.linear_bf16(norm.h if norm else x, packed if packed is not None else w, bias, out,
+            w_any = packed if packed is not None else w
+            emits = (hand_on is not None and residual is not None and isinstance(w_any, ops.PackedMatrix)
+                     and getattr(hand_on, "rms_fusable", False) and can_hand_norm_on(rt, n, m, k))
+            if emits or (norm is not None and norm.prepared and isinstance(w_any, ops.PackedMatrix)):
+                if norm is not None and not norm.prepared:
+                    x, norm = norm.materialize(), None     # (a product cannot take the norm in front both ways at once)
+                xn = ssq = None
+                if emits:
+                    xn = rt.buffer(name + ".xn", (n, m), torch.bfloat16)
+                    ssq = rt.buffer(name + ".ssq", (ops.linear_bf16_link_shares(n, m, k), 16), torch.float32)
+                ops.linear_bf16_link(norm.xn if norm else x, w_any, bias, out, residual=residual,
+                                     ssq_in=norm.ssq if norm else None, eps_in=norm.eps if norm else 0.0,
+                                     xn_out=xn, gain_next=hand_on.gain if emits else None, ssq_out=ssq)
+                return NormedInput(out, hand_on, xn, ssq) if emits else out
+            if norm is not None and norm.prepared:
+                x, norm = norm.materialize(), None
+                if not can_add_residual(rt, n, m, k) and residual is not None:
+                    return ops.residual_add(residual, linear(rt, x, w, bias, name, out_dtype, bias_lowp, packed))
+            return ops.linear_bf16(norm.h if norm else x, w_any, bias, out,
                                    norm_gain=norm.gain if norm else None, norm_eps=norm.eps if norm else 0.0,
                                    residual=residual)
         if residual is not None:

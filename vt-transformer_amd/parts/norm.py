@@ -19,6 +19,9 @@ from .base import NORMS, Part, Runtime, TensorDecl
 @NORMS.register("rmsnorm")
 class RMSNorm(Part):
     replayable = True
+    # out = (gain * x) / sqrt(mean(x^2) + eps) with `gain` and `eps` as attributes: a matrix product can apply it on
+    # the way (NormedInput); any norm of that form may say so
+    rms_fusable = True
 
     def __init__(self, *, rt: Runtime, width: int, prefix: str, eps: float, name: str = "weight", scratch: str = "norm"):
         self.rt = rt
