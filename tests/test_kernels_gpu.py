@@ -163,7 +163,7 @@ def test_linear_bf16_split_k_needs_and_uses_a_workspace():
 def test_linear_bf16_adds_to_a_residual_up_to_64_rows(n, m, k):
     """17 to 64 rows: whole k in a block (two or four token tiles, one or two tile rows of W; 4,100 rows leave the
     last block's second tile row beyond the matrix), the result added to a residual in place; shapes for which the
-    kernel that splits k over blocks is the faster one refuse a residual."""
+    kernel that splits k over blocks is the faster one add the residual in the launch that adds the partial sums."""
     g = torch.Generator().manual_seed(83)
     x = torch.randn(n, k, generator=g).to(torch.bfloat16)
     w = (torch.randn(m, k, generator=g) * 0.05).to(torch.bfloat16)
@@ -171,11 +171,16 @@ def test_linear_bf16_adds_to_a_residual_up_to_64_rows(n, m, k):
     res = torch.randn(n, m, generator=g)
     h = res.to(DEV)
     if not ops().linear_bf16_adds_residual(n, m, k):
-        assert n > 32 and k > 3000
+        assert n > 32 and k > 3000 and m % 4         # k split over blocks, and rows that the adding launch cannot take by fours
         with pytest.raises(ops().KernelError, match="residual"):
             ops().linear_bf16(x.to(DEV), w.to(DEV), b.to(DEV), h, residual=h)
         return
-    out = ops().linear_bf16(x.to(DEV), w.to(DEV), b.to(DEV), h, residual=h)
+    need = ops().linear_bf16_workspace(n, m, k)
+    work = torch.full((need,), float("nan"), device=DEV) if need else None
+    if need:
+        with pytest.raises(ops().KernelError, match="workspace"):
+            ops().linear_bf16(x.to(DEV), w.to(DEV), b.to(DEV), h, residual=h)
+    out = ops().linear_bf16(x.to(DEV), w.to(DEV), b.to(DEV), h, work, residual=h)
     assert out is h
     assert rel_err(h, res.double() + x.double() @ w.double().t() + b.double()) < 2e-5
     with pytest.raises(ops().KernelError, match="residual"):
@@ -189,7 +194,7 @@ def test_linear_bf16_says_which_shapes_take_a_residual():
     assert not o.linear_bf16_adds_residual(8, 50, 53)            # k no multiple of 8: the any-shape kernel
     assert o.linear_bf16_adds_residual(64, 3584, 3584)           # 224 tile rows: one block each, whole k
     assert o.linear_bf16_adds_residual(64, 4608, 3584)           # 288 tile rows: two per block
-    assert not o.linear_bf16_adds_residual(64, 3584, 18944)      # a long k at 64 rows: split over blocks is faster
+    assert o.linear_bf16_adds_residual(64, 3584, 18944)          # a long k at 64 rows: split over blocks, and the launch that adds up adds the residual
     assert not o.linear_bf16_adds_residual(64, 152064, 3584)     # many rows: nothing to split
     assert not o.linear_bf16_adds_residual(65, 3584, 3584)
 
@@ -689,13 +694,16 @@ def test_random_normal_kernel_makes_the_hosts_bits(dtype, n, first):
         assert torch.equal(out.cpu(), want), (key, mean)
 
 
-@pytest.mark.parametrize("n", [1, 5, 8, 16])
+@pytest.mark.parametrize("n", [1, 5, 8, 16, 17, 33, 64])
 @pytest.mark.parametrize("h,k1,m2,gated", [(3584, 3584, 4608, False), (3584, 18944, 1184, True), (200, 96, 320, False),
-                                           (1536, 8960, 2048, False), (8192, 512, 640, True), (72, 40, 56, True)])
+                                           (1536, 8960, 2048, False), (8192, 512, 640, True), (72, 40, 56, True),
+                                           (3584, 18944, 10240, False)])
 def test_rmsnorm_handed_from_one_product_to_the_next(n, h, k1, m2, gated):
     """A product that adds to the residual stream prepares the norm behind it (the stream times the gains in
     bfloat16, its blocks' shares of the rows' sums of squares); the product behind the norm takes those as its
-    tokens and divides by the root.  Against the plain chain: add, RMSNorm, product."""
+    tokens and divides by the root.  Against the plain chain: add, RMSNorm, product.  Up to 16 rows a block per tile
+    row produces; from 17 to 64 the kernel that keeps k inside a block, or the launch that adds the partial sums of a
+    split k."""
     o = ops()
     g = torch.Generator().manual_seed(n * 1000 + h)
     x = (torch.randn(n, k1, generator=g) * 0.5).to(torch.bfloat16)
@@ -705,13 +713,17 @@ def test_rmsnorm_handed_from_one_product_to_the_next(n, h, k1, m2, gated):
     gain = 1.0 + 0.1 * torch.randn(h, generator=g)
     w2 = (torch.randn((2 if gated else 1) * m2, h, generator=g) * 0.05).to(torch.bfloat16)
     eps = 1e-5
-    shares = o.linear_bf16_link_shares(n, h, k1)
-    assert shares == (h + 15) // 16
+    shares, stride = o.linear_bf16_link_shares(n, h, k1), o.link_stride(n)
+    assert shares > 0 and o.linear_bf16_adds_residual(n, h, k1)
+
+    def workspace(rows, m, k):
+        need = o.linear_bf16_workspace(rows, m, k) if rows > 16 else 0
+        return torch.full((need,), float("nan"), device=DEV) if need else None
     hbuf = resid.clone().to(DEV)
     xn = torch.full((n, h), float("nan"), dtype=torch.bfloat16, device=DEV)
-    ssq = torch.full((shares, 16), float("nan"), dtype=torch.float32, device=DEV)
+    ssq = torch.full((shares, stride), float("nan"), dtype=torch.float32, device=DEV)
     o.linear_bf16_link(x.to(DEV), o.pack_matrix_bf16(w1.to(DEV)), bias1.to(DEV), hbuf, residual=hbuf, xn_out=xn,
-                       gain_next=gain.to(DEV), ssq_out=ssq)
+                       gain_next=gain.to(DEV), ssq_out=ssq, workspace=workspace(n, h, k1))
     h_ref = resid.double() + x.double() @ w1.double().t() + bias1.double()
     assert rel_err(hbuf, h_ref) < 1e-5
     assert rel_err(ssq[:, :n].sum(dim=0), (h_ref * h_ref).sum(dim=1)) < 1e-5
@@ -727,11 +739,12 @@ def test_rmsnorm_handed_from_one_product_to_the_next(n, h, k1, m2, gated):
     else:
         bias2 = torch.randn(m2, generator=g) * 0.1
         out = torch.empty(n, m2, dtype=torch.float32, device=DEV)
-        o.linear_bf16_link(xn, o.pack_matrix_bf16(w2.to(DEV)), bias2.to(DEV), out, ssq_in=ssq, eps_in=eps)
+        o.linear_bf16_link(xn, o.pack_matrix_bf16(w2.to(DEV)), bias2.to(DEV), out, ssq_in=ssq, eps_in=eps,
+                           workspace=workspace(n, m2, h))
         ref = normed @ w2.double().t() + bias2.double()
     assert rel_err(out, ref) < 3e-5
-    # and the same bits as the product that applies the norm itself from the float32 stream
-    if gated:
+    # and, up to 16 rows, the same as the product that applies the norm itself from the float32 stream
+    if gated and n <= 16:
         same = torch.empty(n, m2, dtype=torch.float32, device=DEV)
         o.gated_linear_bf16(hbuf, o.pack_matrix_bf16(w2.to(DEV), halves=2), same, norm_gain=gain.to(DEV), norm_eps=eps)
         assert rel_err(out, same) < 2e-6
@@ -739,12 +752,15 @@ def test_rmsnorm_handed_from_one_product_to_the_next(n, h, k1, m2, gated):
 
 def test_rmsnorm_hand_over_is_refused_where_it_cannot_work():
     o = ops()
-    assert o.linear_bf16_link_shares(17, 3584, 3584) == 0        # more than 16 rows
+    assert o.linear_bf16_link_shares(65, 3584, 3584) == 0        # more than 64 rows
     assert o.linear_bf16_link_shares(8, 3584, 100) == 0          # k no multiple of 8
     assert o.linear_bf16_link_shares(8, 100, 64) == 0            # a width that the next product could not read by 16 bytes
-    x = torch.zeros(17, 64, dtype=torch.bfloat16, device=DEV)
+    assert o.linear_bf16_link_shares(64, 152064, 3584) == 0      # many rows at 64 tokens: neither whole k in a block nor a split
+    assert o.linear_bf16_link_shares(64, 3584, 18944) == 4       # k split over blocks: the adding launch, a share per 1,024 columns
+    assert o.linear_bf16_link_shares(64, 3584, 3584) == 224 and o.linear_bf16_link_shares(64, 4608, 3584) == 144
+    x = torch.zeros(65, 64, dtype=torch.bfloat16, device=DEV)
     w = o.pack_matrix_bf16(torch.zeros(32, 64, dtype=torch.bfloat16, device=DEV))
-    out = torch.zeros(17, 32, device=DEV)
-    ssq = torch.zeros(4, 16, device=DEV)
-    with pytest.raises(Exception, match="up to 16 rows"):
+    out = torch.zeros(65, 32, device=DEV)
+    ssq = torch.zeros(4, 64, device=DEV)
+    with pytest.raises(Exception, match="up to 64 rows"):
         o.linear_bf16_link(x, w, None, out, ssq_in=ssq, eps_in=1e-6)

@@ -37,7 +37,7 @@ int vt_linear_bf16_noalloc(const void* x, const void* wp, const float* bias, voi
                            int N, int M, int K, hipStream_t stream);
 
 int vt_linear_bf16_fused(const void* h, const float* gain, float eps, const void* wp, const float* bias,
-                         const float* resid, float* y, int N, int M, int K, hipStream_t stream);
+                         const float* resid, float* y, float* workspace, int N, int M, int K, hipStream_t stream);
 int vt_gated_linear_bf16(const void* x, const void* wp, void* y, int out_dtype, int N, int I, int K,
                          const float* gain, float eps, hipStream_t stream);
 
@@ -46,8 +46,8 @@ int vt_gated_linear_bf16(const void* x, const void* wp, void* y, int out_dtype, 
 // behind it (which reads those as its tokens and divides its sums by the norm's root): see vt_gemm_bf16.hip.
 int vt_linear_bf16_link_shares(int N, int M, int K);
 int vt_linear_bf16_link(const void* x, const void* wp, const float* bias, const float* resid, float* y,
-                        int N, int M, int K, const float* ssq_in, int n_ssq, float eps_in, void* xn_out,
-                        const float* gain_next, float* ssq_out, hipStream_t stream);
+                        float* workspace, int N, int M, int K, const float* ssq_in, int n_ssq, float eps_in,
+                        void* xn_out, const float* gain_next, float* ssq_out, hipStream_t stream);
 int vt_gated_linear_bf16_link(const void* x, const void* wp, void* y, int out_dtype, int N, int I, int K,
                               const float* ssq_in, int n_ssq, float eps_in, hipStream_t stream);
 

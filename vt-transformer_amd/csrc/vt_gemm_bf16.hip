@@ -144,6 +144,40 @@ struct NormLink {
 };
 #define SSQ_STRIDE(N) ((N) <= 16 ? 16 : 64)
 
+// Consumer of a NormLink at 17 to 64 rows (shares 64 floats apart): 1/sqrt(sum / K + eps) of every row into
+// rinv[64], by all THREADS of the block.  Thread t adds rows 4 (t % 16) .. + 3 of shares t / 16, t / 16 + THREADS / 16,
+// ... in that order (eight loads in flight at a time), the four lanes of a wave with the same rows add up, then the
+// waves in wave order: a fixed order, whatever finished first.  part: [THREADS / 64][16]; ends with a barrier.
+template <int THREADS>
+__device__ __forceinline__ void link_row_scales(const NormLink& link, int K, float4 (*part)[16], float* rinv) {
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    float4 sh = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int b0 = tid >> 4; b0 < link.n_ssq; b0 += 8 * (THREADS / 16)) {
+        float4 t4[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {       // eight loads asked for together, then added in order
+            const int b = b0 + j * (THREADS / 16);
+            t4[j] = b < link.n_ssq ? *(const float4*)(link.ssq_in + (size_t)b * 64 + (tid & 15) * 4)
+                                   : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) { sh.x += t4[j].x; sh.y += t4[j].y; sh.z += t4[j].z; sh.w += t4[j].w; }
+    }
+#pragma unroll
+    for (int o = 16; o < 64; o <<= 1) {
+        sh.x += __shfl_xor(sh.x, o, 64); sh.y += __shfl_xor(sh.y, o, 64);
+        sh.z += __shfl_xor(sh.z, o, 64); sh.w += __shfl_xor(sh.w, o, 64);
+    }
+    if (lane < 16) part[wv][lane] = sh;
+    __syncthreads();
+    if (tid < 64) {
+        float tot = 0.f;
+        for (int q = 0; q < THREADS / 64; ++q) tot += ((const float*)&part[q][0])[tid];
+        rinv[tid] = 1.0f / sqrtf(tot / (float)K + link.eps);
+    }
+    __syncthreads();
+}
+
 // ---------------------------------------------------------------------------
 // Up to 16 tokens: a block owns one tile row of W (16 features; two for the gated product) and all of k, which
 // its WPB waves split; the tokens are the B operand.  U tiles are in flight per wave and matrix.
@@ -375,12 +409,16 @@ template <int R, bool SWIGLU, int WM, typename TO>
 __global__ __launch_bounds__(WM * 64) void gemm_mid_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wp,
                                                       const float* __restrict__ bias, TO* __restrict__ y,
                                                       float* __restrict__ partial, int N, int Mout, int K, int KT,
-                                                      int up_tiles, int k_per_split) {
+                                                      int up_tiles, int k_per_split, NormLink link) {
     constexpr int NW = SWIGLU ? 2 : 1;
     constexpr int RW = R * NW;
     __shared__ __attribute__((aligned(16))) bf16_t xs[2][64][MID_XROW];
+    __shared__ float4 link_part[WM][16];
+    __shared__ float link_rinv[64];
     const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63;
     const int r = lane & 15, g = lane >> 4;
+    // behind a norm that the product in front has prepared (up to 64 tokens): the rows' 1/sqrt(mean + eps)
+    const bool consumes = link.ssq_in != nullptr;
     constexpr int MID_XP = (MID_PIECES + WM * 64 - 1) / (WM * 64);  // pieces of x per thread and stage
     const int mt0 = (blockIdx.x * WM + wv) * R, n0 = blockIdx.y * 64;
     const int k_begin = blockIdx.z * k_per_split, k_end = min(pk_cols(K), k_begin + k_per_split);
@@ -448,6 +486,8 @@ __global__ __launch_bounds__(WM * 64) void gemm_mid_kernel(const bf16_t* __restr
         // x first: loads finish in the order they were issued, and parking x must not wait for W
         fetch_x(k_begin);
         fetch_w(wcur, k_begin);
+        // (here, behind the first stage's loads, the shares' way from the second-level cache costs nothing)
+        if (consumes) link_row_scales<WM * 64>(link, K, link_part, link_rinv);
         park_x(0);
         __syncthreads();
         // two stages per turn so that the register buffers alternate without copies
@@ -465,6 +505,8 @@ __global__ __launch_bounds__(WM * 64) void gemm_mid_kernel(const bf16_t* __restr
         }
     }
 
+    else if (consumes) link_row_scales<WM * 64>(link, K, link_part, link_rinv);
+
     // acc[a][i][e] is feature 16 (mt0 + j) + 4 g + e (j = a mod R) of token n0 + 16 i + r
     const bool split = gridDim.z > 1;
 #pragma unroll
@@ -477,8 +519,10 @@ __global__ __launch_bounds__(WM * 64) void gemm_mid_kernel(const bf16_t* __restr
                 const int m = (mt0 + j) * 16 + 4 * g + e;
                 if (m >= Mout || n >= N) continue;
                 float v = acc[j][i][e];
+                if (consumes) v *= link_rinv[i * 16 + r];
                 if (SWIGLU) {
-                    const float u = acc[R + j][i][e];
+                    float u = acc[R + j][i][e];
+                    if (consumes) u *= link_rinv[i * 16 + r];
                     v = v / (1.f + expf(-v)) * u;
                 } else if (bias && blockIdx.z == 0) {
                     v += bias[m];
@@ -508,14 +552,21 @@ __host__ __device__ constexpr int rows_lds_bytes() {
     return exchange > sums ? exchange : sums;
 }
 
+// (The exchange buffers leave room for two blocks of 8 waves per compute unit: four waves per SIMD.  Saying so keeps
+// the compiler from giving up loads in flight for a fifth and sixth wave that can never come.)
 template <int WPB, int NT, int R, typename TO>
-__global__ __launch_bounds__(WPB * 64) void gemm_rows_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wp,
+__global__ __launch_bounds__(WPB * 64) __attribute__((amdgpu_waves_per_eu(2, 4))) void gemm_rows_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wp,
                                                             const float* __restrict__ bias, TO* __restrict__ y, int N,
-                                                            int Mout, int K, int KT, const float* resid) {
+                                                            int Mout, int K, int KT, const float* resid, NormLink link) {
     extern __shared__ __attribute__((aligned(16))) unsigned char rows_lds[];
+    __shared__ float4 link_part[WPB][16];
+    __shared__ float link_rinv[64];
     const int tid = threadIdx.x, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = tid & 63;
     const int r = lane & 15, g = lane >> 4;
     const int m_tiles = (Mout + 15) >> 4;
+    const bool consumes = link.ssq_in != nullptr;
+    if (consumes) link_row_scales<WPB * 64>(link, K, link_part, link_rinv);
+    float ssq_acc = 0.f;        // producer: row tid's sum of squares over this block's features
     // the waves split k in pairs of tiles (KT is a multiple of 4): a token's 64 values of a pair are one cache line
     const int KP = KT >> 1;
     const int p_begin = (int)(((long long)wv * KP) / WPB), p_end = (int)(((long long)(wv + 1) * KP) / WPB);
@@ -587,20 +638,36 @@ __global__ __launch_bounds__(WPB * 64) void gemm_rows_kernel(const bf16_t* __res
         for (int c = tid; c < NT * 256; c += WPB * 64) {
             const int i = c >> 8, cc = c & 255, ln = cc >> 2, e = cc & 3;
             const int m = mt * 16 + 4 * (ln >> 4) + e, n = 16 * i + (ln & 15);
-            float v = 0.f;
+            float v = 0.f, sq = 0.f;
             for (int q = 0; q < WPB; ++q) v += red[((size_t)q * NT + i) * 256 + cc];
             if (m < Mout && n < N) {
+                if (consumes) v *= link_rinv[n];
                 if (bias) v += bias[m];
                 if (resid) v += resid[(size_t)n * Mout + m];
                 store_f32<TO>(y, (size_t)n * Mout + m, v);
+                if (link.xn_out) {
+                    link.xn_out[(size_t)n * Mout + m] = f32_to_bf16(v * link.gain_next[m]);
+                    sq = v * v;
+                }
+            }
+            if (link.xn_out) red[(size_t)i * 256 + cc] = sq;       // (this thread alone has read slot cc of tile i)
+        }
+        if (link.xn_out) {
+            // this tile row's share of the rows' sums of squares: 16 features per row, added in feature order
+            __syncthreads();
+            if (tid < NT * 16) {
+                const int i = tid >> 4, nn = tid & 15;
+                for (int gg = 0; gg < 4; ++gg)
+                    for (int e = 0; e < 4; ++e) ssq_acc += red[(size_t)i * 256 + (((gg * 16 + nn) << 2) + e)];
             }
         }
     }
+    if (link.xn_out && tid < 64) link.ssq_out[(size_t)blockIdx.x * 64 + tid] = tid < NT * 16 ? ssq_acc : 0.f;
 }
 
 template <int WPB, int NT, int R, typename TO>
 static int launch_rows(const bf16_t* x, const bf16_t* wp, const float* bias, TO* y, int N, int Mout, int K, int KT,
-                       const float* resid, hipStream_t stream) {
+                       const float* resid, hipStream_t stream, const NormLink& link) {
     constexpr int lds = rows_lds_bytes<WPB, NT>();
     static bool set = false;
     if (!set) {
@@ -610,7 +677,7 @@ static int launch_rows(const bf16_t* x, const bf16_t* wp, const float* bias, TO*
         set = true;
     }
     const int m_tiles = (Mout + 15) / 16;
-    gemm_rows_kernel<WPB, NT, R, TO><<<(m_tiles + R - 1) / R, WPB * 64, lds, stream>>>(x, wp, bias, y, N, Mout, K, KT, resid);
+    gemm_rows_kernel<WPB, NT, R, TO><<<(m_tiles + R - 1) / R, WPB * 64, lds, stream>>>(x, wp, bias, y, N, Mout, K, KT, resid, link);
     VT_CHECK_LAUNCH("vt_linear_bf16(rows)");
     return 0;
 }
@@ -633,6 +700,46 @@ __global__ void sum_partials_kernel(const float* __restrict__ partial, TO* __res
             for (int s = 1; s < splits; ++s) a += partial[(size_t)s * n + j];
             store_f32<TO>(y, j, a);
         }
+    }
+}
+
+// The same for up to 64 rows with a residual to add to, row by row: block (c, n) adds up columns 1024 c .. + 1023 of
+// row n (four per thread), adds the residual, and as the producer of a NormLink writes bf16(y * gain) and the share
+// c of row n's sum of squares (rows from N to 63: zero).
+#define SUM_COLS 1024
+__global__ __launch_bounds__(256) void sum_partials_rows_kernel(const float* __restrict__ partial, float* __restrict__ y,
+                                                                const float* resid, int N, int M, int splits,
+                                                                NormLink link) {
+    __shared__ float red[4];
+    const int n = blockIdx.y, tid = threadIdx.x, col = (blockIdx.x * 256 + tid) * 4;
+    if (n >= N) {
+        if (link.xn_out && tid == 0) link.ssq_out[(size_t)blockIdx.x * 64 + n] = 0.f;
+        return;
+    }
+    float sq = 0.f;
+    if (col < M) {          // (M is a multiple of 4)
+        const size_t at = (size_t)n * M + col, all = (size_t)N * M;
+        float4 a = *(const float4*)(partial + at);
+        for (int s = 1; s < splits; ++s) {
+            const float4 b = *(const float4*)(partial + (size_t)s * all + at);
+            a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+        }
+        if (resid) {
+            const float4 h = *(const float4*)(resid + at);
+            a.x += h.x; a.y += h.y; a.z += h.z; a.w += h.w;
+        }
+        *(float4*)(y + at) = a;
+        if (link.xn_out) {
+            const float4 gg = *(const float4*)(link.gain_next + col);
+            *(uint2*)(link.xn_out + at) = make_uint2(pack_bf16x2(a.x * gg.x, a.y * gg.y), pack_bf16x2(a.z * gg.z, a.w * gg.w));
+            sq = (a.x * a.x + a.y * a.y) + (a.z * a.z + a.w * a.w);
+        }
+    }
+    if (link.xn_out) {
+        sq = wave_sum(sq);
+        if ((tid & 63) == 0) red[tid >> 6] = sq;
+        __syncthreads();
+        if (tid == 0) link.ssq_out[(size_t)blockIdx.x * 64 + n] = (red[0] + red[1]) + (red[2] + red[3]);
     }
 }
 
@@ -722,7 +829,9 @@ static int rows_tile_rows(int N, int Mout, int K) {
 // whether a plain product of N rows keeps all of k inside a block, so that it can add its result to a residual
 extern "C" int vt_linear_bf16_adds_residual(int N, int M, int K) {
     if (N <= 0 || M <= 0 || K <= 0 || K % 8 != 0) return 0;
-    return N <= 16 || rows_tile_rows(N, M, K) > 0;
+    if (N <= 16 || rows_tile_rows(N, M, K) > 0) return 1;
+    // 17 to 64 rows with k split over blocks: the launch that adds the partial sums adds the residual too
+    return N <= ROWS_MAX && M % 4 == 0 && mid_splits(M, K, 128) > 1;
 }
 
 extern "C" long long vt_linear_bf16_workspace(int N, int M, int K, int gated) {
@@ -739,8 +848,13 @@ static const NormLink NO_LINK = {nullptr, nullptr, nullptr, nullptr, 0, 0.f};
 
 // shares of the rows' sums of squares that a producing product of this shape writes (0: it cannot produce)
 extern "C" int vt_linear_bf16_link_shares(int N, int M, int K) {
-    if (N <= 0 || N > 16 || M <= 0 || K <= 0 || K % 8 != 0 || M % 8 != 0) return 0;
-    return (M + 15) / 16;
+    if (N <= 0 || N > ROWS_MAX || M <= 0 || K <= 0 || K % 8 != 0 || M % 8 != 0) return 0;
+    const int tiles = (M + 15) / 16;
+    if (N <= 16) return tiles;                                          // a block per tile row
+    const int rr = rows_tile_rows(N, M, K);
+    if (rr) return (tiles + rr - 1) / rr;                               // a block per rr tile rows, whole k
+    if (mid_splits(M, K, 128) > 1) return (M + SUM_COLS - 1) / SUM_COLS; // the launch that adds the partial sums
+    return 0;
 }
 
 template <bool SWIGLU, typename TO>
@@ -749,8 +863,8 @@ static int linear_bf16(const void* xv, const bf16_t* wp, const float* bias, TO* 
                        const NormLink& link = NO_LINK) {
     if (N == 0) return 0;
     const bool linked = link.xn_out || link.ssq_in;
-    VT_REQUIRE(!linked || (N <= 16 && K % 8 == 0 && (((uintptr_t)xv) & 15) == 0 && !gain),
-               "vt_linear_bf16: a norm is handed over between products of up to 16 rows with k a multiple of 8 (N=%d, K=%d)", N, K);
+    VT_REQUIRE(!linked || (N <= ROWS_MAX && K % 8 == 0 && (((uintptr_t)xv) & 15) == 0 && !gain),
+               "vt_linear_bf16: a norm is handed over between products of up to 64 rows with k a multiple of 8 (N=%d, K=%d)", N, K);
     VT_REQUIRE(!link.xn_out || (resid && vt_linear_bf16_link_shares(N, Mout, K) > 0 && link.gain_next && link.ssq_out),
                "vt_linear_bf16: a product that hands a norm on adds to a residual and has gains and room for the sums");
     VT_REQUIRE(!link.ssq_in || (link.n_ssq > 0 && (((uintptr_t)link.ssq_in) & 15) == 0),
@@ -769,11 +883,11 @@ static int linear_bf16(const void* xv, const bf16_t* wp, const float* bias, TO* 
         return 0;
     }
     const int rows_rr = SWIGLU ? 0 : rows_tile_rows(N, Mout, K);
-    VT_REQUIRE(!resid || N <= 16 || rows_rr, "vt_linear_bf16: %d rows of [%d, %d] do not take a residual "
-               "(vt_linear_bf16_adds_residual)", N, Mout, K);
+    VT_REQUIRE(!resid || vt_linear_bf16_adds_residual(N, Mout, K), "vt_linear_bf16: %d rows of [%d, %d] do not take a "
+               "residual (vt_linear_bf16_adds_residual)", N, Mout, K);
     if constexpr (!SWIGLU) {
         // whole k in a block of 8 waves (gemm_rows_kernel)
-#define VT_ROWS(NT, RR) launch_rows<8, NT, RR, TO>(x, wp, bias, y, N, Mout, K, KT, resid, stream)
+#define VT_ROWS(NT, RR) launch_rows<8, NT, RR, TO>(x, wp, bias, y, N, Mout, K, KT, resid, stream, link)
         if (rows_rr == 1) return N <= 32 ? VT_ROWS(2, 1) : VT_ROWS(4, 1);
         if (rows_rr == 2) return N <= 32 ? VT_ROWS(2, 2) : VT_ROWS(4, 2);
 #undef VT_ROWS
@@ -788,7 +902,13 @@ static int linear_bf16(const void* xv, const bf16_t* wp, const float* bias, TO* 
         const int wm = SWIGLU ? mid_waves(Mout, 16 * RR, (N + 63) / 64) : 4;
         dim3 grid((Mout + 16 * wm * RR - 1) / (16 * wm * RR), (N + 63) / 64, splits);
         VT_REQUIRE(grid.y <= 65535, "vt_linear_bf16: too many rows (%d)", N);
-#define VT_MID(W) gemm_mid_kernel<RR, SWIGLU, W, TO><<<grid, W * 64, 0, stream>>>(x, wp, bias, y, workspace, N, Mout, K, KT, up_tiles, kps)
+        VT_REQUIRE(!(resid || link.xn_out) || (splits > 1 && N <= ROWS_MAX && Mout % 4 == 0 && sizeof(TO) == 4),
+                   "vt_linear_bf16: %d rows of [%d, %d] do not take a residual (vt_linear_bf16_adds_residual)", N, Mout, K);
+        VT_REQUIRE(!link.ssq_in || grid.y == 1, "vt_linear_bf16: a prepared norm is taken with up to 64 rows (N=%d)", N);
+        // the product takes the norm in front (link.ssq_in); the one behind is prepared where the sums are added up
+        NormLink in = NO_LINK;
+        in.ssq_in = link.ssq_in; in.n_ssq = link.n_ssq; in.eps = link.eps;
+#define VT_MID(W) gemm_mid_kernel<RR, SWIGLU, W, TO><<<grid, W * 64, 0, stream>>>(x, wp, bias, y, workspace, N, Mout, K, KT, up_tiles, kps, in)
         if (wm == 4) VT_MID(4);
         else if (wm == 5) VT_MID(5);
         else if (wm == 6) VT_MID(6);
@@ -797,6 +917,16 @@ static int linear_bf16(const void* xv, const bf16_t* wp, const float* bias, TO* 
         VT_CHECK_LAUNCH("vt_linear_bf16(64 tokens)");
         if (splits > 1) {
             const size_t n = (size_t)N * Mout;
+            if constexpr (sizeof(TO) == 4) {
+                if (resid || link.xn_out) {
+                    NormLink outl = NO_LINK;
+                    outl.xn_out = link.xn_out; outl.gain_next = link.gain_next; outl.ssq_out = link.ssq_out;
+                    sum_partials_rows_kernel<<<dim3((Mout + SUM_COLS - 1) / SUM_COLS, link.xn_out ? 64 : N), 256, 0, stream>>>(
+                        workspace, (float*)y, resid, N, Mout, splits, outl);
+                    VT_CHECK_LAUNCH("vt_linear_bf16(sum rows)");
+                    return 0;
+                }
+            }
             sum_partials_kernel<TO><<<(unsigned)((n / 4 + 255) / 256 + 1), 256, 0, stream>>>(workspace, y, n, splits);
             VT_CHECK_LAUNCH("vt_linear_bf16(sum)");
         }
@@ -869,25 +999,28 @@ extern "C" int vt_linear_bf16_noalloc(const void* x, const void* wp, const float
 // The same with an RMSNorm in front (up to 16 tokens) and a residual addition behind (up to 64), each optional:
 // gain != null: h is the fp32 residual stream [N, K] and y = (rmsnorm(h; gain, eps) . W^T) + bias, else h is x in bf16;
 // resid != null (fp32 [N, M], may be y): y = resid + that.  y is fp32.
+// workspace: for shapes whose k range is split over blocks (vt_linear_bf16_workspace), else null.
 extern "C" int vt_linear_bf16_fused(const void* h, const float* gain, float eps, const void* wp, const float* bias,
-                                    const float* resid, float* y, int N, int M, int K, hipStream_t stream) {
+                                    const float* resid, float* y, float* workspace, int N, int M, int K, hipStream_t stream) {
     VT_REQUIRE(N >= 0 && M > 0 && K > 0, "vt_linear_bf16_fused: bad sizes N=%d M=%d K=%d", N, M, K);
     VT_REQUIRE(gain || resid, "vt_linear_bf16_fused: neither a norm nor a residual: use vt_linear_bf16");
-    return linear_bf16<false, float>(h, (const bf16_t*)wp, bias, y, nullptr, N, M, K, gain, eps, resid, stream);
+    return linear_bf16<false, float>(h, (const bf16_t*)wp, bias, y, workspace, N, M, K, gain, eps, resid, stream);
 }
 
-// The product between two RMSNorms that are no kernels of their own (up to 16 rows):
-// ssq_in != null: x is xn = bf16(h * gain) as a producing product left it, ssq_in [n_ssq][16] its blocks' shares of the
+// The product between two RMSNorms that are no kernels of their own (up to 64 rows; S = 16 floats up to 16 rows,
+// else 64):
+// ssq_in != null: x is xn = bf16(h * gain) as a producing product left it, ssq_in [n_ssq][S] its blocks' shares of the
 // rows' sums of h^2, and the result is multiplied by 1/sqrt(sum / K + eps_in);
 // xn_out != null (needs resid): beside y = resid + product, xn_out [N][M] = bf16(y * gain_next) and this product's
-// shares ssq_out [vt_linear_bf16_link_shares(N, M, K)][16] are written for the product behind the next norm.
+// shares ssq_out [vt_linear_bf16_link_shares(N, M, K)][S] are written for the product behind the next norm.
+// workspace: as for vt_linear_bf16.
 extern "C" int vt_linear_bf16_link(const void* x, const void* wp, const float* bias, const float* resid, float* y,
-                                   int N, int M, int K, const float* ssq_in, int n_ssq, float eps_in, void* xn_out,
-                                   const float* gain_next, float* ssq_out, hipStream_t stream) {
+                                   float* workspace, int N, int M, int K, const float* ssq_in, int n_ssq, float eps_in,
+                                   void* xn_out, const float* gain_next, float* ssq_out, hipStream_t stream) {
     VT_REQUIRE(N >= 0 && M > 0 && K > 0, "vt_linear_bf16_link: bad sizes N=%d M=%d K=%d", N, M, K);
     VT_REQUIRE(ssq_in || xn_out, "vt_linear_bf16_link: neither end of a norm: use vt_linear_bf16");
     const NormLink link = {(bf16_t*)xn_out, gain_next, ssq_out, ssq_in, n_ssq, eps_in};
-    return linear_bf16<false, float>(x, (const bf16_t*)wp, bias, y, nullptr, N, M, K, nullptr, 0.f, resid, stream, link);
+    return linear_bf16<false, float>(x, (const bf16_t*)wp, bias, y, workspace, N, M, K, nullptr, 0.f, resid, stream, link);
 }
 
 // the gated product behind a norm that the product in front has prepared (x = xn, ssq_in, n_ssq, eps_in as above)

@@ -251,12 +251,14 @@ def linear_bf16_workspace(n: int, m: int, k: int) -> int:
 
 
 NORM_MAX_ROWS = 16         # rows up to which the few-row product applies an RMSNorm in front
+LINK_MAX_ROWS = 64         # rows up to which a product takes a norm that the product in front has prepared
 _adds_residual = {}
 
 
 def linear_bf16_adds_residual(n: int, m: int, k: int) -> bool:
-    """Whether linear_bf16 takes `residual` for x [n, k] and W [m, k]: up to 16 rows always (k a multiple of 8), 17
-    to 64 rows where the kernel that keeps all of k inside a block is the faster one for this W."""
+    """Whether linear_bf16 takes `residual` for x [n, k] and W [m, k]: up to 16 rows always (k a multiple of 8); 17
+    to 64 rows where the kernel that keeps all of k inside a block is the faster one for this W, and where k is split
+    over blocks (the launch that adds the partial sums then adds the residual too)."""
     key = (n, m, k)
     if key not in _adds_residual:
         _adds_residual[key] = bool(load_lib("vt_gemm_bf16").vt_linear_bf16_adds_residual(_i(n), _i(m), _i(k)))
@@ -271,7 +273,8 @@ def linear_bf16(x: torch.Tensor, w, bias: Optional[torch.Tensor], out: torch.Ten
     `workspace` (float32, at least linear_bf16_workspace(n, m, k) elements).
     float32 output: with norm_gain (up to 16 rows), x is the float32 residual stream and rmsnorm(x; gain, eps) is
     what gets multiplied; with residual (where linear_bf16_adds_residual says so; float32 [n, m], may be `out`), out =
-    residual + the product."""
+    residual + the product (17 to 64 rows of a shape whose k range is split: by the launch that adds the partial sums,
+    which needs the workspace)."""
     n, k = x.shape
     if not isinstance(w, PackedMatrix):
         _chk(w, "linear_bf16.w", torch.bfloat16, (w.shape[0], k))
@@ -295,8 +298,13 @@ def linear_bf16(x: torch.Tensor, w, bias: Optional[torch.Tensor], out: torch.Ten
             _chk(norm_gain, "linear_bf16.norm_gain", torch.float32, (k,))
         if residual is not None:
             _chk(residual, "linear_bf16.residual", torch.float32, (n, m))
+        need = linear_bf16_workspace(n, m, k) if n > 16 else 0
+        if need and (workspace is None or workspace.numel() < need):
+            raise KernelError(f"linear_bf16: x [{n}, {k}] with W [{m}, {k}] needs a workspace of {need} floats")
+        if need:
+            _chk(workspace, "linear_bf16.workspace", torch.float32)
         _run(load_lib("vt_gemm_bf16"), "vt_linear_bf16_fused", _ptr(x), _ptr(norm_gain), _f(norm_eps), _ptr(w.data), _ptr(bias),
-             _ptr(residual), _ptr(out), _i(n), _i(m), _i(k), _stream())
+             _ptr(residual), _ptr(out), _ptr(workspace if need else None), _i(n), _i(m), _i(k), _stream())
         return out
     need = linear_bf16_workspace(n, m, k) if n > 16 else 0
     if need:
@@ -322,15 +330,21 @@ def linear_bf16_link_shares(n: int, m: int, k: int) -> int:
     return _link_shares[key]
 
 
+def link_stride(n: int) -> int:
+    """Floats between the shares of the rows' sums of squares that products of n rows write and read."""
+    return 16 if n <= 16 else 64
+
+
 def linear_bf16_link(x: torch.Tensor, w: PackedMatrix, bias: Optional[torch.Tensor], out: torch.Tensor,
                      residual: Optional[torch.Tensor] = None, ssq_in: Optional[torch.Tensor] = None, eps_in: float = 0.0,
                      xn_out: Optional[torch.Tensor] = None, gain_next: Optional[torch.Tensor] = None,
-                     ssq_out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """The few-row product between RMSNorms that are no kernels of their own (up to 16 rows).
-    ssq_in (float32 [shares, 16]): x is bf16(h * gain) as the product in front left it, and the result is divided by
-    the norm's root, which the shares of the rows' sums of squares give (eps_in: the norm's eps).
+                     ssq_out: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The few-row product between RMSNorms that are no kernels of their own (up to 64 rows).
+    ssq_in (float32 [shares, link_stride(n)]): x is bf16(h * gain) as the product in front left it, and the result
+    is divided by the norm's root, which the shares of the rows' sums of squares give (eps_in: the norm's eps).
     xn_out (bfloat16 [n, m]; needs residual): beside out = residual + product, xn_out = bf16(out * gain_next) and this
-    product's own shares ssq_out (float32 [linear_bf16_link_shares(n, m, k), 16]) for the product behind the next norm."""
+    product's own shares ssq_out (float32 [linear_bf16_link_shares(n, m, k), link_stride(n)]) for the product behind
+    the next norm.  workspace: as for linear_bf16."""
     n, k = x.shape
     m = w.rows
     if w.cols != k or w.halves != 1:
@@ -342,11 +356,13 @@ def linear_bf16_link(x: torch.Tensor, w: PackedMatrix, bias: Optional[torch.Tens
         _chk(bias, "linear_bf16_link.bias", torch.float32, (m,))
     if residual is not None:
         _chk(residual, "linear_bf16_link.residual", torch.float32, (n, m))
+        if not linear_bf16_adds_residual(n, m, k):
+            raise KernelError(f"linear_bf16_link: {n} rows of [{m}, {k}] do not take a residual (linear_bf16_adds_residual)")
     n_ssq = 0
     if ssq_in is not None:
         _chk(ssq_in, "linear_bf16_link.ssq_in", torch.float32)
-        if ssq_in.dim() != 2 or ssq_in.shape[1] != 16:
-            raise KernelError(f"linear_bf16_link.ssq_in: shape {tuple(ssq_in.shape)}, expected [shares, 16]")
+        if ssq_in.dim() != 2 or ssq_in.shape[1] != link_stride(n):
+            raise KernelError(f"linear_bf16_link.ssq_in: shape {tuple(ssq_in.shape)}, expected [shares, {link_stride(n)}]")
         n_ssq = ssq_in.shape[0]
     if xn_out is not None:
         shares = linear_bf16_link_shares(n, m, k)
@@ -354,16 +370,22 @@ def linear_bf16_link(x: torch.Tensor, w: PackedMatrix, bias: Optional[torch.Tens
             raise KernelError(f"linear_bf16_link: {n} rows of [{m}, {k}] cannot hand a norm on (linear_bf16_link_shares)")
         _chk(xn_out, "linear_bf16_link.xn_out", torch.bfloat16, (n, m))
         _chk(gain_next, "linear_bf16_link.gain_next", torch.float32, (m,))
-        _chk(ssq_out, "linear_bf16_link.ssq_out", torch.float32, (shares, 16))
+        _chk(ssq_out, "linear_bf16_link.ssq_out", torch.float32, (shares, link_stride(n)))
+    need = linear_bf16_workspace(n, m, k) if n > 16 else 0
+    if need:
+        if workspace is None or workspace.numel() < need:
+            raise KernelError(f"linear_bf16_link: x [{n}, {k}] with W [{m}, {k}] needs a workspace of {need} floats")
+        _chk(workspace, "linear_bf16_link.workspace", torch.float32)
     _run(load_lib("vt_gemm_bf16"), "vt_linear_bf16_link", _ptr(x), _ptr(w.data), _ptr(bias), _ptr(residual), _ptr(out),
-         _i(n), _i(m), _i(k), _ptr(ssq_in), _i(n_ssq), _f(eps_in), _ptr(xn_out), _ptr(gain_next), _ptr(ssq_out), _stream())
+         _ptr(workspace if need else None), _i(n), _i(m), _i(k), _ptr(ssq_in), _i(n_ssq), _f(eps_in), _ptr(xn_out),
+         _ptr(gain_next), _ptr(ssq_out), _stream())
     return out
 
 
 def gated_linear_bf16_link(x: torch.Tensor, w: PackedMatrix, out: torch.Tensor, ssq_in: torch.Tensor,
                            eps_in: float) -> torch.Tensor:
     """gated_linear_bf16 behind an RMSNorm that the product in front has prepared: x = bf16(h * gain), ssq_in its
-    shares of the rows' sums of squares (up to 16 rows)."""
+    shares of the rows' sums of squares (up to 64 rows)."""
     n, k = x.shape
     if w.cols != k or w.halves != 2:
         raise KernelError(f"gated_linear_bf16_link: x [{n}, {k}] does not fit a packed matrix [{w.rows}, {w.cols}] x {w.halves}")
@@ -371,8 +393,9 @@ def gated_linear_bf16_link(x: torch.Tensor, w: PackedMatrix, out: torch.Tensor, 
     _chk(w.data, "gated_linear_bf16_link.w", torch.bfloat16)
     _chk(out, "gated_linear_bf16_link.out", None, (n, w.rows))
     _chk(ssq_in, "gated_linear_bf16_link.ssq_in", torch.float32)
-    if ssq_in.dim() != 2 or ssq_in.shape[1] != 16:
-        raise KernelError(f"gated_linear_bf16_link.ssq_in: shape {tuple(ssq_in.shape)}, expected [shares, 16]")
+    if n > 64 or ssq_in.dim() != 2 or ssq_in.shape[1] != link_stride(n):
+        raise KernelError(f"gated_linear_bf16_link: {n} rows, ssq_in of shape {tuple(ssq_in.shape)}: up to 64 rows and "
+                          f"[shares, {link_stride(n)}]")
     _run(load_lib("vt_gemm_bf16"), "vt_gated_linear_bf16_link", _ptr(x), _ptr(w.data), _ptr(out), _i(_code(out)), _i(n),
          _i(w.rows), _i(k), _ptr(ssq_in), _i(ssq_in.shape[0]), _f(eps_in), _stream())
     return out

@@ -52,7 +52,12 @@ def can_add_residual(rt: Runtime, n: int, m: int, k: int) -> bool:
 
 def can_hand_norm_on(rt: Runtime, n: int, m: int, k: int) -> bool:
     """Whether the product of n rows with W [m, k], adding to the residual stream, can prepare the norm behind it."""
-    return rt.dtype == torch.bfloat16 and n <= FUSE_MAX_ROWS and ops.linear_bf16_link_shares(n, m, k) > 0
+    return rt.dtype == torch.bfloat16 and n <= ops.LINK_MAX_ROWS and ops.linear_bf16_link_shares(n, m, k) > 0
+
+
+def takes_prepared_norm(rt: Runtime, n: int, k: int) -> bool:
+    """Whether a product of n rows over k can take a norm that the product in front has prepared."""
+    return rt.dtype == torch.bfloat16 and n <= ops.LINK_MAX_ROWS and k % 8 == 0
 
 
 def linear(rt: Runtime, x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], name: str,
@@ -70,30 +75,31 @@ def linear(rt: Runtime, x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.T
     n, k = x.shape
     m = w.shape[0] if w is not None else packed.rows * packed.halves   # (no row-major copy: the runtime keeps the packed one only)
     if residual is not None or isinstance(x, NormedInput):
-        if isinstance(x, NormedInput) and not (can_fuse(rt, n) and k % 8 == 0):
-            x = x.materialize()
-        if isinstance(x, NormedInput) or can_add_residual(rt, n, m, k):
-            norm = x if isinstance(x, NormedInput) else None
+        w_any = packed if packed is not None else w
+        is_packed = isinstance(w_any, ops.PackedMatrix)
+        if isinstance(x, NormedInput):
+            ok = (takes_prepared_norm(rt, n, k) and is_packed) if x.prepared else (can_fuse(rt, n) and k % 8 == 0)
+            if not ok:
+                x = x.materialize()
+        norm = x if isinstance(x, NormedInput) else None
+        if norm is not None or can_add_residual(rt, n, m, k):
             out = residual if residual is not None else rt.buffer(name, (n, m), torch.float32)
-            w_any = packed if packed is not None else w
-            emits = (hand_on is not None and residual is not None and isinstance(w_any, ops.PackedMatrix)
+            need = ops.linear_bf16_workspace(n, m, k) if n > 16 else 0
+            work = rt.buffer("linear.partials", (need,), torch.float32) if need else None
+            emits = (hand_on is not None and residual is not None and is_packed
                      and getattr(hand_on, "rms_fusable", False) and can_hand_norm_on(rt, n, m, k))
-            if emits or (norm is not None and norm.prepared and isinstance(w_any, ops.PackedMatrix)):
-                if norm is not None and not norm.prepared:
-                    x, norm = norm.materialize(), None     # (a product cannot take the norm in front both ways at once)
+            if emits and norm is not None and not norm.prepared:
+                x, norm = norm.materialize(), None     # (a product cannot take the norm in front both ways at once)
+            if emits or (norm is not None and norm.prepared):
                 xn = ssq = None
                 if emits:
                     xn = rt.buffer(name + ".xn", (n, m), torch.bfloat16)
-                    ssq = rt.buffer(name + ".ssq", (ops.linear_bf16_link_shares(n, m, k), 16), torch.float32)
+                    ssq = rt.buffer(name + ".ssq", (ops.linear_bf16_link_shares(n, m, k), ops.link_stride(n)), torch.float32)
                 ops.linear_bf16_link(norm.xn if norm else x, w_any, bias, out, residual=residual,
                                      ssq_in=norm.ssq if norm else None, eps_in=norm.eps if norm else 0.0,
-                                     xn_out=xn, gain_next=hand_on.gain if emits else None, ssq_out=ssq)
+                                     xn_out=xn, gain_next=hand_on.gain if emits else None, ssq_out=ssq, workspace=work)
                 return NormedInput(out, hand_on, xn, ssq) if emits else out
-            if norm is not None and norm.prepared:
-                x, norm = norm.materialize(), None
-                if not can_add_residual(rt, n, m, k) and residual is not None:
-                    return ops.residual_add(residual, linear(rt, x, w, bias, name, out_dtype, bias_lowp, packed))
-            return ops.linear_bf16(norm.h if norm else x, w_any, bias, out,
+            return ops.linear_bf16(norm.h if norm else x, w_any, bias, out, work,
                                    norm_gain=norm.gain if norm else None, norm_eps=norm.eps if norm else 0.0,
                                    residual=residual)
         if residual is not None:
