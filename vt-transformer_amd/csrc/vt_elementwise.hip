@@ -518,7 +518,9 @@ extern "C" int vt_gather_rows(const void* in, int in_dtype, const int* rows, voi
 // Streaming read: what the memory delivers to a kernel that only reads (the measured ceiling that the weight
 // streaming kernels are compared with).  Every wave reads a contiguous share, 1 KB per load instruction and
 // eight loads in flight, and leaves the XOR of its 32-bit words in sums[wave]; the words behind the last full
-// share of all waves are read by the last wave one load at a time.
+// share of all waves are read by the last wave one load at a time.  The loads are marked non-temporal, as the
+// weight-streaming kernels mark theirs: read once, not to be kept in the caches (6.7 against 6.0 TB/s unmarked).
+typedef unsigned stream_u32x4_t __attribute__((ext_vector_type(4)));
 __global__ __launch_bounds__(1024) void stream_read_kernel(const uint4* __restrict__ p, size_t n16,
                                                           unsigned* __restrict__ sums) {
     constexpr int U = 8;
@@ -531,7 +533,10 @@ __global__ __launch_bounds__(1024) void stream_read_kernel(const uint4* __restri
     for (size_t i = 0; i < per; i += 64 * U) {
         uint4 v[U];
 #pragma unroll
-        for (int u = 0; u < U; ++u) v[u] = q[i + 64 * u];
+        for (int u = 0; u < U; ++u) {
+            const stream_u32x4_t t = __builtin_nontemporal_load((const stream_u32x4_t*)(q + i + 64 * u));
+            v[u] = make_uint4(t.x, t.y, t.z, t.w);
+        }
 #pragma unroll
         for (int u = 0; u < U; ++u) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
     }
