@@ -414,7 +414,8 @@ __global__ __launch_bounds__(WPB * 64) void gemm_skinny_kernel(const void* __res
 #define MID_PIECES (64 * MID_BK / 8) // 16-byte pieces of x per stage
 
 // WM waves per block: the host picks it so that the blocks fill the compute units evenly.
-template <int R, bool SWIGLU, int WM, typename TO>
+// ONCE: one block of tokens, so that no other block reads these rows of W again (see load_w_once).
+template <int R, bool SWIGLU, int WM, typename TO, bool ONCE>
 __global__ __launch_bounds__(WM * 64) void gemm_mid_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wp,
                                                       const float* __restrict__ bias, TO* __restrict__ y,
                                                       float* __restrict__ partial, int N, int Mout, int K, int KT,
@@ -471,7 +472,6 @@ __global__ __launch_bounds__(WM * 64) void gemm_mid_kernel(const bf16_t* __restr
 #pragma unroll
         for (int q = 0; q < MID_XP; ++q) *(uint4*)&xs[buf][xtok[q]][xcol[q]] = xreg[q];
     };
-    const bool once = gridDim.y == 1;      // one block of tokens: no other block reads these rows of W again
     auto fetch_w = [&](Frag (&dst)[RW][MID_KU], int k0) __attribute__((always_inline)) {
         const size_t t0 = (size_t)(k0 >> 5) * PK_TILE;
 #pragma unroll
@@ -479,7 +479,8 @@ __global__ __launch_bounds__(WM * 64) void gemm_mid_kernel(const bf16_t* __restr
 #pragma unroll
             for (int a = 0; a < RW; ++a) {
                 const bf16_t* src = wbase[a] + t0 + (size_t)u * PK_TILE;
-                dst[a][u].u = once ? load_w_once(src) : *(const uint4*)src;
+                if constexpr (ONCE) dst[a][u].u = load_w_once(src);
+                else dst[a][u].u = *(const uint4*)src;
             }
     };
     auto multiply = [&](const Frag (&wf)[RW][MID_KU], int buf) __attribute__((always_inline)) {
@@ -921,12 +922,14 @@ static int linear_bf16(const void* xv, const bf16_t* wp, const float* bias, TO* 
         // the product takes the norm in front (link.ssq_in); the one behind is prepared where the sums are added up
         NormLink in = NO_LINK;
         in.ssq_in = link.ssq_in; in.n_ssq = link.n_ssq; in.eps = link.eps;
-#define VT_MID(W) gemm_mid_kernel<RR, SWIGLU, W, TO><<<grid, W * 64, 0, stream>>>(x, wp, bias, y, workspace, N, Mout, K, KT, up_tiles, kps, in)
+#define VT_MID_(W, O) gemm_mid_kernel<RR, SWIGLU, W, TO, O><<<grid, W * 64, 0, stream>>>(x, wp, bias, y, workspace, N, Mout, K, KT, up_tiles, kps, in)
+#define VT_MID(W) do { if (grid.y == 1) VT_MID_(W, true); else VT_MID_(W, false); } while (0)
         if (wm == 4) VT_MID(4);
         else if (wm == 5) VT_MID(5);
         else if (wm == 6) VT_MID(6);
         else VT_MID(8);
 #undef VT_MID
+#undef VT_MID_
         VT_CHECK_LAUNCH("vt_linear_bf16(64 tokens)");
         if (splits > 1) {
             const size_t n = (size_t)N * Mout;
