@@ -211,7 +211,7 @@ __global__ __launch_bounds__(WPB * 64) void gemm_skinny_kernel(const void* __res
     constexpr int NW = SWIGLU ? 2 : 1;
     constexpr int U = NORM ? 2 : 4;     // tiles in flight (fp32 tokens take three times the registers: measured)
     __shared__ float red[NW][WPB][256];
-    __shared__ uint4 xt[WPB][2][4 * 17];
+    __shared__ uint4 xt[WPB][NORM ? 2 : 4][4 * 17];     // per wave: two exchange buffers of one tile (NORM) or of a pair
     __shared__ float ssq[NORM ? WPB : 1][16];
     __shared__ float4 ssq_part[WPB][4];                       // consumer of a NormLink: the waves' sums of shares
     const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63;
@@ -291,6 +291,67 @@ __global__ __launch_bounds__(WPB * 64) void gemm_skinny_kernel(const void* __res
 #pragma unroll
     for (int a = 0; a < NW; ++a) acc[a] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
     int t = t_begin;
+    if constexpr (!NORM) {
+        // bf16 tokens by pairs of k tiles: a token's 64 values of a pair are one cache line, so lane l reads piece
+        // l % 8 (8 values) of row l / 8 (and of row l / 8 + 8 if there are more than 8 tokens): eight accesses of a
+        // whole line per load, where a tile at a time is sixteen of half a line, and it is the number of accesses
+        // that the first-level cache limits.  The waves split k in pairs (KT is a multiple of 4).
+        const int KP = KT >> 1;
+        const int p_begin = (int)(((long long)wv * KP) / WPB), p_end = (int)(((long long)(wv + 1) * KP) / WPB);
+        const bf16_t* xr_a = (const bf16_t*)xin + (size_t)min(lane >> 3, N - 1) * K;
+        const bf16_t* xr_b = (const bf16_t*)xin + (size_t)min((lane >> 3) + 8, N - 1) * K;
+        const int xpc = (lane & 7) * 8;
+        const bool two = N > 8;
+        uint4* const xw = &xt[wv][0][0];                // [2 buffers][2 tiles][4 * 17]
+        const int ws = ((lane & 7) >> 2) * 68 + (lane & 3) * 17 + (lane >> 3);
+        constexpr int UP = 2;                           // pairs in flight
+        auto pair_exchange = [&](const Frag& xa, const Frag& xb, int b, Frag& f0, Frag& f1) __attribute__((always_inline)) {
+            uint4* const buf = xw + b * 136;
+            buf[ws] = xa.u;
+            if (two) buf[ws + 8] = xb.u;                // (rows from the number of tokens on are never stored)
+            wave_lds_order();
+            f0.u = buf[rslot];
+            f1.u = buf[68 + rslot];
+            wave_lds_order();                           // and the next write to this buffer after these reads
+        };
+        int p = p_begin;
+        for (; p + UP <= p_end; p += UP) {
+            Frag wa[NW][2 * UP], xa[UP], xb[UP], xf[2 * UP];
+#pragma unroll
+            for (int up = 0; up < UP; ++up) {
+#pragma unroll
+                for (int u = 0; u < 2; ++u)
+#pragma unroll
+                    for (int a = 0; a < NW; ++a)
+                        wa[a][2 * up + u].u = load_w_once(wbase[a] + (size_t)(2 * (p + up) + u) * PK_TILE);
+                xa[up].v = load_x(xr_a, (p + up) * 64 + xpc, K);
+                if (two) xb[up].v = load_x(xr_b, (p + up) * 64 + xpc, K);
+            }
+#pragma unroll
+            for (int up = 0; up < UP; ++up) pair_exchange(xa[up], xb[up], up & 1, xf[2 * up], xf[2 * up + 1]);
+#pragma unroll
+            for (int u = 0; u < 2 * UP; ++u)
+#pragma unroll
+                for (int a = 0; a < NW; ++a)
+                    acc[a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[a][u].v, xf[u].v, acc[a], 0, 0, 0);
+        }
+        for (; p < p_end; ++p) {
+            Frag wa[NW][2], xa, xb, xf[2];
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+#pragma unroll
+                for (int a = 0; a < NW; ++a) wa[a][u].u = load_w_once(wbase[a] + (size_t)(2 * p + u) * PK_TILE);
+            xa.v = load_x(xr_a, p * 64 + xpc, K);
+            if (two) xb.v = load_x(xr_b, p * 64 + xpc, K);
+            pair_exchange(xa, xb, 0, xf[0], xf[1]);
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+#pragma unroll
+                for (int a = 0; a < NW; ++a)
+                    acc[a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[a][u].v, xf[u].v, acc[a], 0, 0, 0);
+        }
+        t = t_end;      // (nothing left for the loops below)
+    }
     for (; t + U <= t_end; t += U) {
         Frag wa[NW][U];
         Piece xa[U];
