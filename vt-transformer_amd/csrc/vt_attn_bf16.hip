@@ -320,7 +320,7 @@ __device__ __forceinline__ void merge_parts(float (*sm)[16], float (*sl)[16], co
 
 // RT row tiles of 16 rows per wave share every key/value block they read.
 template <bool DECODE, int RT>
-__global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_kernel(AttnArgs a) {
+__global__ __launch_bounds__(256, D > 128 ? 1 : (DECODE ? 3 : 2)) void attn_bf16_kernel(AttnArgs a) {
     // the wave's index as a scalar: its item and everything read from it then stay in scalar registers, and the
     // tests on them are scalar branches
     const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
@@ -356,6 +356,23 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_kernel(AttnArg
     const int G = a.n_heads / a.n_kv;
     const int r = lane & 15, g = lane >> 4;
     const int n_rows = q_len * G;
+
+    const int* bt = a.block_table + (size_t)entry * a.max_blocks;
+    const int ps = a.page_size;
+    const int last_page = (key_hi - 1) / ps;
+    KVBlock cur;
+    const int j_first = key_lo + (DECODE ? 16 * wv : 0), j_step = DECODE ? 64 : 16;
+    // the last block this wave may read: the last one of its own, or for a wave without keys the item's first
+    const int j_end = j_first < key_hi ? j_first + (key_hi - 1 - j_first) / j_step * j_step : key_lo;
+    // (read through the constant address space: the kernel writes pages and results but never the block table,
+    // and only so is this a scalar load, which neither counts among the vector loads in flight nor waits for them)
+    typedef const __attribute__((address_space(4))) int* const_int_ptr;
+    const const_int_ptr btc = (const_int_ptr)(uintptr_t)bt;
+    auto page_at = [&](int j) __attribute__((always_inline)) { return btc[min(page_index(a, min(j, j_end)), last_page)]; };
+    const int spare = min(max(btc[last_page], 0), a.num_pages - 1);
+    // A decoding wave asks for its first block before it turns to the query, whose loads and rotation would
+    // otherwise stand between the block table and the first keys: one round trip to memory less per launch.
+    if (DECODE && a.qkv) load_block<DECODE>(cur, a, page_at(j_first), spare, min(j_first, j_end), kvh, lane);
 
     bool row_ok[RT];
     int ti[RT], head[RT], p[RT], p_lo[RT], tile_hi[RT], tile_lo[RT], tile_first_p[RT], tile_last_lo[RT];
@@ -451,9 +468,6 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_kernel(AttnArg
         __syncthreads();
     }
 
-    const int* bt = a.block_table + (size_t)entry * a.max_blocks;
-    const int ps = a.page_size;
-    const int last_page = (key_hi - 1) / ps;
     // one block of 16 keys against the RT row tiles of this wave
     extern __shared__ __attribute__((aligned(16))) bf16_t wave_lds[];
     bf16_t* const kl = wave_lds + wv * KV_LDS_ELEMS;      // this wave's buffer: keys, then values
@@ -501,19 +515,13 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_kernel(AttnArg
     // from the block table meanwhile (a scalar load).  Every turn loads, whether or not keys are left (then the
     // wave's last block again, which nobody multiplies), so that no load sits under a branch.  (Two and three
     // buffers were slower inside whole decoding steps.)
-    KVBlock cur;
-    const int j_first = key_lo + (DECODE ? 16 * wv : 0), j_step = DECODE ? 64 : 16;
-    // the last block this wave may read: the last one of its own, or for a wave without keys the item's first
-    const int j_end = j_first < key_hi ? j_first + (key_hi - 1 - j_first) / j_step * j_step : key_lo;
-    // (read through the constant address space: the kernel writes pages and results but never the block table,
-    // and only so is this a scalar load, which neither counts among the vector loads in flight nor waits for them)
-    typedef const __attribute__((address_space(4))) int* const_int_ptr;
-    const const_int_ptr btc = (const_int_ptr)(uintptr_t)bt;
-    auto page_at = [&](int j) __attribute__((always_inline)) { return btc[min(page_index(a, min(j, j_end)), last_page)]; };
-    const int spare = min(max(btc[last_page], 0), a.num_pages - 1);
-    int pg_next;                     // page of the next block to load
-    load_block<DECODE>(cur, a, page_at(j_first), spare, min(j_first, j_end), kvh, lane);
-    pg_next = page_at(j_first + j_step);
+    if (!(DECODE && a.qkv)) {
+        load_block<DECODE>(cur, a, page_at(j_first), spare, min(j_first, j_end), kvh, lane);
+    } else if (dec_writes && min(j_first, j_end) + 16 > pos0) {
+        // the wave's first block holds the token's own key and value, which were written above: read it again
+        load_block<DECODE>(cur, a, page_at(j_first), spare, min(j_first, j_end), kvh, lane);
+    }
+    int pg_next = page_at(j_first + j_step);      // page of the next block to load
     for (int j = j_first; j < key_hi; j += j_step) {
         const bool ok = cur.ok;
         if (ok) park_block(cur, kl, lane);
