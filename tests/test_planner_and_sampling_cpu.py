@@ -50,7 +50,8 @@ def test_every_row_gets_every_key_it_may_see_exactly_once(group, window, target,
 @pytest.mark.parametrize("group,window", [(1, 0), (7, 0), (5, 40)])
 @pytest.mark.parametrize("rt", [1, 2])
 @pytest.mark.parametrize("split", [0., 0.5, 1.4, None])
-def test_tile_items_cover_the_long_entries(group, window, rt, split):
+@pytest.mark.parametrize("direct", [False, True])
+def test_tile_items_cover_the_long_entries(group, window, rt, split, direct):
     """Every row of a long entry meets every key it may see exactly once, whether or not the keys of the longest
     items are cut into ranges; the ranges of an item have consecutive partial indices and one merge per 16-row tile."""
     lens = np.array([1, 300, 40, 2048, 260])
@@ -60,7 +61,7 @@ def test_tile_items_cover_the_long_entries(group, window, rt, split):
     assert sorted(list(short) + list(long)) == list(range(5))
     assert all(lens[e] * group >= 256 for e in long) and all(lens[e] * group < 256 for e in short)
     items, got_rt, citems, n_parts = plan_tile_items(start, pos0.astype(np.int32), group, window, 4, long,
-                                                     rt=rt if split is not None else None, split=split)
+                                                     rt=rt if split is not None else None, split=split, direct=direct)
     if split is not None:
         assert got_rt == rt
     rt = got_rt
@@ -147,3 +148,17 @@ def test_sampling_params_follow_the_front_end():
     for bad in (dict(top_p=0.0), dict(top_k=0), dict(max_tokens=0)):
         with pytest.raises(ValueError):
             SamplingParams(**bad)
+
+
+def test_the_direct_kernels_launch_model_picks_what_was_measured():
+    """A fresh 2,048-token prompt on 28 / 4 heads runs fastest as whole items of one row tile per wave (its longest
+    item is what the launch lasts), the same portion behind 2,048 earlier tokens with two row tiles (every block
+    of keys read serves twice the rows); eight 1,024-token prompts fill the GPU with two row tiles and no cuts."""
+    def pick(lens, pos0, nh=28, nkv=4):
+        start = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        items, rt, citems, n_parts = plan_tile_items(start, np.array(pos0, np.int32), nh // nkv, 0, nkv,
+                                                     np.arange(len(lens)), head_dim=128, direct=True)
+        return rt, n_parts
+    assert pick([2048], [0]) == (1, 0)
+    assert pick([2048], [2048])[0] == 2
+    assert pick([1024] * 8, [0] * 8) == (2, 0)

@@ -630,7 +630,27 @@ constexpr int KROW = D + 8;                    // padded rows: operand reads fro
 constexpr int VROW = KB + 8;
 constexpr int GP = 2 * D;                      // 16-byte pieces of 16 keys (and of their values)
 constexpr int NP = (GP + 255) / 256;           // pieces per thread and group of 16 keys
-constexpr int TILE_LDS_BYTES = 2 * (KB * KROW + D * VROW) * (int)sizeof(bf16_t);
+// With a head of 128 the blocks go from the pages straight into LDS (global_load_lds, 16 bytes per lane): no
+// registers hold them on the way and no thread stores them.  A wave's load writes 64 consecutive 16-byte slots of
+// LDS, one per lane, and each lane chooses what it reads from memory, so the layout is made by the choice of
+// addresses: a key row is 16 slots, and chunk c (8 dims) of LDS row p sits in slot c ^ (p % 16) of the row, so that
+// the sixteen rows of a score tile are read from sixteen different slots modulo 16 (no bank conflicts, no padding);
+// the values of a group of 16 keys are [tile of 16 dims][8 keys of 16][dim of the tile], 16 bytes each.
+constexpr bool TILE_DMA = (D == 128);
+constexpr int KBUF = TILE_DMA ? KB * D : KB * KROW;        // elements of a key buffer, of a value buffer
+constexpr int VBUF = TILE_DMA ? D * KB : D * VROW;
+constexpr int TILE_LDS_BYTES = 2 * (KBUF + VBUF) * (int)sizeof(bf16_t);
+typedef __attribute__((address_space(3))) void* lds_void_ptr;
+// One load of a wave from memory into LDS: lane l's 16 bytes at base + off go to LDS bytes lds + 16 l .. + 15.
+// `base` and `lds` are the same in every lane.  Written as assembly because the compiler, which cannot tell the two
+// buffers of a block apart, makes every later read of LDS wait for such a load when it knows of it; here the
+// program waits itself, before the barrier behind which the buffer is read.  (The compiler's own waits for its own
+// loads stay right: loads return in order, and these only add to the number that it counts.)
+__device__ __forceinline__ void load_to_lds16(const void* base, unsigned off, unsigned lds) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :: "v"(off), "s"(base), "s"(lds) : "memory", "m0");
+}
+__device__ __forceinline__ unsigned lds_address(const void* p) { return (unsigned)(uintptr_t)(lds_void_ptr)p; }
 
 // key (relative to the block's first) of score tile kt, lane group g, register i
 __device__ __forceinline__ int tile_key(int kt, int g, int i) { return 32 * (kt >> 1) + 8 * g + 4 * (kt & 1) + i; }
@@ -695,8 +715,8 @@ __device__ __forceinline__ void tile_softmax(const f32x4_t (&s)[KT], int j0, int
 template <int RT>
 __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_tile_kernel(AttnArgs a) {
     extern __shared__ __attribute__((aligned(16))) bf16_t tile_lds[];
-    bf16_t* const k_lds = tile_lds;                       // [2][KB][KROW]
-    bf16_t* const v_lds = tile_lds + 2 * KB * KROW;       // [2][D][VROW]
+    bf16_t* const k_lds = tile_lds;                       // [2][KBUF]
+    bf16_t* const v_lds = tile_lds + 2 * KBUF;            // [2][VBUF]
     const int tid = threadIdx.x, lane = tid & 63;
     // the wave's index as a scalar: what depends only on it (which keys the wave's tiles see) then stays in scalar
     // registers and its tests are scalar branches
@@ -796,6 +816,57 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_tile_kernel(At
     const char* const v_base = (const char*)(a.v_pages + (size_t)kvh * ps * D);
     // (a native vector type: copies of HIP's uint4 struct become memcpy calls that keep the stage in scratch memory)
     u32x4_t st_k[KT][NP], st_v[KT][NP];
+    // Direct path: wave w brings the key pieces w, w + 4, ... (four LDS rows each: four consecutive keys of one
+    // page, 1 KB in a row) and the value pieces KT w .. KT w + KT - 1 (a group of 16 keys has four pieces of 32 dims).
+    const unsigned dma_k_off = (unsigned)(lane >> 4) * (2 * D) + ((unsigned)((lane & 15) ^ ((4 * wv + (lane >> 4)) & 15)) << 4);
+    const unsigned dma_v_off = (unsigned)((lane & 15) + 16 * (lane >> 5)) * (unsigned)(2 * ps) + (unsigned)((lane >> 4) & 1) * 16u;
+    // This wave's three groups of 16 keys of the next block to fetch (two for its key pieces, one for its values):
+    // the entry's page they lie in and the offset in it, moved on by KB keys per fetch without a division; the page
+    // ids are read from the block table a step ahead, through the constant address space (the kernel never writes
+    // the table): only so are they scalar loads, which do not wait for the loads into LDS that are in flight.
+    typedef const __attribute__((address_space(4))) int* const_int_ptr;
+    const const_int_ptr btc = (const_int_ptr)(uintptr_t)bt;
+    const unsigned lds_k0 = lds_address(k_lds), lds_v0 = lds_address(v_lds);
+    constexpr int NGW = KH + 1;                           // groups of a block that a wave touches
+    const int v_group = (wv * KT) >> 2;                   // the group whose values this wave brings
+    int g_blk[NGW], g_off[NGW], g_pg[NGW];
+    const int adv_blk = KB / ps, adv_off = KB - adv_blk * ps;
+#pragma unroll
+    for (int i = 0; i < NGW; ++i) {
+        const int kp = key_lo + (i < KH ? 32 * i + 16 * (wv >> 1) : 16 * v_group);
+        g_blk[i] = kp / ps;
+        g_off[i] = kp - g_blk[i] * ps;
+    }
+    auto dma_pages = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < NGW; ++i) g_pg[i] = btc[min(g_blk[i], last_page)];
+    };
+    auto fetch_dma = [&](int buf) __attribute__((always_inline)) {
+        const unsigned kd = lds_k0 + buf * (KBUF * 2), vd = lds_v0 + buf * (VBUF * 2);     // byte addresses in LDS
+#pragma unroll
+        for (int n = 0; n < KT; ++n) {
+            const int h = n >> 1, key0 = 8 * (wv & 1) + 4 * (n & 1);
+            const int pg = (g_pg[h] >= 0 && g_pg[h] < a.num_pages) ? g_pg[h] : pg_spare;
+            const char* src = k_base + ((size_t)pg * page_bytes + (unsigned)((g_off[h] + key0) * (2 * D)));
+            load_to_lds16(src, dma_k_off, kd + (wv + 4 * n) * 1024);
+        }
+        const int pg = (g_pg[KH] >= 0 && g_pg[KH] < a.num_pages) ? g_pg[KH] : pg_spare;
+        const char* vsrc = v_base + ((size_t)pg * page_bytes + (unsigned)(g_off[KH] * 2));
+#pragma unroll
+        for (int m = 0; m < KT; ++m) {
+            const int u = (wv * KT + m) & 3;              // the piece of 32 dims
+            load_to_lds16(vsrc + (size_t)(u * 32) * (2 * ps), dma_v_off, vd + v_group * 4096 + u * 1024);
+        }
+#pragma unroll
+        for (int i = 0; i < NGW; ++i) {
+            g_blk[i] += adv_blk;
+            g_off[i] += adv_off;
+            const bool wrap = g_off[i] >= ps;
+            g_off[i] -= wrap ? ps : 0;
+            g_blk[i] += wrap ? 1 : 0;
+        }
+        dma_pages();
+    };
     auto fetch = [&]() __attribute__((always_inline)) {   // this thread's pieces of the next KB keys, pages -> registers
 #pragma unroll
         for (int kt = 0; kt < KT; ++kt) {
@@ -818,8 +889,8 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_tile_kernel(At
         next_pages();
     };
     auto park = [&](int buf) __attribute__((always_inline)) {
-        bf16_t* const kd = k_lds + buf * (KB * KROW);
-        bf16_t* const vd = v_lds + buf * (D * VROW);
+        bf16_t* const kd = k_lds + buf * KBUF;
+        bf16_t* const vd = v_lds + buf * VBUF;
 #pragma unroll
         for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
@@ -835,18 +906,20 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_tile_kernel(At
     // one key block (in LDS buffer `buf`, keys from j0) against the RT row tiles of this wave
     auto multiply = [&](int buf, int j0) __attribute__((always_inline)) {
         if (j0 > wave_hi || j0 + KB - 1 < wave_lo) return;   // every key masked for every row of the wave
-        const bf16_t* const kd = k_lds + buf * (KB * KROW);
-        const bf16_t* const vd = v_lds + buf * (D * VROW);
+        const bf16_t* const kd = k_lds + buf * KBUF;
+        const bf16_t* const vd = v_lds + buf * VBUF;
         f32x4_t s[RT][KT];
 #pragma unroll
         for (int kt = 0; kt < KT; ++kt) {
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) s[rt][kt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
-            const bf16_t* kr = kd + (kt * 16 + r) * KROW;
+            const bf16_t* kr = kd + (kt * 16 + r) * (TILE_DMA ? D : KROW);
             if constexpr (WIDE) {
 #pragma unroll
                 for (int st = 0; st < QSTEPS; ++st) {
-                    U16 t; t.u = *(const uint4*)(kr + st * 32 + g * 8);
+                    U16 t;
+                    if constexpr (TILE_DMA) t.u = *(const uint4*)(kr + (((4 * st + g) ^ r) << 3));
+                    else t.u = *(const uint4*)(kr + st * 32 + g * 8);
 #pragma unroll
                     for (int rt = 0; rt < RT; ++rt)
                         s[rt][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(t.v, q8[rt][st], s[rt][kt], 0, 0, 0);
@@ -886,7 +959,9 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_tile_kernel(At
             }
 #pragma unroll
             for (int t = 0; t < DT; ++t) {
-                U16 vf; vf.u = *(const uint4*)(vd + (t * 16 + r) * VROW + 32 * h + 8 * g);
+                U16 vf;
+                if constexpr (TILE_DMA) vf.u = *(const uint4*)(vd + (2 * h + (g >> 1)) * 2048 + ((2 * t + (g & 1)) * 16 + r) * 8);
+                else vf.u = *(const uint4*)(vd + (t * 16 + r) * VROW + 32 * h + 8 * g);
 #pragma unroll
                 for (int rt = 0; rt < RT; ++rt)
                     o[rt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[rt].v, o[rt][t], 0, 0, 0);
@@ -894,18 +969,32 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_tile_kernel(At
         }
     };
 
-    next_pages();
-    fetch();
-    park(0);
-    __syncthreads();
     int buf = 0;
-    for (int j0 = key_lo; j0 < key_hi; j0 += KB) {
-        const bool more = j0 + KB < key_hi;
-        if (more) fetch();              // the next block is on its way while this one is multiplied
-        multiply(buf, j0);
-        if (more) park(buf ^ 1);
+    if constexpr (TILE_DMA) {
+        dma_pages();
+        fetch_dma(0);
+        __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0): this wave's pieces are in LDS
         __syncthreads();
-        buf ^= 1;
+        for (int j0 = key_lo; j0 < key_hi; j0 += KB) {
+            if (j0 + KB < key_hi) fetch_dma(buf ^ 1);     // the next block is on its way while this one is multiplied
+            multiply(buf, j0);
+            __builtin_amdgcn_s_waitcnt(0x0F70);
+            __syncthreads();
+            buf ^= 1;
+        }
+    } else {
+        next_pages();
+        fetch();
+        park(0);
+        __syncthreads();
+        for (int j0 = key_lo; j0 < key_hi; j0 += KB) {
+            const bool more = j0 + KB < key_hi;
+            if (more) fetch();              // the next block is on its way while this one is multiplied
+            multiply(buf, j0);
+            if (more) park(buf ^ 1);
+            __syncthreads();
+            buf ^= 1;
+        }
     }
 
 #pragma unroll
@@ -1034,6 +1123,10 @@ extern "C" int vt_attn_bf16(const void* q, const void* k_pages, const void* v_pa
 // (item, kv head).  An item holds all the keys its rows may see (partial index -1), or one of several ranges of them:
 // then it leaves its partial result in workspace slot (partial index * 4 rt + tile) and the combine items [m][6]
 // (one per 16-row tile, as above, with 4 rt tiles per item) merge the ranges.
+// 1 if this head size's tiled kernel loads its key/value blocks straight into LDS (which decides how the host
+// cuts its work), else 0
+extern "C" int vt_attn_bf16_tiles_direct() { return TILE_DMA ? 1 : 0; }
+
 extern "C" int vt_attn_bf16_tiles(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
                                   const int* items, int n_items, int rt, const int* citems, int n_citems, void* out,
                                   float* part_o, float* part_ml, int n_heads, int n_kv, int page_size,

@@ -460,7 +460,7 @@ def attention_bf16(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor
     num_pages, kvh, page_size, d = k_pages.shape
     if head_dim % 16 or not 16 <= head_dim <= 256:
         raise KernelError(f"attention_bf16: head size {head_dim} is not a multiple of 16 in 16..256")
-    if rt not in (1, 2):
+    if rt not in (1, 2, 3):
         raise KernelError(f"attention_bf16: {rt} row tiles per item (1 or 2)")
     _chk(q, "attention_bf16.q", torch.bfloat16, (n, n_heads * head_dim))
     _chk(k_pages, "attention_bf16.k_pages", torch.bfloat16, (num_pages, n_kv, page_size, head_dim))
@@ -483,6 +483,12 @@ def attention_bf16(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor
          _ptr(citems), _i(n_citems), _ptr(out), _ptr(part_o), _ptr(part_ml), _i(n_heads), _i(n_kv), _i(page_size),
          _i(block_table.shape[1]), _i(num_pages), _i(window), _f(scale), _stream())
     return out
+
+
+def attention_bf16_tiles_direct(head_dim: int) -> bool:
+    """Whether the tiled kernel of this head size loads its key/value blocks straight into LDS; the host prices
+    its launches differently then (parts.attention_plan.plan_tile_items)."""
+    return bool(load_lib("vt_attn_bf16", head_dim).vt_attn_bf16_tiles_direct())
 
 
 def attention_bf16_tiles(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,

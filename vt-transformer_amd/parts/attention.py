@@ -66,6 +66,7 @@ class PagedAttention(Part):
             shared[key] = POSITIONS.build(pos_spec, rt=rt)
         self.position = shared[key]
         self.w_qkv = self.b_qkv = self.b_qkv_lowp = self.w_o = self.b_o = self.p_qkv = self.p_o = None
+        self._direct_tiles: Optional[bool] = None     # asked of the kernel library at the first planned step
 
     @property
     def replayable(self) -> bool:
@@ -133,7 +134,10 @@ class PagedAttention(Part):
         key = self._items_key()
         if key in ctx.extra_host:
             return None
-        host = plan_step(ctx.h_entry_start, ctx.h_entry_pos0, self.nh // self.nkv, self.window, self.nkv, self.d)
+        if self._direct_tiles is None:
+            self._direct_tiles = ops.attention_bf16_tiles_direct(self.d)
+        host = plan_step(ctx.h_entry_start, ctx.h_entry_pos0, self.nh // self.nkv, self.window, self.nkv, self.d,
+                         direct=self._direct_tiles)
         ctx.memo[key] = host
         return {key: host.flat()}
 

@@ -58,6 +58,17 @@ TILE_STEP_US = {1: 2.1, 2: 2.45}
 # (102), 64 / 8 heads 103 (103): no shorter cut helped anywhere, and cuts at 1 and below cost up to a fifth where the
 # items fill the GPU anyway.
 TILE_CUT = 1.4
+# The kernel that loads straight into LDS (head size 128), fitted to launches of 4 to 8,192 blocks (one to eight
+# prompts of 256 to 4,096 tokens with up to 7,168 earlier ones, 12 to 64 query heads on 2 to 8 kv heads; the choice
+# it makes is within 5 % of the best of one and two row tiles with and without cuts on each of them): a block's
+# step of 64 keys takes DIRECT_STEP_US with one and two row tiles per wave, a block DIRECT_BLOCK_US beside its
+# steps (until its first keys are in LDS, and its results written), DIRECT_SLOTS blocks run at a time, and a merge
+# launch costs DIRECT_MERGE_US[0] + [1] per 16-row tile.
+DIRECT_STEP_US = {1: 1.3, 2: 2.0}
+DIRECT_START_US = 4.0
+DIRECT_BLOCK_US = 4.0
+DIRECT_SLOTS = 448
+DIRECT_MERGE_US = (8.0, 0.03)
 TILE_MIN_STEPS = 6      # no item's keys are cut into ranges of fewer steps than this
 TILE_MAX_PARTS = 8      # ... or into more ranges than this
 LONG_ENTRY_ROWS = 256   # entries with at least this many (token, head-of-group) rows go to the LDS-tiled kernel
@@ -73,18 +84,21 @@ def split_entries(entry_start: np.ndarray, group: int) -> Tuple[np.ndarray, np.n
 
 def plan_tile_items(entry_start: np.ndarray, entry_pos0: np.ndarray, group: int, window: int, n_kv: int,
                     entries: np.ndarray, rt: Optional[int] = None, slots: int = TILE_SLOTS, head_dim: int = 128,
-                    split: Optional[float] = None) -> Tuple[np.ndarray, int, np.ndarray, int]:
+                    split: Optional[float] = None, direct: bool = False) -> Tuple[np.ndarray, int, np.ndarray, int]:
     """Items of the LDS-tiled kernel: 64 * rt rows of one entry and the keys they may see, longest first so that
     the blocks that finish last start first.  Returns (items [n, 8], rt, combine items [m, 6], partial indices).
 
-    A block's step over 64 keys takes about as long with two row tiles per wave as with one (TILE_STEP_US), because
-    a wave waits on its own chain of loads, products and exponentials more than on the machine; `slots` blocks run
-    at a time and the others follow as blocks finish, so a launch lasts as long as its longest item or as all items'
-    steps shared out over the slots, whichever is more.  The longest items of a fresh prompt (its last rows see
-    every key) are what a launch waits for when the items are few (few kv heads, one prompt): their keys are cut
-    into ranges, each an item of its own, whose partial results the merge kernel adds up (TILE_CUT).  `rt` (row
-    tiles per wave) and `split` (the length to cut to, in units of the balanced launch; 0: no cuts) override the
-    choice.  Heads above 128 keep whole items and choose rt by the estimate."""
+    `slots` blocks run at a time and the others follow as blocks finish, so a launch lasts as long as its longest
+    item or as all items' steps shared out over the slots, whichever is more.  The longest items of a fresh prompt
+    (its last rows see every key) are what a launch waits for when the items are few (few kv heads, one prompt):
+    their keys are cut into ranges, each an item of its own, whose partial results the merge kernel adds up.
+    `rt` (row tiles per wave) and `split` (the length to cut to, in units of the balanced launch; 0: no cuts)
+    override the choice.
+
+    `direct`: the kernel brings its key/value blocks from the pages straight into LDS (head size 128).  Then one and
+    two row tiles, with and without cuts at TILE_CUT, are priced with a model of the launch (DIRECT_*) and the
+    cheapest is taken.  Otherwise: two row tiles with cuts up to a head size of 128 (a block's step takes about as
+    long with two row tiles as with one there, TILE_STEP_US), whole items and the cheaper row tiles above."""
     q_len = (entry_start[1:] - entry_start[:-1]).astype(np.int64)[entries]
     rows = q_len * group
     e_pos0_all = entry_pos0[entries].astype(np.int64)
@@ -110,10 +124,37 @@ def plan_tile_items(entry_start: np.ndarray, entry_pos0: np.ndarray, group: int,
     def steps_of(it):
         return (it["hi"] - it["lo"] + 63) // 64
 
+    def parts_of(steps, split_: float):
+        if split_ <= 0:
+            return np.ones_like(steps)
+        balanced = float(steps.sum()) * n_kv / slots
+        target = max(TILE_MIN_STEPS, int(np.ceil(balanced * split_)))
+        return np.minimum(np.where(steps > target, -(-steps // target), 1), TILE_MAX_PARTS)
+
     def estimate(it, rt_: int) -> float:
         steps = steps_of(it)
         return max(float(steps.max()), float(steps.sum()) * n_kv / slots) * TILE_STEP_US[rt_]
 
+    def direct_estimate(it, rt_: int, parts) -> float:
+        steps = steps_of(it)
+        longest = float((-(-steps // parts)).max())
+        blocks = float(parts.sum()) * n_kv
+        merges = float(np.minimum(4 * rt_, -(-(it["rows"] - it["row0"]) // 16))[parts > 1].sum())
+        launch = max(longest * DIRECT_STEP_US[rt_] + DIRECT_START_US,
+                     (float(steps.sum()) * n_kv * DIRECT_STEP_US[rt_] + blocks * DIRECT_BLOCK_US) / DIRECT_SLOTS)
+        return launch + (DIRECT_MERGE_US[0] + DIRECT_MERGE_US[1] * merges if merges else 0.)
+
+    if direct and head_dim <= 128 and (rt is None or split is None):
+        best = None
+        for rt_ in ((1, 2) if rt is None else (rt,)):
+            it = items_for(rt_)
+            if it is None:
+                return none
+            for split_ in ((0., TILE_CUT) if split is None else (split,)):
+                cost = direct_estimate(it, rt_, parts_of(steps_of(it), split_))
+                if best is None or cost < best[0]:
+                    best = (cost, rt_, split_)
+        _, rt, split = best
     if rt is None:
         if head_dim <= 128:
             rt = 2          # (measured: with the longest items cut, two row tiles are as good as one or better)
@@ -128,11 +169,7 @@ def plan_tile_items(entry_start: np.ndarray, entry_pos0: np.ndarray, group: int,
     if it is None:
         return none
     steps = steps_of(it)
-    parts = np.ones_like(steps)
-    if split > 0:
-        balanced = float(steps.sum()) * n_kv / slots
-        target = max(TILE_MIN_STEPS, int(np.ceil(balanced * split)))
-        parts = np.minimum(np.where(steps > target, -(-steps // target), 1), TILE_MAX_PARTS)
+    parts = parts_of(steps, split)
     total = len(parts)
     n_all = int(parts.sum())
     of = np.repeat(np.arange(total), parts)                   # item that each part belongs to
@@ -274,8 +311,9 @@ class HostPlan:
 
 
 def plan_step(entry_start: np.ndarray, entry_pos0: np.ndarray, group: int, window: int, n_kv: int,
-              head_dim: int) -> HostPlan:
-    """All of a step's attention work for one kind of attention layer."""
+              head_dim: int, direct: bool = False) -> HostPlan:
+    """All of a step's attention work for one kind of attention layer.  `direct`: the tiled kernel of this head
+    size loads its keys and values straight into LDS (plan_tile_items)."""
     short, long = split_entries(entry_start, group)
     # (heads above 128: two row tiles per wave do not fit the registers)
     row_tiles = choose_row_tiles(entry_start, group, n_kv, short) if len(short) and head_dim <= 128 else 1
@@ -284,7 +322,7 @@ def plan_step(entry_start: np.ndarray, entry_pos0: np.ndarray, group: int, windo
     # (heads above 128: one block per compute unit at a time)
     t_items, tile_rt, t_citems, t_parts = plan_tile_items(
         entry_start, entry_pos0, group, window, n_kv, long,
-        slots=TILE_SLOTS if head_dim <= 128 else TILE_SLOTS // 2, head_dim=head_dim)
+        slots=TILE_SLOTS if head_dim <= 128 else TILE_SLOTS // 2, head_dim=head_dim, direct=direct)
     return HostPlan((items, citems, t_items, t_citems), row_tiles, n_parts, tile_rt, t_parts)
 
 
