@@ -587,7 +587,9 @@ def test_attention_decode_fused_kernel(nh, kvh, d, rot, window, chunk):
     if rot:
         ang = torch.rand(max_pos, half, generator=g, dtype=torch.float64) * 6.28
         cos, sin = torch.cos(ang).float().to(DEV), torch.sin(ang).float().to(DEV)
-    for cached in ([0, 15, 16, 17, 300, 63, 1000], [31, 1, 999]):
+    # (positions in every wave's first block of keys and in its second one: a wave asks for its first two blocks
+    # before the token's own key and value are written, unless they hold them)
+    for cached in ([0, 15, 16, 17, 300, 63, 1000], [31, 1, 999, 70, 119, 200]):
         n = len(cached)
         lens = [c + 1 for c in cached]
         ks = [torch.randn(t, kvh, d, generator=g).to(torch.bfloat16).float() for t in lens]

@@ -154,7 +154,41 @@ constexpr int DT = D / 16;
 // (KV_LDS_ELEMS elements: keys [16][D + 8], values [D][24]).
 constexpr int KVP = (2 * D + 63) / 64;            // pieces per lane, of the keys and of the values
 constexpr int KL_ROW = D + 8, VL_ROW = 24;        // padded LDS rows: operand reads without bank conflicts
-constexpr int KV_LDS_ELEMS = 16 * KL_ROW + D * VL_ROW;
+
+// With a head of 128 the key/value blocks go from the pages straight into LDS (global_load_lds, 16 bytes per lane):
+// no registers hold them on the way and no thread stores them.  A wave's load writes 64 consecutive 16-byte slots
+// of LDS, one per lane, and each lane chooses what it reads from memory, so the layout is made by the choice of
+// addresses: a key row is 16 slots, and chunk c (8 dims) of LDS row p sits in slot c ^ (p % 16) of the row, so that
+// the sixteen rows of a score tile are read from sixteen different slots modulo 16 (no bank conflicts, no padding);
+// the values of a group of 16 keys are [tile of 16 dims][8 keys of 16][dim of the tile], 16 bytes each.
+constexpr bool DIRECT = (D == 128);
+typedef __attribute__((address_space(3))) void* lds_void_ptr;
+// One load of a wave from memory into LDS: lane l's 16 bytes at base + off go to LDS bytes lds + 16 l .. + 15.
+// `base` and `lds` are the same in every lane.  Written as assembly because the compiler, which cannot tell the
+// buffers of a block apart, makes every later read of LDS wait for such a load when it knows of it; here the
+// program waits itself before it reads a buffer.  (The compiler's own waits for its own loads stay right: loads
+// return in order, and these only add to the number that it counts.)  ONCE: no other wave reads these bytes.
+template <bool ONCE = false>
+__device__ __forceinline__ void load_to_lds16(const void* base, unsigned off, unsigned lds) {
+    if constexpr (ONCE)
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 nt"
+                     :: "v"(off), "s"(base), "s"(lds) : "memory", "m0");
+    else
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                     :: "v"(off), "s"(base), "s"(lds) : "memory", "m0");
+}
+__device__ __forceinline__ unsigned lds_address(const void* p) { return (unsigned)(uintptr_t)(lds_void_ptr)p; }
+// wait until at most N of this wave's loads are in flight; no access to memory moves across it
+template <int N>
+__device__ __forceinline__ void wait_loads() {
+    static_assert(N >= 0 && N < 16, "the count's low four bits");
+    asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory");
+}
+// (direct: two buffers per wave of 16 keys and their values as they come, the next block but one is on its way
+// while a block is multiplied)
+constexpr int WAVE_BUFS = DIRECT ? 2 : 1;
+constexpr int KV_BUF_ELEMS = DIRECT ? 2 * 16 * D : 16 * KL_ROW + D * VL_ROW;
+constexpr int KV_LDS_ELEMS = WAVE_BUFS * KV_BUF_ELEMS;
 struct KVBlock {
     u32x4_t k[KVP], v[KVP];
     bool ok;
@@ -320,7 +354,7 @@ __device__ __forceinline__ void merge_parts(float (*sm)[16], float (*sl)[16], co
 
 // RT row tiles of 16 rows per wave share every key/value block they read.
 template <bool DECODE, int RT>
-__global__ __launch_bounds__(256, D > 128 ? 1 : (DECODE ? 3 : 2)) void attn_bf16_kernel(AttnArgs a) {
+__global__ __launch_bounds__(256, D > 128 ? 1 : (DECODE && !DIRECT ? 3 : 2)) void attn_bf16_kernel(AttnArgs a) {
     // the wave's index as a scalar: its item and everything read from it then stay in scalar registers, and the
     // tests on them are scalar branches
     const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
@@ -370,9 +404,44 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : (DECODE ? 3 : 2)) void attn_bf16
     const const_int_ptr btc = (const_int_ptr)(uintptr_t)bt;
     auto page_at = [&](int j) __attribute__((always_inline)) { return btc[min(page_index(a, min(j, j_end)), last_page)]; };
     const int spare = min(max(btc[last_page], 0), a.num_pages - 1);
-    // A decoding wave asks for its first block before it turns to the query, whose loads and rotation would
+    // Direct loads: lane l brings piece l of a 1 KB run (four keys, or 32 dims of the 16 keys' values) to slot l.
+    const unsigned dk_off = (unsigned)(lane >> 4) * (2 * D) + ((unsigned)((lane & 15) ^ (lane >> 4)) << 4);
+    const unsigned dv_off = (unsigned)((lane & 15) + 16 * (lane >> 5)) * (unsigned)(2 * ps) + (unsigned)((lane >> 4) & 1) * 16u;
+    extern __shared__ __attribute__((aligned(16))) bf16_t wave_lds[];
+    const unsigned wave_lds0 = lds_address(wave_lds + wv * KV_LDS_ELEMS);
+    bool buf_ok[2];
+    auto issue = [&](int j, int pg, int buf) __attribute__((always_inline)) {     // keys j .. j + 15 -> buffer buf
+        const int j0 = min(j, j_end);
+        const int blk = page_index(a, j0);
+        buf_ok[buf] = pg >= 0 && pg < a.num_pages;
+        const int pgc = buf_ok[buf] ? pg : spare;
+        const int off = j0 - blk * ps;
+        const char* kb = (const char*)(a.k_pages + (((size_t)pgc * a.n_kv + kvh) * ps + off) * D);
+        const char* vb = (const char*)(a.v_pages + ((size_t)pgc * a.n_kv + kvh) * D * ps + off);
+        const unsigned dst = wave_lds0 + buf * (KV_BUF_ELEMS * 2);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)      // (the slot of a chunk depends on its key: four keys on, bits 2 and 3 turn)
+            load_to_lds16<DECODE>(kb + i * 1024, dk_off ^ (unsigned)(64 * i), dst + i * 1024);
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            load_to_lds16<DECODE>(vb + (size_t)(u * 32) * (2 * ps), dv_off, dst + 4096 + u * 1024);
+    };
+    // A decoding wave asks for its first blocks before it turns to the query, whose loads and rotation would
     // otherwise stand between the block table and the first keys: one round trip to memory less per launch.
-    if (DECODE && a.qkv) load_block<DECODE>(cur, a, page_at(j_first), spare, min(j_first, j_end), kvh, lane);
+    // Not a block that holds the token's own key and value, which are written below: the wave's first block
+    // (late_first), or its second (late_second), is then asked for after that.
+    const bool late_first = DECODE && a.qkv && dec_writes && min(j_first, j_end) + 16 > pos0;
+    const bool late_second = DECODE && a.qkv && dec_writes && j_first + j_step + 16 > pos0;
+    if (DECODE && a.qkv) {
+        if constexpr (DIRECT) {
+            if (!late_first) {
+                if (j_first < key_hi) issue(j_first, page_at(j_first), 0);
+                if (j_first + j_step < key_hi && !late_second) issue(j_first + j_step, page_at(j_first + j_step), 1);
+            }
+        } else {
+            load_block<DECODE>(cur, a, page_at(j_first), spare, min(j_first, j_end), kvh, lane);
+        }
+    }
 
     bool row_ok[RT];
     int ti[RT], head[RT], p[RT], p_lo[RT], tile_hi[RT], tile_lo[RT], tile_first_p[RT], tile_last_lo[RT];
@@ -468,11 +537,11 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : (DECODE ? 3 : 2)) void attn_bf16
         __syncthreads();
     }
 
-    // one block of 16 keys against the RT row tiles of this wave
-    extern __shared__ __attribute__((aligned(16))) bf16_t wave_lds[];
-    bf16_t* const kl = wave_lds + wv * KV_LDS_ELEMS;      // this wave's buffer: keys, then values
-    const bf16_t* const vl = kl + 16 * KL_ROW;
-    auto compute = [&](int j0) __attribute__((always_inline)) {
+    // one block of 16 keys (in the wave's buffer `buf`) against the RT row tiles of this wave
+    bf16_t* const kl0 = wave_lds + wv * KV_LDS_ELEMS;     // this wave's buffers: keys, then values
+    auto compute = [&](int j0, int buf) __attribute__((always_inline)) {
+        bf16_t* const kl = kl0 + buf * KV_BUF_ELEMS;
+        const bf16_t* const vl = kl + 16 * (DIRECT ? D : KL_ROW);
         wave_lds_order();
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
@@ -481,7 +550,9 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : (DECODE ? 3 : 2)) void attn_bf16
             if constexpr (WIDE) {
 #pragma unroll
                 for (int st = 0; st < QSTEPS; ++st) {
-                    U16 t; t.u = *(const uint4*)(kl + r * KL_ROW + st * 32 + g * 8);
+                    U16 t;
+                    if constexpr (DIRECT) t.u = *(const uint4*)(kl + r * D + (((4 * st + g) ^ r) << 3));
+                    else t.u = *(const uint4*)(kl + r * KL_ROW + st * 32 + g * 8);
                     s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(t.v, q8[rt][st], s, 0, 0, 0);
                 }
             } else {
@@ -503,7 +574,9 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : (DECODE ? 3 : 2)) void attn_bf16
             const bool rescale = __any(alpha != 1.f);      // the maximum of some row moved
 #pragma unroll
             for (int t = 0; t < DT; ++t) {
-                U8 vf; vf.u = *(const uint2*)(vl + (t * 16 + r) * VL_ROW + 4 * g);
+                U8 vf;
+                if constexpr (DIRECT) vf.u = *(const uint2*)(vl + ((2 * t + (g >> 1)) * 16 + r) * 8 + (g & 1) * 4);
+                else vf.u = *(const uint2*)(vl + (t * 16 + r) * VL_ROW + 4 * g);
                 if (rescale) o[rt][t] *= alpha;
                 o[rt][t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf.v, pf.v, o[rt][t], 0, 0, 0);
             }
@@ -515,20 +588,44 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : (DECODE ? 3 : 2)) void attn_bf16
     // from the block table meanwhile (a scalar load).  Every turn loads, whether or not keys are left (then the
     // wave's last block again, which nobody multiplies), so that no load sits under a branch.  (Two and three
     // buffers were slower inside whole decoding steps.)
-    if (!(DECODE && a.qkv)) {
-        load_block<DECODE>(cur, a, page_at(j_first), spare, min(j_first, j_end), kvh, lane);
-    } else if (dec_writes && min(j_first, j_end) + 16 > pos0) {
-        // the wave's first block holds the token's own key and value, which were written above: read it again
-        load_block<DECODE>(cur, a, page_at(j_first), spare, min(j_first, j_end), kvh, lane);
-    }
-    int pg_next = page_at(j_first + j_step);      // page of the next block to load
-    for (int j = j_first; j < key_hi; j += j_step) {
-        const bool ok = cur.ok;
-        if (ok) park_block(cur, kl, lane);
-        load_block<DECODE>(cur, a, pg_next, spare, min(j + j_step, j_end), kvh, lane);
-        pg_next = page_at(j + 2 * j_step);
-        __builtin_amdgcn_sched_barrier(0);
-        if (ok) compute(j);
+    if constexpr (DIRECT) {
+        // Two blocks are on their way while keys are left: the one that is multiplied next, and the one after it,
+        // which was asked for into the buffer that the last multiplication left.  (Nothing is tested around these
+        // loads for the compiler's sake, which does not know of them: a block that the wave does not have is not
+        // asked for, and the wait counts the loads that are.)
+        if (!(DECODE && a.qkv) || late_first) {
+            if (j_first < key_hi) issue(j_first, page_at(j_first), 0);
+            if (j_first + j_step < key_hi) issue(j_first + j_step, page_at(j_first + j_step), 1);
+        } else if (late_second && j_first + j_step < key_hi) {
+            issue(j_first + j_step, page_at(j_first + j_step), 1);
+        }
+        int pg_next = page_at(j_first + 2 * j_step);
+        int buf = 0;
+        for (int j = j_first; j < key_hi; j += j_step) {
+            if (j + j_step < key_hi) wait_loads<8>();       // the older of two blocks (eight loads each) has landed
+            else wait_loads<0>();
+            if (buf_ok[buf]) compute(j, buf);
+            if (j + 2 * j_step < key_hi) issue(j + 2 * j_step, pg_next, buf);
+            pg_next = page_at(j + 3 * j_step);
+            buf ^= 1;
+        }
+    } else {
+        if (!(DECODE && a.qkv)) {
+            load_block<DECODE>(cur, a, page_at(j_first), spare, min(j_first, j_end), kvh, lane);
+        } else if (late_first) {
+            // the wave's first block holds the token's own key and value, which were written above: read it again
+            load_block<DECODE>(cur, a, page_at(j_first), spare, min(j_first, j_end), kvh, lane);
+        }
+        int pg_next = page_at(j_first + j_step);      // page of the next block to load
+        bf16_t* const kl = kl0;
+        for (int j = j_first; j < key_hi; j += j_step) {
+            const bool ok = cur.ok;
+            if (ok) park_block(cur, kl, lane);
+            load_block<DECODE>(cur, a, pg_next, spare, min(j + j_step, j_end), kvh, lane);
+            pg_next = page_at(j + 2 * j_step);
+            __builtin_amdgcn_sched_barrier(0);
+            if (ok) compute(j, 0);
+        }
     }
 
     if constexpr (DECODE) {
@@ -630,27 +727,11 @@ constexpr int KROW = D + 8;                    // padded rows: operand reads fro
 constexpr int VROW = KB + 8;
 constexpr int GP = 2 * D;                      // 16-byte pieces of 16 keys (and of their values)
 constexpr int NP = (GP + 255) / 256;           // pieces per thread and group of 16 keys
-// With a head of 128 the blocks go from the pages straight into LDS (global_load_lds, 16 bytes per lane): no
-// registers hold them on the way and no thread stores them.  A wave's load writes 64 consecutive 16-byte slots of
-// LDS, one per lane, and each lane chooses what it reads from memory, so the layout is made by the choice of
-// addresses: a key row is 16 slots, and chunk c (8 dims) of LDS row p sits in slot c ^ (p % 16) of the row, so that
-// the sixteen rows of a score tile are read from sixteen different slots modulo 16 (no bank conflicts, no padding);
-// the values of a group of 16 keys are [tile of 16 dims][8 keys of 16][dim of the tile], 16 bytes each.
-constexpr bool TILE_DMA = (D == 128);
+// With a head of 128 the blocks go from the pages straight into LDS, in the layout described at DIRECT above.
+constexpr bool TILE_DMA = DIRECT;
 constexpr int KBUF = TILE_DMA ? KB * D : KB * KROW;        // elements of a key buffer, of a value buffer
 constexpr int VBUF = TILE_DMA ? D * KB : D * VROW;
 constexpr int TILE_LDS_BYTES = 2 * (KBUF + VBUF) * (int)sizeof(bf16_t);
-typedef __attribute__((address_space(3))) void* lds_void_ptr;
-// One load of a wave from memory into LDS: lane l's 16 bytes at base + off go to LDS bytes lds + 16 l .. + 15.
-// `base` and `lds` are the same in every lane.  Written as assembly because the compiler, which cannot tell the two
-// buffers of a block apart, makes every later read of LDS wait for such a load when it knows of it; here the
-// program waits itself, before the barrier behind which the buffer is read.  (The compiler's own waits for its own
-// loads stay right: loads return in order, and these only add to the number that it counts.)
-__device__ __forceinline__ void load_to_lds16(const void* base, unsigned off, unsigned lds) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                 :: "v"(off), "s"(base), "s"(lds) : "memory", "m0");
-}
-__device__ __forceinline__ unsigned lds_address(const void* p) { return (unsigned)(uintptr_t)(lds_void_ptr)p; }
 
 // key (relative to the block's first) of score tile kt, lane group g, register i
 __device__ __forceinline__ int tile_key(int kt, int g, int i) { return 32 * (kt >> 1) + 8 * g + 4 * (kt & 1) + i; }
@@ -1123,9 +1204,9 @@ extern "C" int vt_attn_bf16(const void* q, const void* k_pages, const void* v_pa
 // (item, kv head).  An item holds all the keys its rows may see (partial index -1), or one of several ranges of them:
 // then it leaves its partial result in workspace slot (partial index * 4 rt + tile) and the combine items [m][6]
 // (one per 16-row tile, as above, with 4 rt tiles per item) merge the ranges.
-// 1 if this head size's tiled kernel loads its key/value blocks straight into LDS (which decides how the host
-// cuts its work), else 0
-extern "C" int vt_attn_bf16_tiles_direct() { return TILE_DMA ? 1 : 0; }
+// 1 if this head size's kernels load their key/value blocks straight into LDS (which decides how the host cuts
+// their work), else 0
+extern "C" int vt_attn_bf16_direct() { return DIRECT ? 1 : 0; }
 
 extern "C" int vt_attn_bf16_tiles(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
                                   const int* items, int n_items, int rt, const int* citems, int n_citems, void* out,

@@ -485,10 +485,10 @@ def attention_bf16(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor
     return out
 
 
-def attention_bf16_tiles_direct(head_dim: int) -> bool:
-    """Whether the tiled kernel of this head size loads its key/value blocks straight into LDS; the host prices
-    its launches differently then (parts.attention_plan.plan_tile_items)."""
-    return bool(load_lib("vt_attn_bf16", head_dim).vt_attn_bf16_tiles_direct())
+def attention_bf16_direct(head_dim: int) -> bool:
+    """Whether the bfloat16 attention kernels of this head size load their key/value blocks straight into LDS; the
+    host cuts their work differently then (parts.attention_plan)."""
+    return bool(load_lib("vt_attn_bf16", head_dim).vt_attn_bf16_direct())
 
 
 def attention_bf16_tiles(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,

@@ -22,7 +22,7 @@ from ..config.base import PartSpec
 import numpy as np
 
 from ..kernels import ops
-from .attention_plan import decode_chunk, decode_parts_max, device_plan, plan_step
+from .attention_plan import DECODE_BLOCKS, DECODE_BLOCKS_DIRECT, decode_chunk, decode_parts_max, device_plan, plan_step
 from .base import MIXERS, POSITIONS, CacheNeed, Part, Runtime, StateNeed, TensorDecl
 from .linear import can_add_residual, linear
 
@@ -66,7 +66,7 @@ class PagedAttention(Part):
             shared[key] = POSITIONS.build(pos_spec, rt=rt)
         self.position = shared[key]
         self.w_qkv = self.b_qkv = self.b_qkv_lowp = self.w_o = self.b_o = self.p_qkv = self.p_o = None
-        self._direct_tiles: Optional[bool] = None     # asked of the kernel library at the first planned step
+        self._direct_loads: Optional[bool] = None     # asked of the kernel library at the first planned step
 
     @property
     def replayable(self) -> bool:
@@ -118,6 +118,13 @@ class PagedAttention(Part):
     def _items_key(self):
         return ("attention.items", self.nh // self.nkv, self.window, self.nkv, self.d)
 
+    def _direct(self) -> bool:
+        """Whether this head size's bfloat16 kernels load keys and values straight into LDS: the host cuts their
+        work differently then."""
+        if self._direct_loads is None:
+            self._direct_loads = ops.attention_bf16_direct(self.d)
+        return self._direct_loads
+
     def prepare_step(self, ctx) -> Optional[Dict[tuple, np.ndarray]]:
         """The integers that this step's bfloat16 attention launches read from device memory.  A decoding step
         (one token per entry): the number of keys per work item, one integer, so that a captured step can be
@@ -129,15 +136,14 @@ class PagedAttention(Part):
             key = self._decode_key()
             if key in ctx.extra_host:
                 return None
-            chunk = decode_chunk(ctx.h_kv_lens, decode_parts_max(ctx.n_positions), n_kv=self.nkv)
+            chunk = decode_chunk(ctx.h_kv_lens, decode_parts_max(ctx.n_positions), n_kv=self.nkv,
+                                 want_blocks=DECODE_BLOCKS_DIRECT if self._direct() else DECODE_BLOCKS)
             return {key: np.array([chunk], np.int32)}
         key = self._items_key()
         if key in ctx.extra_host:
             return None
-        if self._direct_tiles is None:
-            self._direct_tiles = ops.attention_bf16_tiles_direct(self.d)
         host = plan_step(ctx.h_entry_start, ctx.h_entry_pos0, self.nh // self.nkv, self.window, self.nkv, self.d,
-                         direct=self._direct_tiles)
+                         direct=self._direct())
         ctx.memo[key] = host
         return {key: host.flat()}
 

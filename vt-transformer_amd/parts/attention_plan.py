@@ -275,10 +275,15 @@ def plan_attention_items(entry_start: np.ndarray, entry_pos0: np.ndarray, group:
     return items, citems, tot_parts
 
 
-def decode_chunk(kv_lens: np.ndarray, p_max: int, n_kv: int = 4, want_blocks: int = 768, min_chunk: int = 64) -> int:
+DECODE_BLOCKS = 768          # blocks that a decoding launch is cut for: three to a compute unit
+DECODE_BLOCKS_DIRECT = 512   # ... two where the kernel's waves load straight into two LDS buffers each (head size 128)
+
+
+def decode_chunk(kv_lens: np.ndarray, p_max: int, n_kv: int = 4, want_blocks: int = DECODE_BLOCKS, min_chunk: int = 64) -> int:
     """Keys per attention item of a decoding step.  A block of four waves takes one item of one (entry, kv head);
     with enough entries every entry is one item, otherwise the keys are cut so that about `want_blocks` blocks
-    run (three to a compute unit: measured inside whole decoding steps, where the keys come from memory), never into more than p_max items; a multiple of 64 (the four waves take 16 keys each in turn)."""
+    run (as many as the GPU holds at a time: measured inside whole decoding steps, where the keys come from
+    memory), never into more than p_max items; a multiple of 64 (the four waves take 16 keys each in turn)."""
     pairs = max(1, len(kv_lens) * n_kv)
     splits = min(p_max, max(1, -(-want_blocks // pairs)))
     longest = int(kv_lens.max())
