@@ -464,36 +464,104 @@ __global__ __launch_bounds__(WPB * 64) void gemm_skinny_kernel(const void* __res
 
 // ---------------------------------------------------------------------------
 // 17 to 64 tokens per block (a large decoding batch, a short portion): a block of WM waves takes 16*WM*R features
-// and 64 tokens.  The tokens' values pass through LDS once per block (coalesced loads, two buffers), so they cost
-// a fraction of W's traffic instead of a multiple; each wave streams the tiles of its own R tile rows of W from
-// memory into registers a stage (128 k, four tiles) ahead.  For matrices with few rows the k range is split over
-// blockIdx.z and the partial sums (fp32, [split][N][M]) are added by sum_partials_kernel in split order.
+// and 64 tokens.  The tokens' values pass through LDS once per block, so they cost a fraction of W's traffic
+// instead of a multiple; each wave streams the tiles of its own R tile rows of W from memory into registers,
+// MID_WD stages (of 128 k, four tiles) ahead.  For matrices with few rows the k range is split over blockIdx.z and
+// the partial sums (fp32, [split][N][M]) are added by sum_partials_kernel in split order.
+//
+// The tokens are brought by one more wave that does nothing else: it loads them from memory straight into LDS
+// (global_load_lds, 16 bytes per lane, MID_XST - 1 stages ahead of the stage that is multiplied), so that neither a
+// stage's tokens nor its rows of W have to come within the time of one stage, which is shorter than the way from
+// memory.  A wave's load writes 64 consecutive 16-byte slots of LDS, one per lane, and each lane chooses what it
+// reads, so the layout is made by the addresses: a token's 128 values of a stage are 16 slots, and chunk c sits in
+// slot c ^ (token % 16), which keeps the sixteen rows of an operand tile on different banks without padding.
+// Only that wave has such loads in flight; the others' waits for their rows of W count what they asked for.
 // ---------------------------------------------------------------------------
 #define MID_BK 128                 // k values per stage = PK_KPAD: a stage never leaves the packed matrix
-#define MID_XROW (MID_BK + 8)
 #define MID_KU (MID_BK / 32)       // tiles along k per stage
-#define MID_PIECES (64 * MID_BK / 8) // 16-byte pieces of x per stage
+#define MID_XST 3                  // stages of tokens in LDS
+#define MID_WD 2                   // stages of W in registers (3 and 4: the same times)
+#define MID_STAGE_BYTES (64 * MID_BK * 2)
 
-// WM waves per block: the host picks it so that the blocks fill the compute units evenly.
+typedef __attribute__((address_space(3))) void* lds_void_ptr;
+// One load of a wave from memory into LDS: lane l's 16 bytes at base + off go to LDS bytes lds + 16 l .. + 15;
+// `base` and `lds` are the same in every lane.  (Assembly: the compiler makes every later read of LDS wait for such a
+// load when it knows of it, since it cannot tell the stage buffers apart; the wave that loads waits itself, before
+// the barrier behind which the stage is read.)
+__device__ __forceinline__ void load_to_lds16(const void* base, unsigned off, unsigned lds) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" :: "v"(off), "s"(base), "s"(lds) : "memory", "m0");
+}
+// wait until at most N of this wave's loads are in flight; no access to memory moves across it
+template <int N>
+__device__ __forceinline__ void wait_loads() {
+    static_assert(N >= 0 && N < 64, "the counter has six bits");
+    asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory");
+}
+
+// WM waves that multiply per block (and one that loads the tokens): the host picks it so that the blocks fill the
+// compute units evenly.
 // ONCE: one block of tokens, so that no other block reads these rows of W again (see load_w_once).
 template <int R, bool SWIGLU, int WM, typename TO, bool ONCE>
-__global__ __launch_bounds__(WM * 64) void gemm_mid_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wp,
-                                                      const float* __restrict__ bias, TO* __restrict__ y,
-                                                      float* __restrict__ partial, int N, int Mout, int K, int KT,
-                                                      int up_tiles, int k_per_split, NormLink link) {
+__global__ __launch_bounds__((WM + 1) * 64) void gemm_mid_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wp,
+                                                            const float* __restrict__ bias, TO* __restrict__ y,
+                                                            float* __restrict__ partial, int N, int Mout, int K, int KT,
+                                                            int up_tiles, int k_per_split, NormLink link) {
     constexpr int NW = SWIGLU ? 2 : 1;
     constexpr int RW = R * NW;
-    __shared__ __attribute__((aligned(16))) bf16_t xs[2][64][MID_XROW];
-    __shared__ float4 link_part[WM][16];
+    __shared__ __attribute__((aligned(1024))) bf16_t xs[MID_XST][64 * MID_BK];
+    __shared__ float4 link_part[WM + 1][16];
     __shared__ float link_rinv[64];
-    const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63;
+    const int tid = threadIdx.x, wv = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int r = lane & 15, g = lane >> 4;
     // behind a norm that the product in front has prepared (up to 64 tokens): the rows' 1/sqrt(mean + eps)
     const bool consumes = link.ssq_in != nullptr;
-    constexpr int MID_XP = (MID_PIECES + WM * 64 - 1) / (WM * 64);  // pieces of x per thread and stage
-    const int mt0 = (blockIdx.x * WM + wv) * R, n0 = blockIdx.y * 64;
+    const int n0 = blockIdx.y * 64;
     const int k_begin = blockIdx.z * k_per_split, k_end = min(pk_cols(K), k_begin + k_per_split);
+    const int S = k_begin < k_end ? (k_end - k_begin + MID_BK - 1) / MID_BK : 0;      // stages of this block
+    const bool loader = wv == WM;
+    const int mw = loader ? 0 : wv;                       // (the loading wave's sums are never stored)
+    const int mt0 = (blockIdx.x * WM + mw) * R;
     const int m_tiles = pk_rows(Mout) >> 4;
+    f32x4_t acc[RW][4];
+#pragma unroll
+    for (int a = 0; a < RW; ++a)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[a][i] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+
+    if (loader) {
+        // A stage is 16 loads of four tokens each: lane l brings chunk (l % 16) ^ (token % 16) of token 4 i + l / 16
+        // to slot l.  Tokens beyond the last repeat it; k beyond the row reads the row's last chunk again (the
+        // packed matrix is zero there).
+        const unsigned lds0 = (unsigned)(uintptr_t)(lds_void_ptr)&xs[0][0];
+        unsigned tok_off[16];
+        int chunk_k[4];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) tok_off[i] = (unsigned)min(n0 + 4 * i + (lane >> 4), N - 1) * (unsigned)K * 2u;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) chunk_k[i] = 8 * ((lane & 15) ^ ((4 * i + (lane >> 4)) & 15));
+        auto issue = [&](int st) __attribute__((always_inline)) {
+            const int k0 = k_begin + st * MID_BK;
+            const unsigned dst = lds0 + (unsigned)(st % MID_XST) * MID_STAGE_BYTES;
+#pragma unroll
+            for (int i = 0; i < 16; ++i)
+                load_to_lds16(x, tok_off[i] + 2u * (unsigned)min(k0 + chunk_k[i & 3], K - 8), dst + i * 1024);
+        };
+#pragma unroll
+        for (int st = 0; st < MID_XST - 1; ++st)
+            if (st < S) issue(st);
+        if (consumes) link_row_scales<(WM + 1) * 64>(link, K, link_part, link_rinv);
+        for (int st = 0; st < S; ++st) {
+            // stage st has landed when no more loads are in flight than those of the stages asked for after it
+            const int later = min(st + MID_XST - 1, S) - (st + 1);
+            if (later >= 2) wait_loads<32>();
+            else if (later == 1) wait_loads<16>();
+            else wait_loads<0>();
+            __syncthreads();
+            // every wave has left stage st - 1, whose buffer the stage MID_XST - 1 ahead takes
+            if (st + MID_XST - 1 < S) issue(st + MID_XST - 1);
+        }
+        return;
+    }
 
     // this wave's tile rows; beyond the matrix the last one again (its results are not stored)
     const bf16_t* wbase[RW];
@@ -503,38 +571,9 @@ __global__ __launch_bounds__(WM * 64) void gemm_mid_kernel(const bf16_t* __restr
         wbase[j] = wp + ((size_t)mt * KT * 64 + lane) * 8;
         if (SWIGLU) wbase[R + j] = wp + ((size_t)(mt + up_tiles) * KT * 64 + lane) * 8;
     }
-    // this thread's 16-byte pieces of a stage of x: a token's MID_BK values are MID_BK/8 consecutive pieces
-    const bf16_t* xsrc[MID_XP];
-    int xtok[MID_XP], xcol[MID_XP];
-#pragma unroll
-    for (int q = 0; q < MID_XP; ++q) {
-        const int pidx = min(tid + WM * 64 * q, MID_PIECES - 1);  // spare threads repeat the last piece
-        xtok[q] = pidx / (MID_BK / 8);
-        xcol[q] = (pidx % (MID_BK / 8)) * 8;
-        xsrc[q] = x + (size_t)min(n0 + xtok[q], N - 1) * K;
-    }
-    f32x4_t acc[RW][4];
-#pragma unroll
-    for (int a = 0; a < RW; ++a)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) acc[a][i] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
-
-    uint4 xreg[MID_XP];
-    Frag wcur[RW][MID_KU], wnxt[RW][MID_KU];
-    auto fetch_x = [&](int k0) __attribute__((always_inline)) {
-#pragma unroll
-        for (int q = 0; q < MID_XP; ++q) {
-            Frag f;
-            f.v = load_x(xsrc[q], k0 + xcol[q], K);
-            xreg[q] = f.u;
-        }
-    };
-    auto park_x = [&](int buf) __attribute__((always_inline)) {
-#pragma unroll
-        for (int q = 0; q < MID_XP; ++q) *(uint4*)&xs[buf][xtok[q]][xcol[q]] = xreg[q];
-    };
-    auto fetch_w = [&](Frag (&dst)[RW][MID_KU], int k0) __attribute__((always_inline)) {
-        const size_t t0 = (size_t)(k0 >> 5) * PK_TILE;
+    Frag wst[MID_WD][RW][MID_KU];
+    auto fetch_w = [&](Frag (&dst)[RW][MID_KU], int st) __attribute__((always_inline)) {
+        const size_t t0 = (size_t)((k_begin + st * MID_BK) >> 5) * PK_TILE;
 #pragma unroll
         for (int u = 0; u < MID_KU; ++u)
 #pragma unroll
@@ -544,43 +583,46 @@ __global__ __launch_bounds__(WM * 64) void gemm_mid_kernel(const bf16_t* __restr
                 else dst[a][u].u = *(const uint4*)src;
             }
     };
-    auto multiply = [&](const Frag (&wf)[RW][MID_KU], int buf) __attribute__((always_inline)) {
+    // token 16 i + r's chunk 4 u + g of stage buffer b
+    const bf16_t* const xrd = &xs[0][0] + r * MID_BK;
+    int xsw[MID_KU];
+#pragma unroll
+    for (int u = 0; u < MID_KU; ++u) xsw[u] = ((4 * u + g) ^ r) << 3;
+    auto multiply = [&](const Frag (&wf)[RW][MID_KU], int st) __attribute__((always_inline)) {
+        const bf16_t* const xb = xrd + (st % MID_XST) * (64 * MID_BK);
+        // all of the stage's token operands are asked for before the first product: a wave is alone on its SIMD when
+        // a block has a compute unit to itself, and read two at a time the way from LDS is waited for eight times
+        Frag xf[MID_KU][4];
 #pragma unroll
         for (int u = 0; u < MID_KU; ++u)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                Frag xf;
-                xf.u = *(const uint4*)&xs[buf][i * 16 + r][u * 32 + g * 8];
+            for (int i = 0; i < 4; ++i) xf[u][i].u = *(const uint4*)(xb + i * 16 * MID_BK + xsw[u]);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < MID_KU; ++u)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
 #pragma unroll
                 for (int a = 0; a < RW; ++a)
-                    acc[a][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[a][u].v, xf.v, acc[a][i], 0, 0, 0);
-            }
+                    acc[a][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[a][u].v, xf[u][i].v, acc[a][i], 0, 0, 0);
     };
-
-    if (k_begin < k_end) {
-        // x first: loads finish in the order they were issued, and parking x must not wait for W
-        fetch_x(k_begin);
-        fetch_w(wcur, k_begin);
-        // (here, behind the first stage's loads, the shares' way from the second-level cache costs nothing)
-        if (consumes) link_row_scales<WM * 64>(link, K, link_part, link_rinv);
-        park_x(0);
-        __syncthreads();
-        // two stages per turn so that the register buffers alternate without copies
-        for (int k0 = k_begin; k0 < k_end; k0 += 2 * MID_BK) {
-            const int k1 = k0 + MID_BK, k2 = k0 + 2 * MID_BK;
-            if (k1 < k_end) { fetch_x(k1); fetch_w(wnxt, k1); }
-            multiply(wcur, 0);
-            if (k1 < k_end) park_x(1);
-            __syncthreads();
-            if (k1 >= k_end) break;
-            if (k2 < k_end) { fetch_x(k2); fetch_w(wcur, k2); }
-            multiply(wnxt, 1);
-            if (k2 < k_end) park_x(0);
-            __syncthreads();
+#pragma unroll
+    for (int d = 0; d < MID_WD; ++d)
+        if (d < S) fetch_w(wst[d], d);
+    // (here, behind the first stages' loads, the shares' way from the second-level cache costs nothing)
+    if (consumes) link_row_scales<(WM + 1) * 64>(link, K, link_part, link_rinv);
+    // MID_WD stages per turn so that the register stages rotate without copies; one barrier per stage, which the
+    // loading wave meets when the stage's tokens have landed
+    for (int st = 0; st < S; st += MID_WD) {
+#pragma unroll
+        for (int d = 0; d < MID_WD; ++d) {
+            if (st + d < S) {
+                __syncthreads();
+                multiply(wst[d], st + d);
+                if (st + d + MID_WD < S) fetch_w(wst[d], st + d + MID_WD);
+            }
         }
     }
-
-    else if (consumes) link_row_scales<WM * 64>(link, K, link_part, link_rinv);
 
     // acc[a][i][e] is feature 16 (mt0 + j) + 4 g + e (j = a mod R) of token n0 + 16 i + r
     const bool split = gridDim.z > 1;
@@ -983,7 +1025,7 @@ static int linear_bf16(const void* xv, const bf16_t* wp, const float* bias, TO* 
         // the product takes the norm in front (link.ssq_in); the one behind is prepared where the sums are added up
         NormLink in = NO_LINK;
         in.ssq_in = link.ssq_in; in.n_ssq = link.n_ssq; in.eps = link.eps;
-#define VT_MID_(W, O) gemm_mid_kernel<RR, SWIGLU, W, TO, O><<<grid, W * 64, 0, stream>>>(x, wp, bias, y, workspace, N, Mout, K, KT, up_tiles, kps, in)
+#define VT_MID_(W, O) gemm_mid_kernel<RR, SWIGLU, W, TO, O><<<grid, (W + 1) * 64, 0, stream>>>(x, wp, bias, y, workspace, N, Mout, K, KT, up_tiles, kps, in)
 #define VT_MID(W) do { if (grid.y == 1) VT_MID_(W, true); else VT_MID_(W, false); } while (0)
         if (wm == 4) VT_MID(4);
         else if (wm == 5) VT_MID(5);
