@@ -481,7 +481,9 @@ __global__ __launch_bounds__(WPB * 64) void gemm_skinny_kernel(const void* __res
 #define MID_KU (MID_BK / 32)       // tiles along k per stage
 #define MID_XST 3                  // stages of tokens in LDS
 #define MID_WD 2                   // stages of W in registers (3 and 4: the same times)
-#define MID_STAGE_BYTES (64 * MID_BK * 2)
+// bytes of a stage of NTT token tiles in LDS, and of a block's stages
+#define MID_STAGE_BYTES(NTT) ((NTT) * 16 * MID_BK * 2)
+#define MID_LDS_BYTES(NTT) (MID_XST * MID_STAGE_BYTES(NTT))
 
 typedef __attribute__((address_space(3))) void* lds_void_ptr;
 // One load of a wave from memory into LDS: lane l's 16 bytes at base + off go to LDS bytes lds + 16 l .. + 15;
@@ -499,51 +501,54 @@ __device__ __forceinline__ void wait_loads() {
 }
 
 // WM waves that multiply per block (and one that loads the tokens): the host picks it so that the blocks fill the
-// compute units evenly.
+// compute units evenly.  NTT: token tiles of 16 per block, 4 (up to 64 tokens in a launch) or 8 (more: W is then
+// read once per 128 tokens).
 // ONCE: one block of tokens, so that no other block reads these rows of W again (see load_w_once).
-template <int R, bool SWIGLU, int WM, typename TO, bool ONCE>
+template <int R, bool SWIGLU, int WM, typename TO, bool ONCE, int NTT>
 __global__ __launch_bounds__((WM + 1) * 64) void gemm_mid_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wp,
                                                             const float* __restrict__ bias, TO* __restrict__ y,
                                                             float* __restrict__ partial, int N, int Mout, int K, int KT,
                                                             int up_tiles, int k_per_split, NormLink link) {
     constexpr int NW = SWIGLU ? 2 : 1;
     constexpr int RW = R * NW;
-    __shared__ __attribute__((aligned(1024))) bf16_t xs[MID_XST][64 * MID_BK];
+    extern __shared__ __attribute__((aligned(1024))) bf16_t xs[];      // [MID_XST][NTT * 16 * MID_BK]
     __shared__ float4 link_part[WM + 1][16];
     __shared__ float link_rinv[64];
     const int tid = threadIdx.x, wv = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int r = lane & 15, g = lane >> 4;
     // behind a norm that the product in front has prepared (up to 64 tokens): the rows' 1/sqrt(mean + eps)
     const bool consumes = link.ssq_in != nullptr;
-    const int n0 = blockIdx.y * 64;
+    const int n0 = blockIdx.y * (NTT * 16);
     const int k_begin = blockIdx.z * k_per_split, k_end = min(pk_cols(K), k_begin + k_per_split);
     const int S = k_begin < k_end ? (k_end - k_begin + MID_BK - 1) / MID_BK : 0;      // stages of this block
     const bool loader = wv == WM;
     const int mw = loader ? 0 : wv;                       // (the loading wave's sums are never stored)
     const int mt0 = (blockIdx.x * WM + mw) * R;
     const int m_tiles = pk_rows(Mout) >> 4;
-    f32x4_t acc[RW][4];
+    f32x4_t acc[RW][NTT];
 #pragma unroll
     for (int a = 0; a < RW; ++a)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) acc[a][i] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+        for (int i = 0; i < NTT; ++i) acc[a][i] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 
     if (loader) {
-        // A stage is 16 loads of four tokens each: lane l brings chunk (l % 16) ^ (token % 16) of token 4 i + l / 16
+        // A stage is 4 NTT loads of four tokens each: lane l brings chunk (l % 16) ^ (token % 16) of token 4 i + l / 16
         // to slot l.  Tokens beyond the last repeat it; k beyond the row reads the row's last chunk again (the
         // packed matrix is zero there).
-        const unsigned lds0 = (unsigned)(uintptr_t)(lds_void_ptr)&xs[0][0];
-        unsigned tok_off[16];
+        constexpr int NL = 4 * NTT;      // loads per stage
+        static_assert(NL < 64, "the wait for a stage counts its loads in six bits");
+        const unsigned lds0 = (unsigned)(uintptr_t)(lds_void_ptr)xs;
+        unsigned tok_off[NL];
         int chunk_k[4];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) tok_off[i] = (unsigned)min(n0 + 4 * i + (lane >> 4), N - 1) * (unsigned)K * 2u;
+        for (int i = 0; i < NL; ++i) tok_off[i] = (unsigned)min(n0 + 4 * i + (lane >> 4), N - 1) * (unsigned)K * 2u;
 #pragma unroll
         for (int i = 0; i < 4; ++i) chunk_k[i] = 8 * ((lane & 15) ^ ((4 * i + (lane >> 4)) & 15));
         auto issue = [&](int st) __attribute__((always_inline)) {
             const int k0 = k_begin + st * MID_BK;
-            const unsigned dst = lds0 + (unsigned)(st % MID_XST) * MID_STAGE_BYTES;
+            const unsigned dst = lds0 + (unsigned)(st % MID_XST) * MID_STAGE_BYTES(NTT);
 #pragma unroll
-            for (int i = 0; i < 16; ++i)
+            for (int i = 0; i < NL; ++i)
                 load_to_lds16(x, tok_off[i] + 2u * (unsigned)min(k0 + chunk_k[i & 3], K - 8), dst + i * 1024);
         };
 #pragma unroll
@@ -552,9 +557,9 @@ __global__ __launch_bounds__((WM + 1) * 64) void gemm_mid_kernel(const bf16_t* _
         if (consumes) link_row_scales<(WM + 1) * 64>(link, K, link_part, link_rinv);
         for (int st = 0; st < S; ++st) {
             // stage st has landed when no more loads are in flight than those of the stages asked for after it
+            static_assert(MID_XST == 3, "at most one stage is asked for behind the one that is waited for");
             const int later = min(st + MID_XST - 1, S) - (st + 1);
-            if (later >= 2) wait_loads<32>();
-            else if (later == 1) wait_loads<16>();
+            if (later == 1) wait_loads<NL>();
             else wait_loads<0>();
             __syncthreads();
             // every wave has left stage st - 1, whose buffer the stage MID_XST - 1 ahead takes
@@ -584,27 +589,31 @@ __global__ __launch_bounds__((WM + 1) * 64) void gemm_mid_kernel(const bf16_t* _
             }
     };
     // token 16 i + r's chunk 4 u + g of stage buffer b
-    const bf16_t* const xrd = &xs[0][0] + r * MID_BK;
+    const bf16_t* const xrd = xs + r * MID_BK;
     int xsw[MID_KU];
 #pragma unroll
     for (int u = 0; u < MID_KU; ++u) xsw[u] = ((4 * u + g) ^ r) << 3;
     auto multiply = [&](const Frag (&wf)[RW][MID_KU], int st) __attribute__((always_inline)) {
-        const bf16_t* const xb = xrd + (st % MID_XST) * (64 * MID_BK);
-        // all of the stage's token operands are asked for before the first product: a wave is alone on its SIMD when
-        // a block has a compute unit to itself, and read two at a time the way from LDS is waited for eight times
-        Frag xf[MID_KU][4];
+        const bf16_t* const xb = xrd + (st % MID_XST) * (NTT * 16 * MID_BK);
+        // 16 token operands are asked for together, ahead of their products: a wave is alone on its SIMD when a
+        // block has a compute unit to itself, and read two at a time the way from LDS is waited for eight times
+        constexpr int UB = 16 / NTT;     // k tiles whose operands are read together
 #pragma unroll
-        for (int u = 0; u < MID_KU; ++u)
+        for (int u0 = 0; u0 < MID_KU; u0 += UB) {
+            Frag xf[UB][NTT];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) xf[u][i].u = *(const uint4*)(xb + i * 16 * MID_BK + xsw[u]);
-        __builtin_amdgcn_sched_barrier(0);
+            for (int u = 0; u < UB; ++u)
 #pragma unroll
-        for (int u = 0; u < MID_KU; ++u)
+                for (int i = 0; i < NTT; ++i) xf[u][i].u = *(const uint4*)(xb + i * 16 * MID_BK + xsw[u0 + u]);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
+            for (int u = 0; u < UB; ++u)
 #pragma unroll
-                for (int a = 0; a < RW; ++a)
-                    acc[a][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[a][u].v, xf[u][i].v, acc[a][i], 0, 0, 0);
+                for (int i = 0; i < NTT; ++i)
+#pragma unroll
+                    for (int a = 0; a < RW; ++a)
+                        acc[a][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[a][u0 + u].v, xf[u][i].v, acc[a][i], 0, 0, 0);
+        }
     };
 #pragma unroll
     for (int d = 0; d < MID_WD; ++d)
@@ -629,17 +638,17 @@ __global__ __launch_bounds__((WM + 1) * 64) void gemm_mid_kernel(const bf16_t* _
 #pragma unroll
     for (int j = 0; j < R; ++j)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < NTT; ++i) {
             const int n = n0 + i * 16 + r;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const int m = (mt0 + j) * 16 + 4 * g + e;
                 if (m >= Mout || n >= N) continue;
                 float v = acc[j][i][e];
-                if (consumes) v *= link_rinv[i * 16 + r];
+                if (consumes) v *= link_rinv[(i * 16 + r) & 63];      // (a norm is taken over with up to 64 tokens)
                 if (SWIGLU) {
                     float u = acc[R + j][i][e];
-                    if (consumes) u *= link_rinv[i * 16 + r];
+                    if (consumes) u *= link_rinv[(i * 16 + r) & 63];
                     v = v / (1.f + expf(-v)) * u;
                 } else if (bias && blockIdx.z == 0) {
                     v += bias[m];
@@ -1016,8 +1025,10 @@ static int linear_bf16(const void* xv, const bf16_t* wp, const float* bias, TO* 
         const int splits = SWIGLU ? 1 : mid_splits(Mout, K, 64 * RR);
         VT_REQUIRE(splits == 1 || workspace, "vt_linear_bf16: this shape needs a workspace (vt_linear_bf16_workspace)");
         int kps = ((pk_cols(K) + splits - 1) / splits + MID_BK - 1) / MID_BK * MID_BK;
-        const int wm = SWIGLU ? mid_waves(Mout, 16 * RR, (N + 63) / 64) : 4;
-        dim3 grid((Mout + 16 * wm * RR - 1) / (16 * wm * RR), (N + 63) / 64, splits);
+        // more than 64 tokens: 128 per block, so that W is read once per 128
+        const int tok = N > 64 ? 128 : 64, token_blocks = (N + tok - 1) / tok;
+        const int wm = SWIGLU ? mid_waves(Mout, 16 * RR, token_blocks) : 4;
+        dim3 grid((Mout + 16 * wm * RR - 1) / (16 * wm * RR), token_blocks, splits);
         VT_REQUIRE(grid.y <= 65535, "vt_linear_bf16: too many rows (%d)", N);
         VT_REQUIRE(!(resid || link.xn_out) || (splits > 1 && N <= ROWS_MAX && Mout % 4 == 0 && sizeof(TO) == 4),
                    "vt_linear_bf16: %d rows of [%d, %d] do not take a residual (vt_linear_bf16_adds_residual)", N, Mout, K);
@@ -1025,7 +1036,16 @@ static int linear_bf16(const void* xv, const bf16_t* wp, const float* bias, TO* 
         // the product takes the norm in front (link.ssq_in); the one behind is prepared where the sums are added up
         NormLink in = NO_LINK;
         in.ssq_in = link.ssq_in; in.n_ssq = link.n_ssq; in.eps = link.eps;
-#define VT_MID_(W, O) gemm_mid_kernel<RR, SWIGLU, W, TO, O><<<grid, (W + 1) * 64, 0, stream>>>(x, wp, bias, y, workspace, N, Mout, K, KT, up_tiles, kps, in)
+#define VT_MID__(W, O, T) do { \
+            static bool lds_set = false; \
+            if (!lds_set) { \
+                hipError_t e = hipFuncSetAttribute((const void*)gemm_mid_kernel<RR, SWIGLU, W, TO, O, T>, hipFuncAttributeMaxDynamicSharedMemorySize, MID_LDS_BYTES(T)); \
+                VT_REQUIRE(e == hipSuccess, "vt_linear_bf16: cannot get %d bytes of LDS: %s", MID_LDS_BYTES(T), hipGetErrorString(e)); \
+                lds_set = true; \
+            } \
+            gemm_mid_kernel<RR, SWIGLU, W, TO, O, T><<<grid, (W + 1) * 64, MID_LDS_BYTES(T), stream>>>(x, wp, bias, y, workspace, N, Mout, K, KT, up_tiles, kps, in); \
+        } while (0)
+#define VT_MID_(W, O) do { if (tok == 64) VT_MID__(W, O, 4); else VT_MID__(W, O, 8); } while (0)
 #define VT_MID(W) do { if (grid.y == 1) VT_MID_(W, true); else VT_MID_(W, false); } while (0)
         if (wm == 4) VT_MID(4);
         else if (wm == 5) VT_MID(5);
@@ -1033,6 +1053,7 @@ static int linear_bf16(const void* xv, const bf16_t* wp, const float* bias, TO* 
         else VT_MID(8);
 #undef VT_MID
 #undef VT_MID_
+#undef VT_MID__
         VT_CHECK_LAUNCH("vt_linear_bf16(64 tokens)");
         if (splits > 1) {
             const size_t n = (size_t)N * Mout;

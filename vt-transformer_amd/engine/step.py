@@ -92,7 +92,7 @@ class _DecodeGraph:
         self.wanted = None          # the view of `logits` that the last step returned
 
 
-GRAPH_BATCHES = (1, 2, 4, 8, 16, 32, 64)
+GRAPH_BATCHES = (1, 2, 4, 8, 16, 32, 64, 96, 128)
 
 
 class ModelRunner:

@@ -22,6 +22,9 @@ SKINNY_MAX_ROWS = 64
 # ... and up to this many for a matrix with few rows and a long k (the down projection), where the GEMM library is
 # at its worst: 59 against 99 us at 128 rows of 3,584 x 18,944, 86 against 125 us at 256 (measured)
 LONG_K_MAX_ROWS = 256
+# ... and up to this many for the gated pair of matrices (gate/up), 128 rows to a block: one launch that also
+# applies the gate against the library's product and a gating kernel behind it
+GATED_MAX_ROWS = 128
 
 
 # A model that keeps the packed copy only: from this many rows on, a product unpacks its matrix into scratch memory
