@@ -92,7 +92,8 @@ class _DecodeGraph:
         self.wanted = None          # the view of `logits` that the last step returned
 
 
-GRAPH_BATCHES = (1, 2, 4, 8, 16, 32, 64, 96, 128)
+# (captured steps of 256 entries are slower than launched ones: 11.3 against 10.8 ms at 7B sizes; of 192 faster, 9.7 against 10.8)
+GRAPH_BATCHES = (1, 2, 4, 8, 16, 32, 64, 96, 128, 192)
 
 
 class ModelRunner:
