@@ -162,28 +162,6 @@ constexpr int KL_ROW = D + 8, VL_ROW = 24;        // padded LDS rows: operand re
 // the sixteen rows of a score tile are read from sixteen different slots modulo 16 (no bank conflicts, no padding);
 // the values of a group of 16 keys are [tile of 16 dims][8 keys of 16][dim of the tile], 16 bytes each.
 constexpr bool DIRECT = (D == 128);
-typedef __attribute__((address_space(3))) void* lds_void_ptr;
-// One load of a wave from memory into LDS: lane l's 16 bytes at base + off go to LDS bytes lds + 16 l .. + 15.
-// `base` and `lds` are the same in every lane.  Written as assembly because the compiler, which cannot tell the
-// buffers of a block apart, makes every later read of LDS wait for such a load when it knows of it; here the
-// program waits itself before it reads a buffer.  (The compiler's own waits for its own loads stay right: loads
-// return in order, and these only add to the number that it counts.)  ONCE: no other wave reads these bytes.
-template <bool ONCE = false>
-__device__ __forceinline__ void load_to_lds16(const void* base, unsigned off, unsigned lds) {
-    if constexpr (ONCE)
-        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 nt"
-                     :: "v"(off), "s"(base), "s"(lds) : "memory", "m0");
-    else
-        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                     :: "v"(off), "s"(base), "s"(lds) : "memory", "m0");
-}
-__device__ __forceinline__ unsigned lds_address(const void* p) { return (unsigned)(uintptr_t)(lds_void_ptr)p; }
-// wait until at most N of this wave's loads are in flight; no access to memory moves across it
-template <int N>
-__device__ __forceinline__ void wait_loads() {
-    static_assert(N >= 0 && N < 16, "the count's low four bits");
-    asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory");
-}
 // (direct: two buffers per wave of 16 keys and their values as they come, the next block but one is on its way
 // while a block is multiplied)
 constexpr int WAVE_BUFS = DIRECT ? 2 : 1;

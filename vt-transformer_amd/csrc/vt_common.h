@@ -71,6 +71,35 @@ __device__ __forceinline__ void wave_lds_order() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// ---------------------------------------------------------------------------
+// Loads from memory straight into LDS (global_load_lds_dwordx4, 16 bytes per lane).  A wave's load writes 64
+// consecutive 16-byte slots of LDS, one per lane, and every lane chooses its own address in memory: lane l's 16
+// bytes at base + off go to LDS bytes lds + 16 l .. + 15; `base` and `lds` are the same in every lane.  No register
+// holds the data on its way and no thread stores it, and the layout in LDS is made by the choice of addresses.
+// Written as assembly: when the compiler knows of such a load it makes every later read of LDS wait for it, since
+// it cannot tell one buffer from another; the program waits itself (wait_loads) before it reads what has landed.
+// The compiler's own waits for its own loads stay right: loads return in the order they were asked for, and these
+// only add to the number that it counts.  ONCE: no other wave reads these bytes (a non-temporal load).
+// ---------------------------------------------------------------------------
+typedef __attribute__((address_space(3))) void* vt_lds_void_ptr;
+template <bool ONCE = false>
+__device__ __forceinline__ void load_to_lds16(const void* base, unsigned off, unsigned lds) {
+    if constexpr (ONCE)
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 nt"
+                     :: "v"(off), "s"(base), "s"(lds) : "memory", "m0");
+    else
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                     :: "v"(off), "s"(base), "s"(lds) : "memory", "m0");
+}
+// the address in LDS of an object there, as the loads above want it
+__device__ __forceinline__ unsigned lds_address(const void* p) { return (unsigned)(uintptr_t)(vt_lds_void_ptr)p; }
+// wait until at most N of this wave's loads are in flight; no access to memory moves across it
+template <int N>
+__device__ __forceinline__ void wait_loads() {
+    static_assert(N >= 0 && N < 64, "the counter has six bits");
+    asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory");
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);

@@ -485,21 +485,6 @@ __global__ __launch_bounds__(WPB * 64) void gemm_skinny_kernel(const void* __res
 #define MID_STAGE_BYTES(NTT) ((NTT) * 16 * MID_BK * 2)
 #define MID_LDS_BYTES(NTT) (MID_XST * MID_STAGE_BYTES(NTT))
 
-typedef __attribute__((address_space(3))) void* lds_void_ptr;
-// One load of a wave from memory into LDS: lane l's 16 bytes at base + off go to LDS bytes lds + 16 l .. + 15;
-// `base` and `lds` are the same in every lane.  (Assembly: the compiler makes every later read of LDS wait for such a
-// load when it knows of it, since it cannot tell the stage buffers apart; the wave that loads waits itself, before
-// the barrier behind which the stage is read.)
-__device__ __forceinline__ void load_to_lds16(const void* base, unsigned off, unsigned lds) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" :: "v"(off), "s"(base), "s"(lds) : "memory", "m0");
-}
-// wait until at most N of this wave's loads are in flight; no access to memory moves across it
-template <int N>
-__device__ __forceinline__ void wait_loads() {
-    static_assert(N >= 0 && N < 64, "the counter has six bits");
-    asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory");
-}
-
 // WM waves that multiply per block (and one that loads the tokens): the host picks it so that the blocks fill the
 // compute units evenly.  NTT: token tiles of 16 per block, 4 (up to 64 tokens in a launch) or 8 (more: W is then
 // read once per 128 tokens).
@@ -537,7 +522,7 @@ __global__ __launch_bounds__((WM + 1) * 64) void gemm_mid_kernel(const bf16_t* _
         // packed matrix is zero there).
         constexpr int NL = 4 * NTT;      // loads per stage
         static_assert(NL < 64, "the wait for a stage counts its loads in six bits");
-        const unsigned lds0 = (unsigned)(uintptr_t)(lds_void_ptr)xs;
+        const unsigned lds0 = lds_address(xs);
         unsigned tok_off[NL];
         int chunk_k[4];
 #pragma unroll
