@@ -687,7 +687,8 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : (DECODE && !DIRECT ? 3 : 2)) voi
 // Long portions of prompts: a block of 4 waves takes 64 * RT consecutive rows of one (entry, kv head) and walks
 // their keys KB at a time.  Every key/value block is fetched from the pages once per block of waves, by all 256
 // threads together with 16-byte loads, and parked in LDS (two buffers: the next block comes from memory into
-// registers while this one is multiplied, and is parked in the other buffer afterwards); the four waves read their
+// registers while this one is multiplied, and is parked in the other buffer afterwards; with a head of 128 it comes
+// from memory straight into the other buffer, see DIRECT); the four waves read their
 // matrix operands from there, each operand once for all RT row tiles of the wave.  Rows of an item that lie wholly
 // above a key block skip it (the upper triangle of a causal portion costs nothing).
 //
@@ -706,9 +707,8 @@ constexpr int VROW = KB + 8;
 constexpr int GP = 2 * D;                      // 16-byte pieces of 16 keys (and of their values)
 constexpr int NP = (GP + 255) / 256;           // pieces per thread and group of 16 keys
 // With a head of 128 the blocks go from the pages straight into LDS, in the layout described at DIRECT above.
-constexpr bool TILE_DMA = DIRECT;
-constexpr int KBUF = TILE_DMA ? KB * D : KB * KROW;        // elements of a key buffer, of a value buffer
-constexpr int VBUF = TILE_DMA ? D * KB : D * VROW;
+constexpr int KBUF = DIRECT ? KB * D : KB * KROW;        // elements of a key buffer, of a value buffer
+constexpr int VBUF = DIRECT ? D * KB : D * VROW;
 constexpr int TILE_LDS_BYTES = 2 * (KBUF + VBUF) * (int)sizeof(bf16_t);
 
 // key (relative to the block's first) of score tile kt, lane group g, register i
@@ -972,12 +972,12 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_tile_kernel(At
         for (int kt = 0; kt < KT; ++kt) {
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) s[rt][kt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
-            const bf16_t* kr = kd + (kt * 16 + r) * (TILE_DMA ? D : KROW);
+            const bf16_t* kr = kd + (kt * 16 + r) * (DIRECT ? D : KROW);
             if constexpr (WIDE) {
 #pragma unroll
                 for (int st = 0; st < QSTEPS; ++st) {
                     U16 t;
-                    if constexpr (TILE_DMA) t.u = *(const uint4*)(kr + (((4 * st + g) ^ r) << 3));
+                    if constexpr (DIRECT) t.u = *(const uint4*)(kr + (((4 * st + g) ^ r) << 3));
                     else t.u = *(const uint4*)(kr + st * 32 + g * 8);
 #pragma unroll
                     for (int rt = 0; rt < RT; ++rt)
@@ -1019,7 +1019,7 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_tile_kernel(At
 #pragma unroll
             for (int t = 0; t < DT; ++t) {
                 U16 vf;
-                if constexpr (TILE_DMA) vf.u = *(const uint4*)(vd + (2 * h + (g >> 1)) * 2048 + ((2 * t + (g & 1)) * 16 + r) * 8);
+                if constexpr (DIRECT) vf.u = *(const uint4*)(vd + (2 * h + (g >> 1)) * 2048 + ((2 * t + (g & 1)) * 16 + r) * 8);
                 else vf.u = *(const uint4*)(vd + (t * 16 + r) * VROW + 32 * h + 8 * g);
 #pragma unroll
                 for (int rt = 0; rt < RT; ++rt)
@@ -1029,7 +1029,7 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_tile_kernel(At
     };
 
     int buf = 0;
-    if constexpr (TILE_DMA) {
+    if constexpr (DIRECT) {
         dma_pages();
         fetch_dma(0);
         __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0): this wave's pieces are in LDS
