@@ -526,7 +526,8 @@ __global__ __launch_bounds__((WM + 1) * 64) void gemm_mid_kernel(const bf16_t* _
         unsigned tok_off[NL];
         int chunk_k[4];
 #pragma unroll
-        for (int i = 0; i < NL; ++i) tok_off[i] = (unsigned)min(n0 + 4 * i + (lane >> 4), N - 1) * (unsigned)K * 2u;
+        for (int i = 0; i < NL; ++i) tok_off[i] = (unsigned)min(4 * i + (lane >> 4), N - 1 - n0) * (unsigned)K * 2u;
+        const bf16_t* const xblk = x + (size_t)n0 * K;       // (32-bit offsets from the block's first token)
 #pragma unroll
         for (int i = 0; i < 4; ++i) chunk_k[i] = 8 * ((lane & 15) ^ ((4 * i + (lane >> 4)) & 15));
         auto issue = [&](int st) __attribute__((always_inline)) {
@@ -534,7 +535,7 @@ __global__ __launch_bounds__((WM + 1) * 64) void gemm_mid_kernel(const bf16_t* _
             const unsigned dst = lds0 + (unsigned)(st % MID_XST) * MID_STAGE_BYTES(NTT);
 #pragma unroll
             for (int i = 0; i < NL; ++i)
-                load_to_lds16(x, tok_off[i] + 2u * (unsigned)min(k0 + chunk_k[i & 3], K - 8), dst + i * 1024);
+                load_to_lds16(xblk, tok_off[i] + 2u * (unsigned)min(k0 + chunk_k[i & 3], K - 8), dst + i * 1024);
         };
 #pragma unroll
         for (int st = 0; st < MID_XST - 1; ++st)
