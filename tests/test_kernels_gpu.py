@@ -239,10 +239,10 @@ def test_linear_bf16_batch_invariant():
     assert rel_err(small, full[:16]) < 1e-5
 
 
-@pytest.mark.parametrize("n", [1, 9, 40, 64, 300])
+@pytest.mark.parametrize("n", [1, 9, 40, 64, 100, 128, 300])
 @pytest.mark.parametrize("inter,k", [(200, 96), (128, 64), (1184, 3584), (18944, 40), (22016, 32), (29568, 24)])
 def test_gated_linear_bf16(n, inter, k):
-    # the three wide ones make the 64-token kernel take 5, 6 and 8 waves a block
+    # the three wide ones make the 64-token kernel take 5, 6 and 8 waves a block; from 65 rows on a block takes 128 tokens
     g = torch.Generator().manual_seed(10)
     x = torch.randn(n, k, generator=g).to(torch.bfloat16)
     w = (torch.randn(2 * inter, k, generator=g) * 0.05).to(torch.bfloat16)
