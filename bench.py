@@ -45,6 +45,8 @@ def main() -> int:
     ap.add_argument("--prompt-len", type=int, default=1024)
     ap.add_argument("--sizes", choices=sorted(SIZES), default="7b",
                     help="layer sizes; 72b keeps one copy of the weights (long prompt portions unpack each matrix for the library)")
+    ap.add_argument("--dtype", choices=["bfloat16", "float16"], default="bfloat16",
+                    help="the 16-bit type of weights, activations and cache (the same kernels and rates either way)")
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the model has (named in config)")
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
@@ -86,7 +88,9 @@ def main() -> int:
         pool_tokens = int(sum(-(-(int(n) + args.mixed_decode + 16) // 16) * 16 for n in mixed_lens))
         max_batch, ctx_len = args.mixed, min(ctx_len, 8192)
     t0 = time.time()
-    eng = Engine(config=cfg, random_weights_seed=0, dtype="bfloat16", page_size=16, num_pages=pool_tokens // 16,
+    dtype_name = {"bfloat16": "bf16", "float16": "fp16"}[args.dtype]
+    lowp = getattr(torch, args.dtype)
+    eng = Engine(config=cfg, random_weights_seed=0, dtype=args.dtype, page_size=16, num_pages=pool_tokens // 16,
                  max_running_reqs=max(max_batch, 1), max_seq_len=ctx_len, max_extend_tokens=8192, chunk_size=2048,
                  decode_graphs=not args.no_graphs, single_weight_copy=single_copy)
     torch.cuda.synchronize()
@@ -158,13 +162,13 @@ def main() -> int:
 
     def measured_peaks():
         """What this machine delivers: GB/s of a kernel that only reads 2 GB (beyond the last-level cache), and
-        TFLOP/s of the GEMM library on an 8,192-cube in bfloat16."""
+        TFLOP/s of the GEMM library on an 8,192-cube in the run's 16-bit type."""
         from vt_transformer_amd.kernels import ops
         buf = torch.randint(0, 1 << 30, (1 << 29,), dtype=torch.int32, device="cuda")
         sums = torch.empty(256 * 16, dtype=torch.int32, device="cuda")
-        a = torch.randn(8192, 8192, device="cuda").to(torch.bfloat16)
-        b = torch.randn(8192, 8192, device="cuda").to(torch.bfloat16)
-        c = torch.empty(8192, 8192, dtype=torch.bfloat16, device="cuda")
+        a = torch.randn(8192, 8192, device="cuda").to(lowp)
+        b = torch.randn(8192, 8192, device="cuda").to(lowp)
+        c = torch.empty(8192, 8192, dtype=lowp, device="cuda")
 
         def best_ms(fn, reps=6):
             best = None
@@ -180,7 +184,7 @@ def main() -> int:
         read_ms = best_ms(lambda: ops.stream_read(buf, sums))
         mm_ms = best_ms(lambda: torch.mm(a, b.t(), out=c))
         out = {"hbm_read_GBps": round(buf.numel() * 4 / read_ms / 1e6, 1),
-               "gemm_bf16_TFLOPs": round(2 * 8192 ** 3 / mm_ms / 1e9, 1)}
+               "gemm_TFLOPs": round(2 * 8192 ** 3 / mm_ms / 1e9, 1)}
         print(f"[bench] measured peaks: {out}", file=sys.stderr, flush=True)
         return out
 
@@ -188,7 +192,7 @@ def main() -> int:
     H, I, V, L = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size, cfg.num_hidden_layers
     qkv = (cfg.num_attention_heads + 2 * cfg.num_key_value_heads) * cfg.head_dim
     layer_params = qkv * H + qkv + cfg.num_attention_heads * cfg.head_dim * H + 3 * I * H + 2 * H
-    weight_bytes = 2 * (L * layer_params + V * H + H)                  # every weight the step uses, once (bf16)
+    weight_bytes = 2 * (L * layer_params + V * H + H)                  # every weight the step uses, once (16 bits each)
     kv_bytes_per_token = 2 * 2 * L * cfg.num_key_value_heads * cfg.head_dim
 
     if args.mixed:
@@ -199,7 +203,7 @@ def main() -> int:
                       f"{args.mixed_decode} decoded tokens each, {model_name} layer sizes",
             "value": round(gen / dt, 1), "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": 0,
             "ms_per_step": round(dt / steps * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-            "dtype": "bf16", "data": "synthetic (random weights N(0,0.02), uniform random token ids)",
+            "dtype": dtype_name, "data": "synthetic (random weights N(0,0.02), uniform random token ids)",
             "config": {"model": f"{model_name} sizes", "layers": cfg.num_hidden_layers, "layers_full": FULL_LAYERS,
                        "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
                        "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
@@ -233,7 +237,7 @@ def main() -> int:
         "metric": f"decode tok/s at batch {args.batch}, {model_name} layer sizes, {args.prompt_len:,}-token prompts",
         "value": round(tps, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16", "data": "synthetic (random weights N(0,0.02), uniform random token ids)",
+        "dtype": dtype_name, "data": "synthetic (random weights N(0,0.02), uniform random token ids)",
         "config": {"model": f"{model_name} sizes", "layers": L, "layers_full": FULL_LAYERS, "hidden": H,
                    "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
                    "intermediate": I, "vocab": V, "global_batch": args.batch, "seq_len": args.prompt_len,
@@ -241,7 +245,7 @@ def main() -> int:
                    "parallelism": "1 GPU", "decode_graphs": not args.no_graphs, "gemm_tuning": not (args.no_tune or single_copy),
                    "weight_copies": 1 if single_copy else 2},
         "prefill": None if p_dt is None else {"value": round(T / p_dt, 1), "tokens": T, "ms": round(p_dt * 1e3, 3),
-                                              "frac": round(p_flops / p_dt / PEAK_FLOPS["bf16"], 4)},
+                                              "frac": round(p_flops / p_dt / PEAK_FLOPS[dtype_name], 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_GBPS, 4)},
         "points": points,
@@ -253,7 +257,7 @@ def main() -> int:
         # the same fractions against what this machine was measured to deliver
         vs = {"decode": round(achieved / peaks["hbm_read_GBps"], 4)}
         if p_dt is not None:
-            vs["prefill"] = round(p_flops / p_dt / (peaks["gemm_bf16_TFLOPs"] * 1e12), 4)
+            vs["prefill"] = round(p_flops / p_dt / (peaks["gemm_TFLOPs"] * 1e12), 4)
         for k_, f in points_frac.items():
             vs[k_] = round(f * HBM_GBPS / peaks["hbm_read_GBps"], 4)
         line["vs_measured_peaks"] = vs

@@ -16,8 +16,9 @@ import plain_model
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 # max |engine - plain| over a row of logits, relative to the row's largest |plain| logit
-# (bfloat16: about twice the worst error that any of the comparisons built on this has shown, 6.6e-3)
-TOL = {"float32": 2e-5, "bfloat16": 1.5e-2}
+# (bfloat16 and float16: about twice the worst error that any of the comparisons built on this has shown, 7.5e-3 and
+# 9.8e-4)
+TOL = {"float32": 2e-5, "bfloat16": 1.5e-2, "float16": 2e-3}
 
 
 def random_requests(vocab: int, lengths: Sequence[int], seed: int) -> Dict[str, List[int]]:

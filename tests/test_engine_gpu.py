@@ -15,7 +15,7 @@ from replay_helpers import (check_against_plain, cut, max_live_tokens, random_re
 
 pytestmark = pytest.mark.gpu
 
-DTYPES = ["float32", "bfloat16"]
+DTYPES = ["float32", "bfloat16", "float16"]
 CONFIGS = ["A", "B", "W"]
 _plain_cache = {}
 _models = {}

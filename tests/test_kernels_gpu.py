@@ -28,7 +28,7 @@ def bf16_round(x: torch.Tensor) -> torch.Tensor:
 
 
 # ---------------------------------------------------------------------------
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("vocab,hidden,n", [(203, 80, 7), (1000, 3584, 33)])
 def test_embed(dtype, vocab, hidden, n):
     g = torch.Generator().manual_seed(1)
@@ -40,13 +40,15 @@ def test_embed(dtype, vocab, hidden, n):
     assert torch.equal(out.cpu(), table.float()[ids.long()])
 
 
-@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("delta_dtype", [None, torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("delta_dtype", [None, torch.float32, "out"])
 @pytest.mark.parametrize("n,hidden,eps", [(5, 80, 1e-5), (3, 3584, 1e-6), (2, 1000, 1e-2)])
 def test_rmsnorm_with_residual(out_dtype, delta_dtype, n, hidden, eps):
     g = torch.Generator().manual_seed(2)
     h = torch.randn(n, hidden, generator=g) * 3
     gain = 1 + 0.1 * torch.randn(hidden, generator=g)
+    if delta_dtype == "out":        # a 16-bit delta is of the build's 16-bit type, like the output
+        delta_dtype = torch.bfloat16 if out_dtype == torch.float32 else out_dtype
     delta = None if delta_dtype is None else torch.randn(n, hidden, generator=g).to(delta_dtype)
     x = h.double() + (delta.double() if delta is not None else 0)
     ref = gain.double() * x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
@@ -60,7 +62,7 @@ def test_rmsnorm_with_residual(out_dtype, delta_dtype, n, hidden, eps):
     # eps sits inside the root: a large eps must show
     if eps == 1e-2:
         wrong = gain.double() * x / (torch.sqrt((x * x).mean(-1, keepdim=True)) + eps)
-        assert rel_err(out, wrong) > 10 * tol or out_dtype == torch.bfloat16
+        assert rel_err(out, wrong) > 10 * tol or out_dtype != torch.float32
 
 
 def test_rmsnorm_rows_gather():
@@ -78,7 +80,7 @@ def test_rmsnorm_rows_gather():
     assert torch.equal(hd.cpu(), h)  # a row list never writes the residual
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("n,inter", [(5, 200), (3, 204), (2, 203), (300, 1184)])   # widths in steps of 8, of 4, odd
 def test_silu_mul(dtype, n, inter):
     g = torch.Generator().manual_seed(4)
@@ -125,11 +127,13 @@ def test_linear_f32_is_true_fp32_and_batch_invariant():
 
 @pytest.mark.parametrize("n", [1, 3, 16, 17, 33, 64, 100, 300])
 @pytest.mark.parametrize("m,k", [(320, 96), (200, 200), (1030, 3584), (96, 18944 // 8)])
-@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
-def test_linear_bf16(n, m, k, out_dtype):
+@pytest.mark.parametrize("out_dtype", [torch.float32, "lowp"])
+@pytest.mark.parametrize("lp", [torch.bfloat16, torch.float16])
+def test_linear_bf16(n, m, k, out_dtype, lp):
     g = torch.Generator().manual_seed(7)
-    x = torch.randn(n, k, generator=g).to(torch.bfloat16)
-    w = (torch.randn(m, k, generator=g) * 0.05).to(torch.bfloat16)
+    out_dtype = lp if out_dtype == "lowp" else out_dtype
+    x = torch.randn(n, k, generator=g).to(lp)
+    w = (torch.randn(m, k, generator=g) * 0.05).to(lp)
     b = torch.randn(m, generator=g)
     ref = x.double() @ w.double().t() + b.double()
     out = torch.empty(n, m, dtype=out_dtype, device=DEV)
@@ -241,15 +245,16 @@ def test_linear_bf16_batch_invariant():
 
 @pytest.mark.parametrize("n", [1, 9, 40, 64, 100, 128, 300])
 @pytest.mark.parametrize("inter,k", [(200, 96), (128, 64), (1184, 3584), (18944, 40), (22016, 32), (29568, 24)])
-def test_gated_linear_bf16(n, inter, k):
+@pytest.mark.parametrize("lp", [torch.bfloat16, torch.float16])
+def test_gated_linear_bf16(n, inter, k, lp):
     # the three wide ones make the 64-token kernel take 5, 6 and 8 waves a block; from 65 rows on a block takes 128 tokens
     g = torch.Generator().manual_seed(10)
-    x = torch.randn(n, k, generator=g).to(torch.bfloat16)
-    w = (torch.randn(2 * inter, k, generator=g) * 0.05).to(torch.bfloat16)
+    x = torch.randn(n, k, generator=g).to(lp)
+    w = (torch.randn(2 * inter, k, generator=g) * 0.05).to(lp)
     gate = x.double() @ w[:inter].double().t()
     up = x.double() @ w[inter:].double().t()
     ref = gate / (1 + torch.exp(-gate)) * up
-    out = torch.empty(n, inter, dtype=torch.bfloat16, device=DEV)
+    out = torch.empty(n, inter, dtype=lp, device=DEV)
     ops().gated_linear_bf16(x.to(DEV), w.to(DEV), out)
     assert rel_err(out, ref) < 6e-3
     out32 = torch.empty(n, inter, dtype=torch.float32, device=DEV)
@@ -311,8 +316,8 @@ def attention_case(dtype, nh, kvh, d, page_size, window, entries, seed, spike=Fa
             qs[e][-1] *= 0
             qs[e][-1, :, 0] = 30.0 * math.sqrt(d) / 30.0 * 2.0
             vs[e][far] = 5.0
-    if dtype == torch.bfloat16:
-        ks, vs, qs = ([t.to(torch.bfloat16).float() for t in x] for x in (ks, vs, qs))
+    if dtype != torch.float32:
+        ks, vs, qs = ([t.to(dtype).float() for t in x] for x in (ks, vs, qs))
     kp, vp, bt = make_pages(ks, vs, lens, page_size, dtype, seed)
     n_tok = sum(n for _, n in entries)
     q = torch.cat(qs).reshape(n_tok, nh * d).to(dtype).to(DEV)
@@ -364,10 +369,10 @@ def attention_case(dtype, nh, kvh, d, page_size, window, entries, seed, spike=Fa
     return out, ref
 
 
-ATT_TOL = {torch.float32: 1e-5, torch.bfloat16: 1.5e-2}
+ATT_TOL = {torch.float32: 1e-5, torch.bfloat16: 1.5e-2, torch.float16: 2e-3}
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("nh,kvh,d", [(4, 2, 16), (3, 3, 32), (5, 1, 48), (14, 2, 64), (7, 7, 80), (28, 4, 128), (6, 2, 144),
                                       (2, 1, 256)])
 def test_attention_mixed_batch(dtype, nh, kvh, d):
@@ -377,7 +382,7 @@ def test_attention_mixed_batch(dtype, nh, kvh, d):
     assert rel_err(got, ref) < ATT_TOL[dtype]
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("page_size", [16, 32, 64])
 def test_attention_page_sizes_and_edges(dtype, page_size):
     # lengths that end exactly on, one before and one after a page's edge
@@ -386,7 +391,7 @@ def test_attention_page_sizes_and_edges(dtype, page_size):
     assert rel_err(got, ref) < ATT_TOL[dtype]
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("window", [1, 5, 16, 40])
 def test_attention_window_edge(dtype, window):
     entries = [(0, 70), (130, 1), (window, 1), (window - 1, 1) if window > 1 else (0, 1), (20, 30)]
@@ -403,7 +408,7 @@ def test_attention_long_portion_bf16():
     assert rel_err(got, ref) < ATT_TOL[torch.bfloat16]
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 def test_attention_far_key_among_hundreds(dtype):
     entries = [(700, 1), (0, 600), (513, 7)]
     got, ref = attention_case(dtype, 8, 2, 64, 16, 0, entries, seed=77, spike=True)
@@ -430,7 +435,7 @@ def test_attention_fp32_one_key_is_value_row_and_zero_query_is_mean():
 
 
 # ---------------------------------------------------------------------------
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("nh,kvh,d,page_size", [(4, 2, 16, 16), (5, 1, 48, 32), (28, 4, 128, 16), (64, 8, 128, 16)])
 def test_rope_store(dtype, nh, kvh, d, page_size):
     from vt_transformer_amd.parts.rotary import rotary_table
@@ -546,37 +551,39 @@ def test_sample_top_k_and_top_p():
 @pytest.mark.parametrize("nh,kvh,d", [(28, 4, 128), (4, 2, 16), (16, 1, 48), (6, 2, 144)])   # 144: nine tiles of 16 dims
 @pytest.mark.parametrize("window", [0, 37])
 @pytest.mark.parametrize("chunk", [64, 128, 1024])
-def test_attention_decode_kernel(nh, kvh, d, window, chunk):
+@pytest.mark.parametrize("lp", [torch.bfloat16, torch.float16])
+def test_attention_decode_kernel(nh, kvh, d, window, chunk, lp):
     """One token per entry, the keys cut into items on the device from the positions in memory."""
     o = ops()
     g = torch.Generator().manual_seed(nh + d + chunk)
     cached = [0, 15, 16, 17, 300, 63, 1000]
     lens = [c + 1 for c in cached]
-    ks = [torch.randn(t, kvh, d, generator=g).to(torch.bfloat16).float() for t in lens]
-    vs = [torch.randn(t, kvh, d, generator=g).to(torch.bfloat16).float() for t in lens]
-    qs = [torch.randn(1, nh, d, generator=g).to(torch.bfloat16).float() for _ in lens]
-    kp, vp, bt = make_pages(ks, vs, lens, 16, torch.bfloat16, 9)
+    ks = [torch.randn(t, kvh, d, generator=g).to(lp).float() for t in lens]
+    vs = [torch.randn(t, kvh, d, generator=g).to(lp).float() for t in lens]
+    qs = [torch.randn(1, nh, d, generator=g).to(lp).float() for _ in lens]
+    kp, vp, bt = make_pages(ks, vs, lens, 16, lp, 9)
     n = len(lens)
-    q = torch.cat(qs).reshape(n, nh * d).to(torch.bfloat16).to(DEV)
+    q = torch.cat(qs).reshape(n, nh * d).to(lp).to(DEV)
     p_max = 16
     if -(-max(lens) // chunk) > p_max:
         pytest.skip("the host never chooses a chunk that needs more items than p_max")
     part_o = torch.full((n * p_max * kvh * 16 * d,), float("nan"), device=DEV)
     part_ml = torch.full((n * p_max * kvh * 32,), float("nan"), device=DEV)
-    out = torch.full((n, nh * d), float("nan"), dtype=torch.bfloat16, device=DEV)
+    out = torch.full((n, nh * d), float("nan"), dtype=lp, device=DEV)
     scale = 1.0 / math.sqrt(d)
     o.attention_bf16_decode(q, kp.to(DEV), vp.to(DEV), bt.to(DEV), torch.tensor(cached, dtype=torch.int32, device=DEV),
                             torch.tensor([chunk, 0, 0, 0], dtype=torch.int32, device=DEV), p_max, out, part_o, part_ml,
                             nh, kvh, d, window, scale)
     ref = torch.cat([ref_attention(qs[e][0], ks[e], vs[e], cached[e], window, scale).reshape(1, -1) for e in range(n)])
-    assert rel_err(out, ref) < ATT_TOL[torch.bfloat16]
+    assert rel_err(out, ref) < ATT_TOL[lp]
 
 
 @pytest.mark.parametrize("nh,kvh,d,rot", [(28, 4, 128, 128), (4, 2, 64, 32), (6, 2, 80, 0), (16, 1, 256, 256), (3, 1, 48, 32),
                                           (6, 2, 256, 256), (6, 2, 144, 128)])
 @pytest.mark.parametrize("window", [0, 37])
 @pytest.mark.parametrize("chunk", [64, 1024])
-def test_attention_decode_fused_kernel(nh, kvh, d, rot, window, chunk):
+@pytest.mark.parametrize("lp", [torch.bfloat16, torch.float16])
+def test_attention_decode_fused_kernel(nh, kvh, d, rot, window, chunk, lp):
     """The decode attention that rotates and writes the pages itself against the separate rotation kernel followed
     by the plain decode attention, at two sets of positions."""
     o = ops()
@@ -592,25 +599,25 @@ def test_attention_decode_fused_kernel(nh, kvh, d, rot, window, chunk):
     for cached in ([0, 15, 16, 17, 300, 63, 1000], [31, 1, 999, 70, 119, 200]):
         n = len(cached)
         lens = [c + 1 for c in cached]
-        ks = [torch.randn(t, kvh, d, generator=g).to(torch.bfloat16).float() for t in lens]
-        vs = [torch.randn(t, kvh, d, generator=g).to(torch.bfloat16).float() for t in lens]
-        kp, vp, bt = make_pages(ks, vs, lens, ps, torch.bfloat16, 9)
+        ks = [torch.randn(t, kvh, d, generator=g).to(lp).float() for t in lens]
+        vs = [torch.randn(t, kvh, d, generator=g).to(lp).float() for t in lens]
+        kp, vp, bt = make_pages(ks, vs, lens, ps, lp, 9)
         kp, vp, bt = kp.to(DEV), vp.to(DEV), bt.to(DEV)
         # the last key and value of every entry come from the projection's row instead of the pages
         qkv = torch.randn(n, (nh + 2 * kvh) * d, generator=g).to(DEV)
         pos = torch.tensor(cached, dtype=torch.int32, device=DEV)
         tok_entry = torch.arange(n, dtype=torch.int32, device=DEV)
         kp_ref, vp_ref = kp.clone(), vp.clone()
-        q_ref = torch.empty(n, nh * d, dtype=torch.bfloat16, device=DEV)
+        q_ref = torch.empty(n, nh * d, dtype=lp, device=DEV)
         o.rope_store(qkv, cos, sin, pos, tok_entry, bt, q_ref, kp_ref, vp_ref, nh, kvh, d)
         part_o = torch.full((n * p_max * kvh * 16 * d,), float("nan"), device=DEV)
         part_ml = torch.full((n * p_max * kvh * 32,), float("nan"), device=DEV)
         dec = torch.tensor([chunk, 0, 0, 0], dtype=torch.int32, device=DEV)
         scale = 1.0 / math.sqrt(d)
-        out_ref = torch.full((n, nh * d), float("nan"), dtype=torch.bfloat16, device=DEV)
+        out_ref = torch.full((n, nh * d), float("nan"), dtype=lp, device=DEV)
         o.attention_bf16_decode(q_ref, kp_ref, vp_ref, bt, pos, dec, p_max, out_ref, part_o.clone(), part_ml.clone(), nh, kvh,
                                 d, window, scale)
-        out = torch.full((n, nh * d), float("nan"), dtype=torch.bfloat16, device=DEV)
+        out = torch.full((n, nh * d), float("nan"), dtype=lp, device=DEV)
         o.attention_bf16_decode_fused(qkv, cos, sin, kp, vp, bt, pos, dec, p_max, out, part_o, part_ml, nh, kvh, d, window,
                                       scale)
         torch.cuda.synchronize()
@@ -620,14 +627,15 @@ def test_attention_decode_fused_kernel(nh, kvh, d, rot, window, chunk):
 
 
 @pytest.mark.parametrize("d", list(range(16, 257, 16)))
-def test_attention_every_head_size(d):
-    """Every head size the kernels are compiled for, through every bfloat16 attention kernel: portions (per-wave and
+@pytest.mark.parametrize("lp", [torch.bfloat16, torch.float16])
+def test_attention_every_head_size(d, lp):
+    """Every head size the kernels are compiled for, through every 16-bit attention kernel: portions (per-wave and
     tiled, keys split and unsplit), decoding, and decoding that rotates and writes the pages itself."""
     entries = [(0, 37), (300, 1), (45, 19), (0, 1), (16, 2), (0, 150)]
-    got, ref = attention_case(torch.bfloat16, 6, 2, d, 16, 0, entries, seed=d)
-    assert rel_err(got, ref) < ATT_TOL[torch.bfloat16]
-    test_attention_decode_kernel(6, 2, d, 37, 128)
-    test_attention_decode_fused_kernel(6, 2, d, d if d % 32 == 0 else d - 16, 0, 64)
+    got, ref = attention_case(lp, 6, 2, d, 16, 0, entries, seed=d)
+    assert rel_err(got, ref) < ATT_TOL[lp]
+    test_attention_decode_kernel(6, 2, d, 37, 128, lp)
+    test_attention_decode_fused_kernel(6, 2, d, d if d % 32 == 0 else d - 16, 0, 64, lp)
 
 
 @pytest.mark.parametrize("n,m,k", [(1, 48, 64), (8, 3584, 3584), (16, 100, 200), (5, 4608, 1000), (3, 40, 24)])

@@ -27,7 +27,7 @@ LONG = dict(architectures=["Qwen2ForCausalLM"], model_type="qwen2", vocab_size=3
             hidden_act="silu", use_sliding_window=False, torch_dtype="bfloat16")
 QK_SCALE = 6.0
 # about twice the worst error seen (relative to a row's largest logit): 1.1e-6 in float32, 7.3e-3 in bfloat16
-TOL = {"float32": 3e-6, "bfloat16": 1.5e-2}
+TOL = {"float32": 3e-6, "bfloat16": 1.5e-2, "float16": 2e-3}
 
 
 @pytest.fixture(scope="module")
@@ -78,7 +78,7 @@ def test_the_long_model_spreads_its_weight_over_far_keys(long_folder):
     assert effect > 2.5 * TOL["bfloat16"], effect
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16", "float16"])
 @pytest.mark.parametrize("n_long", [8192, 20480])
 def test_long_context_in_portions_then_token_by_token_beside_another_prompt(long_folder, dtype, n_long):
     from vt_transformer_amd.engine import StepEntry, load_model, make_runner
@@ -115,7 +115,7 @@ def test_long_context_in_portions_then_token_by_token_beside_another_prompt(long
             rows.insert(0, ("b", ref_b, 2047 + j))
         check(runner.step(entries), rows)
     assert len(runner.cache.get("a").tables[0]) == (n_long + 32 + 15) // 16
-    if dtype == "bfloat16":
+    if dtype != "float32":
         assert runner._graphs, "decoding did not go through captured steps"
     runner.release("a"); runner.release("b")
     assert sum(runner.cache.held_pages()) == 0

@@ -53,7 +53,7 @@ def check_configuration(cfg, seed, tmp_path):
     toks = rs.randint(0, cfg["vocab_size"], size=n).tolist()
     ref = plain_model.forward(pcfg, w, toks)
     worst = {}
-    for dtype, tol in (("float32", 3e-5), ("bfloat16", 1.5e-2)):
+    for dtype, tol in (("float32", 3e-5), ("bfloat16", 1.5e-2), ("float16", 2e-3)):
         model = load_model(folder, dtype)
         for mode in ("whole", "cut", "decode", "graph"):
             runner = make_runner(model, pool_tokens=-(-n // 16) * 16 + 32, page_size=16, max_requests=2, max_seq_len=512)
@@ -109,7 +109,7 @@ def test_real_layer_sizes(name, hidden, heads, kv, inter, tmp_path):
     toks = np.random.RandomState(0).randint(0, 4099, size=n).tolist()
     ref = plain_model.forward(pcfg, w, toks)
     scale = ref.abs().max()
-    for dtype, tol in (("bfloat16", 2e-2), ("float32", 3e-5)):
+    for dtype, tol in (("bfloat16", 2e-2), ("float16", 3e-3), ("float32", 3e-5)):
         model = load_model(folder, dtype)
         for mode in ("whole", "cut", "decode", "graph", "batch"):
             runner = make_runner(model, pool_tokens=10240, page_size=16, max_requests=48, max_seq_len=512)

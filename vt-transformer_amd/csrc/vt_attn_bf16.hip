@@ -37,8 +37,8 @@ static_assert(VT_HEAD_DIM % 16 == 0 && VT_HEAD_DIM >= 16 && VT_HEAD_DIM <= 256, 
 #define D VT_HEAD_DIM
 #define ITEM_INTS 8  // entry, q_tok0, q_len, pos0, q_row0, key_lo, key_hi, part (-1: final)
 
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
-typedef __attribute__((ext_vector_type(4))) short bf16x4_t;
+typedef vt_lowp8_t bf16x8_t;
+typedef vt_lowp4_t bf16x4_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
 struct AttnArgs {
@@ -74,14 +74,8 @@ __device__ __forceinline__ int page_index(const AttnArgs& a, int j) {
 union U8 { uint2 u; bf16x4_t v; };
 union U16 { uint4 u; bf16x8_t v; };
 
-typedef __attribute__((ext_vector_type(2))) float f32x2_t;
-typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
-
-// two floats to two bf16 (round to nearest even) in one instruction
-__device__ __forceinline__ unsigned pack2(float a, float b) {
-    f32x2_t v = {a, b};
-    return __builtin_bit_cast(unsigned, __builtin_convertvector(v, bf16x2_t));
-}
+// two floats to two 16-bit values (round to nearest even) in one instruction
+__device__ __forceinline__ unsigned pack2(float a, float b) { return vt_pack2(a, b); }
 
 // Maximum over the four lanes that share a row (lane % 16): two register swaps between rows of 16 and halves of 32
 // lanes, which stay in the vector unit (a shuffle would go through the LDS crossbar).
@@ -531,13 +525,13 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : (DECODE && !DIRECT ? 3 : 2)) voi
                     U16 t;
                     if constexpr (DIRECT) t.u = *(const uint4*)(kl + r * D + (((4 * st + g) ^ r) << 3));
                     else t.u = *(const uint4*)(kl + r * KL_ROW + st * 32 + g * 8);
-                    s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(t.v, q8[rt][st], s, 0, 0, 0);
+                    s = VT_MFMA_16X16X32(t.v, q8[rt][st], s);
                 }
             } else {
 #pragma unroll
                 for (int st = 0; st < QSTEPS; ++st) {
                     U8 t; t.u = *(const uint2*)(kl + r * KL_ROW + st * 16 + g * 4);
-                    s = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(t.v, q4[rt][st], s, 0, 0, 0);
+                    s = VT_MFMA_16X16X16(t.v, q4[rt][st], s);
                 }
             }
             // s[i] is key j0 + 4 g + i against row r of the tile
@@ -556,7 +550,7 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : (DECODE && !DIRECT ? 3 : 2)) voi
                 if constexpr (DIRECT) vf.u = *(const uint2*)(vl + ((2 * t + (g >> 1)) * 16 + r) * 8 + (g & 1) * 4);
                 else vf.u = *(const uint2*)(vl + (t * 16 + r) * VL_ROW + 4 * g);
                 if (rescale) o[rt][t] *= alpha;
-                o[rt][t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf.v, pf.v, o[rt][t], 0, 0, 0);
+                o[rt][t] = VT_MFMA_16X16X16(vf.v, pf.v, o[rt][t]);
             }
         }
         wave_lds_order();       // the next block is parked after these reads
@@ -961,7 +955,7 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_tile_kernel(At
     };
 
     bf16x8_t ones8;
-    { U16 t; t.u = make_uint4(0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u); ones8 = t.v; }
+    { U16 t; t.u = make_uint4(VT_LOWP_ONE_PAIR, VT_LOWP_ONE_PAIR, VT_LOWP_ONE_PAIR, VT_LOWP_ONE_PAIR); ones8 = t.v; }
     // one key block (in LDS buffer `buf`, keys from j0) against the RT row tiles of this wave
     auto multiply = [&](int buf, int j0) __attribute__((always_inline)) {
         if (j0 > wave_hi || j0 + KB - 1 < wave_lo) return;   // every key masked for every row of the wave
@@ -981,7 +975,7 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_tile_kernel(At
                     else t.u = *(const uint4*)(kr + st * 32 + g * 8);
 #pragma unroll
                     for (int rt = 0; rt < RT; ++rt)
-                        s[rt][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(t.v, q8[rt][st], s[rt][kt], 0, 0, 0);
+                        s[rt][kt] = VT_MFMA_16X16X32(t.v, q8[rt][st], s[rt][kt]);
                 }
             } else {
 #pragma unroll
@@ -989,7 +983,7 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_tile_kernel(At
                     U8 t; t.u = *(const uint2*)(kr + st * 16 + g * 4);
 #pragma unroll
                     for (int rt = 0; rt < RT; ++rt)
-                        s[rt][kt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(t.v, q4[rt][st], s[rt][kt], 0, 0, 0);
+                        s[rt][kt] = VT_MFMA_16X16X16(t.v, q4[rt][st], s[rt][kt]);
                 }
             }
         }
@@ -1014,7 +1008,7 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_tile_kernel(At
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
                 pf[rt].u = make_uint4(pk[rt][4 * h], pk[rt][4 * h + 1], pk[rt][4 * h + 2], pk[rt][4 * h + 3]);
-                ol[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones8, pf[rt].v, ol[rt], 0, 0, 0);
+                ol[rt] = VT_MFMA_16X16X32(ones8, pf[rt].v, ol[rt]);
             }
 #pragma unroll
             for (int t = 0; t < DT; ++t) {
@@ -1023,7 +1017,7 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_tile_kernel(At
                 else vf.u = *(const uint4*)(vd + (t * 16 + r) * VROW + 32 * h + 8 * g);
 #pragma unroll
                 for (int rt = 0; rt < RT; ++rt)
-                    o[rt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[rt].v, o[rt][t], 0, 0, 0);
+                    o[rt][t] = VT_MFMA_16X16X32(vf.v, pf[rt].v, o[rt][t]);
             }
         }
     };

@@ -1,4 +1,4 @@
-// Shared helpers of the gfx950 kernels: bf16 conversion, wave and block
+// Shared helpers of the gfx950 kernels: conversion of the 16-bit type, wave and block
 // reductions for 64-wide wavefronts, launch checking.
 //
 // Every entry point is extern "C", takes raw device pointers and a stream,
@@ -43,6 +43,29 @@ static int vt_fail(const char* fmt, ...) {
         if (!(cond)) return vt_fail(__VA_ARGS__); \
     } while (0)
 
+// The 16-bit type of a build is bfloat16, or IEEE half when the source is compiled with -DVT_LOWP_F16: the same
+// kernels, another conversion and another matrix instruction of the same shape and rate.  A library is built once
+// per 16-bit type and its file name says which; `bf16_t` is the raw 16 bits either way, and VT_BF16 the code of "the
+// build's 16-bit type" in the entry points' dtype arguments.
+typedef __attribute__((ext_vector_type(2))) float vt_f32x2_t;
+#ifdef VT_LOWP_F16
+typedef _Float16 vt_lowp_t;
+typedef __attribute__((ext_vector_type(4))) _Float16 vt_lowp4_t;
+#define VT_MFMA_16X16X32(a, b, c) __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0)
+#define VT_MFMA_16X16X16(a, b, c) __builtin_amdgcn_mfma_f32_16x16x16f16(a, b, c, 0, 0, 0)
+#define VT_LOWP_ONE_PAIR 0x3c003c00u       // two ones
+__device__ __forceinline__ float bf16_to_f32(bf16_t v) { return (float)__builtin_bit_cast(_Float16, v); }
+// round to nearest even; NaN stays NaN, what is too large becomes infinity
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) { return __builtin_bit_cast(bf16_t, (_Float16)f); }
+// the two values of a 32-bit word
+__device__ __forceinline__ float lowp_lo(unsigned u) { return bf16_to_f32((bf16_t)(u & 0xffffu)); }
+__device__ __forceinline__ float lowp_hi(unsigned u) { return bf16_to_f32((bf16_t)(u >> 16)); }
+#else
+typedef __bf16 vt_lowp_t;
+typedef __attribute__((ext_vector_type(4))) short vt_lowp4_t;
+#define VT_MFMA_16X16X32(a, b, c) __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0)
+#define VT_MFMA_16X16X16(a, b, c) __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, b, c, 0, 0, 0)
+#define VT_LOWP_ONE_PAIR 0x3f803f80u
 __device__ __forceinline__ float bf16_to_f32(bf16_t v) {
     return __uint_as_float(((uint32_t)v) << 16);
 }
@@ -53,6 +76,16 @@ __device__ __forceinline__ bf16_t f32_to_bf16(float f) {
     if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40u);
     u += 0x7fffu + ((u >> 16) & 1u);
     return (bf16_t)(u >> 16);
+}
+__device__ __forceinline__ float lowp_lo(unsigned u) { return __uint_as_float(u << 16); }
+__device__ __forceinline__ float lowp_hi(unsigned u) { return __uint_as_float(u & 0xffff0000u); }
+#endif
+typedef __attribute__((ext_vector_type(8))) vt_lowp_t vt_lowp8_t;
+typedef __attribute__((ext_vector_type(2))) vt_lowp_t vt_lowp2_t;
+// two floats to two 16-bit values (round to nearest even) in one instruction
+__device__ __forceinline__ unsigned vt_pack2(float a, float b) {
+    vt_f32x2_t v = {a, b};
+    return __builtin_bit_cast(unsigned, __builtin_convertvector(v, vt_lowp2_t));
 }
 
 template <typename T> __device__ __forceinline__ float load_f32(const T* p, size_t i);

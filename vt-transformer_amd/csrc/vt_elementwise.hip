@@ -79,8 +79,7 @@ __global__ void rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__ del
 __device__ __forceinline__ float4 load4(const float* p) { return *(const float4*)p; }
 __device__ __forceinline__ float4 load4(const bf16_t* p) {
     uint2 u = *(const uint2*)p;
-    return make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u), __uint_as_float(u.y << 16),
-                       __uint_as_float(u.y & 0xffff0000u));
+    return make_float4(lowp_lo(u.x), lowp_hi(u.x), lowp_lo(u.y), lowp_hi(u.y));
 }
 __device__ __forceinline__ void store4(float* p, float4 v) { *(float4*)p = v; }
 __device__ __forceinline__ void store4(bf16_t* p, float4 v) {
@@ -253,8 +252,8 @@ __global__ __launch_bounds__(256) void silu_mul_vec_kernel(const TI* __restrict_
 // bfloat16 in and out, widths that are a multiple of 8: 16 bytes per access, two accesses of gate and of up in
 // flight per thread.
 __device__ __forceinline__ unsigned silu_mul_pair(unsigned g, unsigned u) {
-    const float g0 = __uint_as_float(g << 16), g1 = __uint_as_float(g & 0xffff0000u);
-    const float u0 = __uint_as_float(u << 16), u1 = __uint_as_float(u & 0xffff0000u);
+    const float g0 = lowp_lo(g), g1 = lowp_hi(g);
+    const float u0 = lowp_lo(u), u1 = lowp_hi(u);
     return (unsigned)f32_to_bf16(g0 / (1.f + __expf(-g0)) * u0) | ((unsigned)f32_to_bf16(g1 / (1.f + __expf(-g1)) * u1) << 16);
 }
 __global__ __launch_bounds__(256) void silu_mul_bf16x8_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ out,

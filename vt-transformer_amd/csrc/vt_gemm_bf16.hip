@@ -32,7 +32,7 @@
 
 VT_DEFINE_LAST_ERROR()
 
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef vt_lowp8_t bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
 union Frag {
@@ -119,13 +119,7 @@ extern "C" int vt_unpack_matrix_bf16(const void* wp, void* w, int M, int K, hipS
     return 0;
 }
 
-typedef __attribute__((ext_vector_type(2))) float f32x2_t;
-typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
-// two floats to two bf16 (round to nearest even) in one instruction
-__device__ __forceinline__ unsigned pack_bf16x2(float a, float b) {
-    f32x2_t v = {a, b};
-    return __builtin_bit_cast(unsigned, __builtin_convertvector(v, bf16x2_t));
-}
+__device__ __forceinline__ unsigned pack_bf16x2(float a, float b) { return vt_pack2(a, b); }
 
 // x[row][k .. k + 8); beyond the end of the row its last eight values are read instead (W is zero there)
 __device__ __forceinline__ bf16x8_t load_x(const bf16_t* row, int k, int K) {
@@ -333,7 +327,7 @@ __global__ __launch_bounds__(WPB * 64) void gemm_skinny_kernel(const void* __res
             for (int u = 0; u < 2 * UP; ++u)
 #pragma unroll
                 for (int a = 0; a < NW; ++a)
-                    acc[a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[a][u].v, xf[u].v, acc[a], 0, 0, 0);
+                    acc[a] = VT_MFMA_16X16X32(wa[a][u].v, xf[u].v, acc[a]);
         }
         for (; p < p_end; ++p) {
             Frag wa[NW][2], xa, xb, xf[2];
@@ -348,7 +342,7 @@ __global__ __launch_bounds__(WPB * 64) void gemm_skinny_kernel(const void* __res
             for (int u = 0; u < 2; ++u)
 #pragma unroll
                 for (int a = 0; a < NW; ++a)
-                    acc[a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[a][u].v, xf[u].v, acc[a], 0, 0, 0);
+                    acc[a] = VT_MFMA_16X16X32(wa[a][u].v, xf[u].v, acc[a]);
         }
         t = t_end;      // (nothing left for the loops below)
     }
@@ -371,7 +365,7 @@ __global__ __launch_bounds__(WPB * 64) void gemm_skinny_kernel(const void* __res
         for (int u = 0; u < U; ++u)
 #pragma unroll
             for (int a = 0; a < NW; ++a)
-                acc[a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[a][u].v, xa[u].f.v, acc[a], 0, 0, 0);
+                acc[a] = VT_MFMA_16X16X32(wa[a][u].v, xa[u].f.v, acc[a]);
     }
     for (; t < t_end; ++t) {
         Piece xa = load_piece(t);
@@ -381,7 +375,7 @@ __global__ __launch_bounds__(WPB * 64) void gemm_skinny_kernel(const void* __res
         for (int a = 0; a < NW; ++a) {
             Frag wa;
             wa.u = load_w_once(wbase[a] + (size_t)t * PK_TILE);
-            acc[a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa.v, xa.f.v, acc[a], 0, 0, 0);
+            acc[a] = VT_MFMA_16X16X32(wa.v, xa.f.v, acc[a]);
         }
     }
     if constexpr (NORM) {
@@ -598,7 +592,7 @@ __global__ __launch_bounds__((WM + 1) * 64) void gemm_mid_kernel(const bf16_t* _
                 for (int i = 0; i < NTT; ++i)
 #pragma unroll
                     for (int a = 0; a < RW; ++a)
-                        acc[a][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[a][u0 + u].v, xf[u][i].v, acc[a][i], 0, 0, 0);
+                        acc[a][i] = VT_MFMA_16X16X32(wf[a][u0 + u].v, xf[u][i].v, acc[a][i]);
         }
     };
 #pragma unroll
@@ -733,7 +727,7 @@ __global__ __launch_bounds__(WPB * 64) __attribute__((amdgpu_waves_per_eu(2, 4))
                 xf.u = xt[u * TS + i * 4 * 17 + rslot];
 #pragma unroll
                 for (int j = 0; j < R; ++j)
-                    acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[u][j].v, xf.v, acc[j][i], 0, 0, 0);
+                    acc[j][i] = VT_MFMA_16X16X32(wa[u][j].v, xf.v, acc[j][i]);
             }
         wave_lds_order();       // the next pair is written after these reads
     }

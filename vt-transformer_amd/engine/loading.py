@@ -13,19 +13,20 @@ from ..weights.loader import check_tensors, load_model_weights
 from ..weights.random_init import random_tensor
 from .step import ModelRunner
 
-_DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32,
+_DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float16": torch.float16, "fp16": torch.float16,
+           "f16": torch.float16, "half": torch.float16, "float32": torch.float32, "fp32": torch.float32,
            "f32": torch.float32}
 
 
 def parse_dtype(name) -> torch.dtype:
     if isinstance(name, torch.dtype):
-        if name in (torch.bfloat16, torch.float32):
+        if name in (torch.bfloat16, torch.float16, torch.float32):
             return name
-        raise ValueError(f"dtype {name} is not supported (bfloat16 and float32 are)")
+        raise ValueError(f"dtype {name} is not supported (bfloat16, float16 and float32 are)")
     try:
         return _DTYPES[str(name).lower()]
     except KeyError:
-        raise ValueError(f"dtype '{name}' is not supported (bfloat16 and float32 are)") from None
+        raise ValueError(f"dtype '{name}' is not supported (bfloat16, float16 and float32 are)") from None
 
 
 def build_model(config: ModelConfig, dtype, device: Optional[torch.device] = None,

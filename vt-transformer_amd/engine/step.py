@@ -110,7 +110,7 @@ class ModelRunner:
         self.steps = 0
         self.tokens = 0
         self._staging = HostStaging(torch.int32)
-        # Decoding steps of a bfloat16 model are captured once per batch size and replayed, unless a mixer keeps
+        # Decoding steps of a 16-bit model are captured once per batch size and replayed, unless a mixer keeps
         # state of its own between steps (the warm-up run before a capture would advance it twice) or a part does
         # not declare that its step can be replayed.
         self.decode_graphs = False
@@ -239,7 +239,7 @@ class ModelRunner:
 
     def replays(self, n_entries: int) -> bool:
         """Whether a decoding step of this many entries goes through a captured graph."""
-        return (self.decode_graphs and self._replayable and self.rt.dtype == torch.bfloat16
+        return (self.decode_graphs and self._replayable and self.rt.lowp
                 and 0 < n_entries <= GRAPH_BATCHES[-1])
 
     def step(self, entries: Sequence[StepEntry], ids_dev: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:

@@ -29,9 +29,12 @@ ARCH = "gfx950"
 FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC", "-shared",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
-# libraries that every model needs; attention for bf16 is built per head size
+# libraries that every model needs; attention for the 16-bit types is built per head size
 BASE_LIBS = ["vt_elementwise", "vt_gemm_f32", "vt_gemm_bf16", "vt_attn_f32", "vt_sampling"]
 DEFAULT_HEAD_DIMS = list(range(16, 257, 16))
+# The libraries that handle 16-bit values are built once for bfloat16 and once for float16 (-DVT_LOWP_F16: the same
+# sources with the other conversion and the other matrix instruction); the float16 build's name ends in _f16.
+HALF_LIBS = ("vt_elementwise", "vt_gemm_bf16", "vt_attn_bf16")
 
 
 class KernelBuildError(RuntimeError):
@@ -78,23 +81,29 @@ def _source_hash(src: str, defines: Dict[str, str]) -> str:
     return h.hexdigest()[:16]
 
 
-def lib_spec(name: str, head_dim: Optional[int] = None) -> Tuple[str, str, Dict[str, str]]:
-    """(library name, source path, defines)"""
+def lib_spec(name: str, head_dim: Optional[int] = None, half: bool = False) -> Tuple[str, str, Dict[str, str]]:
+    """(library name, source path, defines).  half: the build whose 16-bit type is float16 (for the libraries that
+    have one; the others are the same either way)."""
+    half = half and name in HALF_LIBS
+    defines: Dict[str, str] = {"VT_LOWP_F16": "1"} if half else {}
+    suffix = "_f16" if half else ""
     if name == "vt_attn_bf16":
         if head_dim is None:
             raise ValueError("vt_attn_bf16 is built per head size")
-        return f"vt_attn_bf16_d{head_dim}", os.path.join(CSRC, "vt_attn_bf16.hip"), {"VT_HEAD_DIM": str(head_dim)}
-    return name, os.path.join(CSRC, name + ".hip"), {}
+        defines["VT_HEAD_DIM"] = str(head_dim)
+        return f"vt_attn_bf16_d{head_dim}{suffix}", os.path.join(CSRC, "vt_attn_bf16.hip"), defines
+    return name + suffix, os.path.join(CSRC, name + ".hip"), defines
 
 
-def lib_path(name: str, head_dim: Optional[int] = None) -> str:
-    lname, src, defines = lib_spec(name, head_dim)
+def lib_path(name: str, head_dim: Optional[int] = None, half: bool = False) -> str:
+    lname, src, defines = lib_spec(name, head_dim, half)
     return os.path.join(_build_dir(), f"lib{lname}-{_source_hash(src, defines)}.so")
 
 
-def compile_lib(name: str, head_dim: Optional[int] = None, force: bool = False, verbose: bool = True) -> str:
-    lname, src, defines = lib_spec(name, head_dim)
-    out = lib_path(name, head_dim)
+def compile_lib(name: str, head_dim: Optional[int] = None, force: bool = False, verbose: bool = True,
+                half: bool = False) -> str:
+    lname, src, defines = lib_spec(name, head_dim, half)
+    out = lib_path(name, head_dim, half)
     if os.path.isfile(out) and not force:
         return out
     if not os.path.isfile(src):
@@ -145,22 +154,24 @@ def compile_lib(name: str, head_dim: Optional[int] = None, force: bool = False, 
 
 def build_all(head_dims: Iterable[int] = DEFAULT_HEAD_DIMS, force: bool = True, jobs: int = 8, verbose: bool = True) -> List[str]:
     """Compile every library (used by the build check); returns their paths."""
-    tasks = [(n, None) for n in BASE_LIBS] + [("vt_attn_bf16", d) for d in head_dims]
+    head_dims = list(head_dims)
+    tasks = [(n, None, False) for n in BASE_LIBS] + [("vt_attn_bf16", d, False) for d in head_dims]
+    tasks += [(n, None, True) for n in BASE_LIBS if n in HALF_LIBS] + [("vt_attn_bf16", d, True) for d in head_dims]
     with ThreadPoolExecutor(max_workers=max(1, min(jobs, 16))) as ex:
-        return list(ex.map(lambda t: compile_lib(t[0], t[1], force=force, verbose=verbose), tasks))
+        return list(ex.map(lambda t: compile_lib(t[0], t[1], force=force, verbose=verbose, half=t[2]), tasks))
 
 
 _loaded: Dict[str, ctypes.CDLL] = {}
 _lock = threading.Lock()
 
 
-def load_lib(name: str, head_dim: Optional[int] = None) -> ctypes.CDLL:
-    """Load a library, compiling it first if no build of the current source exists."""
-    key = name if head_dim is None else f"{name}_d{head_dim}"
+def load_lib(name: str, head_dim: Optional[int] = None, half: bool = False) -> ctypes.CDLL:
+    """Load a library, compiling it first if no build of the current source exists.  half: its float16 build."""
+    key = lib_spec(name, head_dim, half)[0]
     with _lock:
         if key in _loaded:
             return _loaded[key]
-        path = compile_lib(name, head_dim)
+        path = compile_lib(name, head_dim, half=half)
         try:
             lib = ctypes.CDLL(path)
         except OSError as e:

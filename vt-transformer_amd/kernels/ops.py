@@ -13,10 +13,14 @@ from typing import Optional
 
 import torch
 
+from . import build as _build
 from .build import KernelBuildError, load_lib
 
 F32, BF16 = 0, 1
-_CODES = {torch.float32: F32, torch.bfloat16: BF16}
+# The 16-bit types.  A library that handles 16-bit values exists once for each (kernels.build.HALF_LIBS); BF16 is the
+# code of "the library's 16-bit type" in the entry points' dtype arguments, whichever build is called.
+LOWP = (torch.bfloat16, torch.float16)
+_CODES = {torch.float32: F32, torch.bfloat16: BF16, torch.float16: BF16}
 
 
 class KernelError(RuntimeError):
@@ -27,7 +31,33 @@ def _code(t: torch.Tensor) -> int:
     try:
         return _CODES[t.dtype]
     except KeyError:
-        raise KernelError(f"dtype {t.dtype} is not handled by the kernels (float32 and bfloat16 are)") from None
+        raise KernelError(f"dtype {t.dtype} is not handled by the kernels (float32, bfloat16 and float16 are)") from None
+
+
+def _half(*ts) -> bool:
+    """Which build of a library a call needs: True if the 16-bit tensors among `ts` are float16.  The two 16-bit
+    types do not meet in one call."""
+    kinds = {t.dtype for t in ts if t is not None and t.dtype in LOWP}
+    if len(kinds) > 1:
+        raise KernelError("bfloat16 and float16 tensors in one call")
+    return torch.float16 in kinds
+
+
+def _any_build(name: str, head_dim: Optional[int] = None):
+    """A library for a question whose answer is the same in both of its builds (launch shapes, sizes of scratch
+    memory): the build that is loaded already, so that a float16 model does not compile the bfloat16 one for it."""
+    for half in (False, True):
+        lib = _build._loaded.get(_build.lib_spec(name, head_dim, half)[0])
+        if lib is not None:
+            return lib
+    return load_lib(name, head_dim)
+
+
+def _lowp(t: torch.Tensor, name: str) -> torch.dtype:
+    """The 16-bit type of a call's leading tensor."""
+    if t.dtype not in LOWP:
+        raise KernelError(f"{name}: dtype {t.dtype}, expected bfloat16 or float16")
+    return t.dtype
 
 
 def _chk(t: torch.Tensor, name: str, dtype=None, shape=None) -> None:
@@ -70,7 +100,7 @@ def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> torch.Te
     _chk(table, "embed.table")
     _chk(ids, "embed.ids", torch.int32)
     _chk(out, "embed.out", torch.float32, (n, hidden))
-    _run(load_lib("vt_elementwise"), "vt_embed", _ptr(table), _i(_code(table)), _ptr(ids), _ptr(out), _i(n), _i(hidden),
+    _run(load_lib("vt_elementwise", half=_half(table)), "vt_embed", _ptr(table), _i(_code(table)), _ptr(ids), _ptr(out), _i(n), _i(hidden),
          _i(vocab), _stream())
     return out
 
@@ -90,7 +120,7 @@ def rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], gain: torch.Tensor, 
     else:
         n_out = h.shape[0]
     _chk(out, "rmsnorm.out", None, (n_out, hidden))
-    _run(load_lib("vt_elementwise"), "vt_rmsnorm", _ptr(h), _ptr(delta), _i(_code(delta) if delta is not None else -1),
+    _run(load_lib("vt_elementwise", half=_half(delta, out)), "vt_rmsnorm", _ptr(h), _ptr(delta), _i(_code(delta) if delta is not None else -1),
          _ptr(gain), _ptr(out), _i(_code(out)), _ptr(rows), _i(n_out), _i(hidden), _f(eps),
          _i(1 if (update_h and delta is not None) else 0), _stream())
     return out
@@ -99,7 +129,7 @@ def rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], gain: torch.Tensor, 
 def residual_add(h: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
     _chk(h, "residual_add.h", torch.float32)
     _chk(delta, "residual_add.delta", None, h.shape)
-    _run(load_lib("vt_elementwise"), "vt_residual_add", _ptr(h), _ptr(delta), _i(_code(delta)),
+    _run(load_lib("vt_elementwise", half=_half(delta)), "vt_residual_add", _ptr(h), _ptr(delta), _i(_code(delta)),
          ctypes.c_longlong(h.numel()), _stream())
     return h
 
@@ -110,7 +140,7 @@ def silu_mul(gu: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     _chk(out, "silu_mul.out", None, (n, two_i // 2))
     if two_i % 2:
         raise KernelError(f"silu_mul: input width {two_i} is odd")
-    _run(load_lib("vt_elementwise"), "vt_silu_mul", _ptr(gu), _i(_code(gu)), _ptr(out), _i(_code(out)), _i(n),
+    _run(load_lib("vt_elementwise", half=_half(gu, out)), "vt_silu_mul", _ptr(gu), _i(_code(gu)), _ptr(out), _i(_code(out)), _i(n),
          _i(two_i // 2), _stream())
     return out
 
@@ -121,7 +151,7 @@ def gather_rows(x: torch.Tensor, rows: Optional[torch.Tensor], out: torch.Tensor
     if rows is not None:
         _chk(rows, "gather_rows.rows", torch.int32)
     _chk(out, "gather_rows.out", None, (n, x.shape[1]))
-    _run(load_lib("vt_elementwise"), "vt_gather_rows", _ptr(x), _i(_code(x)), _ptr(rows), _ptr(out), _i(_code(out)),
+    _run(load_lib("vt_elementwise", half=_half(x, out)), "vt_gather_rows", _ptr(x), _i(_code(x)), _ptr(rows), _ptr(out), _i(_code(out)),
          _i(n), _i(x.shape[1]), _stream())
     return out
 
@@ -142,7 +172,7 @@ def random_normal(out: torch.Tensor, key: int, scale: float, mean: float, first:
     """out.flat[i] = mean + scale * (twelve 16-bit integers of element first + i, summed and centred): close to
     N(mean, (65536 scale)^2), and the same bits as weights.random_init.counter_normal makes on the host."""
     _chk(out, "random_normal.out")
-    _run(load_lib("vt_elementwise"), "vt_random_normal", _ptr(out), _i(_code(out)), ctypes.c_longlong(out.numel()),
+    _run(load_lib("vt_elementwise", half=_half(out)), "vt_random_normal", _ptr(out), _i(_code(out)), ctypes.c_longlong(out.numel()),
          ctypes.c_longlong(int(first)), ctypes.c_ulonglong(int(key) & 0xFFFFFFFFFFFFFFFF), _f(scale), _f(mean), _stream())
     return out
 
@@ -177,7 +207,7 @@ def rope_store(qkv: torch.Tensor, cos: Optional[torch.Tensor], sin: Optional[tor
         _chk(v_pages, "rope_store.v_pages", q_out.dtype, (num_pages, n_kv, head_dim, page_size))
         _chk(block_table, "rope_store.block_table", torch.int32)
         max_blocks = block_table.shape[1]
-    _run(load_lib("vt_elementwise"), "vt_rope_store", _ptr(qkv), _i(_code(qkv)), ctypes.c_longlong(qkv.stride(0)),
+    _run(load_lib("vt_elementwise", half=_half(qkv, q_out, k_pages)), "vt_rope_store", _ptr(qkv), _i(_code(qkv)), ctypes.c_longlong(qkv.stride(0)),
          _ptr(cos), _ptr(sin), _i(rot), _i(max_pos), _ptr(positions), _ptr(tok_entry), _ptr(block_table),
          _i(max_blocks), _ptr(q_out), _ptr(k_pages), _ptr(v_pages), _i(_code(q_out)), _i(page_size), _i(num_pages),
          _i(n), _i(n_heads), _i(n_kv), _i(head_dim), _i(1 if write_kv else 0), _stream())
@@ -217,14 +247,15 @@ class PackedMatrix:
 def pack_matrix_bf16(w: torch.Tensor, halves: int = 1) -> PackedMatrix:
     """Pack W [rows, cols] (halves = 2: [2 * rows, cols], the two matrices stacked) for linear_bf16 /
     gated_linear_bf16."""
-    _chk(w, "pack_matrix_bf16.w", torch.bfloat16)
+    lp = _lowp(w, "pack_matrix_bf16.w")
+    _chk(w, "pack_matrix_bf16.w", lp)
     if w.dim() != 2 or w.shape[0] % halves:
         raise KernelError(f"pack_matrix_bf16: shape {tuple(w.shape)} is not {halves} stacked matrices")
     rows, cols = w.shape[0] // halves, w.shape[1]
-    lib = load_lib("vt_gemm_bf16")
+    lib = load_lib("vt_gemm_bf16", half=_half(w))
     lib.vt_packed_elems.restype = ctypes.c_longlong
     per = int(lib.vt_packed_elems(_i(rows), _i(cols)))
-    data = torch.empty(halves * per, dtype=torch.bfloat16, device=w.device)
+    data = torch.empty(halves * per, dtype=lp, device=w.device)
     for h in range(halves):
         _run(lib, "vt_pack_matrix_bf16", _ptr(w[h * rows:(h + 1) * rows]), _ptr(data[h * per:(h + 1) * per]), _i(rows),
              _i(cols), _stream())
@@ -233,9 +264,9 @@ def pack_matrix_bf16(w: torch.Tensor, halves: int = 1) -> PackedMatrix:
 
 def unpack_matrix_bf16(packed: PackedMatrix, out: torch.Tensor) -> torch.Tensor:
     """The row-major matrix [halves * rows, cols] back from its packed form, into `out`."""
-    _chk(packed.data, "unpack_matrix_bf16.packed", torch.bfloat16)
-    _chk(out, "unpack_matrix_bf16.out", torch.bfloat16, (packed.halves * packed.rows, packed.cols))
-    lib = load_lib("vt_gemm_bf16")
+    lp = _lowp(packed.data, "unpack_matrix_bf16.packed")
+    _chk(out, "unpack_matrix_bf16.out", lp, (packed.halves * packed.rows, packed.cols))
+    lib = load_lib("vt_gemm_bf16", half=_half(packed.data))
     per = packed.data.numel() // packed.halves
     for h in range(packed.halves):
         _run(lib, "vt_unpack_matrix_bf16", _ptr(packed.data[h * per:(h + 1) * per]),
@@ -245,7 +276,7 @@ def unpack_matrix_bf16(packed: PackedMatrix, out: torch.Tensor) -> torch.Tensor:
 
 def linear_bf16_workspace(n: int, m: int, k: int) -> int:
     """Floats of scratch memory that linear_bf16 needs for x [n, k], W [m, k] (0: none)."""
-    lib = load_lib("vt_gemm_bf16")
+    lib = _any_build("vt_gemm_bf16")
     lib.vt_linear_bf16_workspace.restype = ctypes.c_longlong
     return int(lib.vt_linear_bf16_workspace(_i(n), _i(m), _i(k), _i(0)))
 
@@ -261,7 +292,7 @@ def linear_bf16_adds_residual(n: int, m: int, k: int) -> bool:
     over blocks (the launch that adds the partial sums then adds the residual too)."""
     key = (n, m, k)
     if key not in _adds_residual:
-        _adds_residual[key] = bool(load_lib("vt_gemm_bf16").vt_linear_bf16_adds_residual(_i(n), _i(m), _i(k)))
+        _adds_residual[key] = bool(_any_build("vt_gemm_bf16").vt_linear_bf16_adds_residual(_i(n), _i(m), _i(k)))
     return _adds_residual[key]
 
 
@@ -276,15 +307,16 @@ def linear_bf16(x: torch.Tensor, w, bias: Optional[torch.Tensor], out: torch.Ten
     residual + the product (17 to 64 rows of a shape whose k range is split: by the launch that adds the partial sums,
     which needs the workspace)."""
     n, k = x.shape
+    lp = _lowp((w.data if isinstance(w, PackedMatrix) else w), "linear_bf16.w")
     if not isinstance(w, PackedMatrix):
-        _chk(w, "linear_bf16.w", torch.bfloat16, (w.shape[0], k))
+        _chk(w, "linear_bf16.w", lp, (w.shape[0], k))
         w = pack_matrix_bf16(w)
     m = w.rows
     if w.cols != k or w.halves != 1:
         raise KernelError(f"linear_bf16: x [{n}, {k}] does not fit a packed matrix [{w.rows}, {w.cols}] x {w.halves}")
     fused = norm_gain is not None or residual is not None
-    _chk(x, "linear_bf16.x", torch.float32 if norm_gain is not None else torch.bfloat16)
-    _chk(w.data, "linear_bf16.w", torch.bfloat16)
+    _chk(x, "linear_bf16.x", torch.float32 if norm_gain is not None else lp)
+    _chk(w.data, "linear_bf16.w", lp)
     _chk(out, "linear_bf16.out", torch.float32 if fused else None, (n, m))
     if bias is not None:
         _chk(bias, "linear_bf16.bias", torch.float32, (m,))
@@ -303,7 +335,7 @@ def linear_bf16(x: torch.Tensor, w, bias: Optional[torch.Tensor], out: torch.Ten
             raise KernelError(f"linear_bf16: x [{n}, {k}] with W [{m}, {k}] needs a workspace of {need} floats")
         if need:
             _chk(workspace, "linear_bf16.workspace", torch.float32)
-        _run(load_lib("vt_gemm_bf16"), "vt_linear_bf16_fused", _ptr(x), _ptr(norm_gain), _f(norm_eps), _ptr(w.data), _ptr(bias),
+        _run(load_lib("vt_gemm_bf16", half=_half(w.data, x, out)), "vt_linear_bf16_fused", _ptr(x), _ptr(norm_gain), _f(norm_eps), _ptr(w.data), _ptr(bias),
              _ptr(residual), _ptr(out), _ptr(workspace if need else None), _i(n), _i(m), _i(k), _stream())
         return out
     need = linear_bf16_workspace(n, m, k) if n > 16 else 0
@@ -313,7 +345,7 @@ def linear_bf16(x: torch.Tensor, w, bias: Optional[torch.Tensor], out: torch.Ten
         _chk(workspace, "linear_bf16.workspace", torch.float32)
         if workspace.numel() < need:
             raise KernelError(f"linear_bf16: workspace of {workspace.numel()} floats, need {need}")
-    _run(load_lib("vt_gemm_bf16"), "vt_linear_bf16", _ptr(x), _ptr(w.data), _ptr(bias), _ptr(out), _i(_code(out)),
+    _run(load_lib("vt_gemm_bf16", half=_half(w.data, x, out)), "vt_linear_bf16", _ptr(x), _ptr(w.data), _ptr(bias), _ptr(out), _i(_code(out)),
          _ptr(workspace if need else None), _i(n), _i(m), _i(k), _stream())
     return out
 
@@ -326,7 +358,7 @@ def linear_bf16_link_shares(n: int, m: int, k: int) -> int:
     the product behind it (linear_bf16_link with xn_out); 0: this shape cannot."""
     key = (n, m, k)
     if key not in _link_shares:
-        _link_shares[key] = int(load_lib("vt_gemm_bf16").vt_linear_bf16_link_shares(_i(n), _i(m), _i(k)))
+        _link_shares[key] = int(_any_build("vt_gemm_bf16").vt_linear_bf16_link_shares(_i(n), _i(m), _i(k)))
     return _link_shares[key]
 
 
@@ -346,11 +378,12 @@ def linear_bf16_link(x: torch.Tensor, w: PackedMatrix, bias: Optional[torch.Tens
     product's own shares ssq_out (float32 [linear_bf16_link_shares(n, m, k), link_stride(n)]) for the product behind
     the next norm.  workspace: as for linear_bf16."""
     n, k = x.shape
+    lp = _lowp(w.data, "linear_bf16_link.w")
     m = w.rows
     if w.cols != k or w.halves != 1:
         raise KernelError(f"linear_bf16_link: x [{n}, {k}] does not fit a packed matrix [{w.rows}, {w.cols}] x {w.halves}")
-    _chk(x, "linear_bf16_link.x", torch.bfloat16)
-    _chk(w.data, "linear_bf16_link.w", torch.bfloat16)
+    _chk(x, "linear_bf16_link.x", lp)
+    _chk(w.data, "linear_bf16_link.w", lp)
     _chk(out, "linear_bf16_link.out", torch.float32, (n, m))
     if bias is not None:
         _chk(bias, "linear_bf16_link.bias", torch.float32, (m,))
@@ -368,7 +401,7 @@ def linear_bf16_link(x: torch.Tensor, w: PackedMatrix, bias: Optional[torch.Tens
         shares = linear_bf16_link_shares(n, m, k)
         if residual is None or shares == 0:
             raise KernelError(f"linear_bf16_link: {n} rows of [{m}, {k}] cannot hand a norm on (linear_bf16_link_shares)")
-        _chk(xn_out, "linear_bf16_link.xn_out", torch.bfloat16, (n, m))
+        _chk(xn_out, "linear_bf16_link.xn_out", lp, (n, m))
         _chk(gain_next, "linear_bf16_link.gain_next", torch.float32, (m,))
         _chk(ssq_out, "linear_bf16_link.ssq_out", torch.float32, (shares, link_stride(n)))
     need = linear_bf16_workspace(n, m, k) if n > 16 else 0
@@ -376,7 +409,7 @@ def linear_bf16_link(x: torch.Tensor, w: PackedMatrix, bias: Optional[torch.Tens
         if workspace is None or workspace.numel() < need:
             raise KernelError(f"linear_bf16_link: x [{n}, {k}] with W [{m}, {k}] needs a workspace of {need} floats")
         _chk(workspace, "linear_bf16_link.workspace", torch.float32)
-    _run(load_lib("vt_gemm_bf16"), "vt_linear_bf16_link", _ptr(x), _ptr(w.data), _ptr(bias), _ptr(residual), _ptr(out),
+    _run(load_lib("vt_gemm_bf16", half=_half(w.data, x, out)), "vt_linear_bf16_link", _ptr(x), _ptr(w.data), _ptr(bias), _ptr(residual), _ptr(out),
          _ptr(workspace if need else None), _i(n), _i(m), _i(k), _ptr(ssq_in), _i(n_ssq), _f(eps_in), _ptr(xn_out),
          _ptr(gain_next), _ptr(ssq_out), _stream())
     return out
@@ -387,16 +420,17 @@ def gated_linear_bf16_link(x: torch.Tensor, w: PackedMatrix, out: torch.Tensor, 
     """gated_linear_bf16 behind an RMSNorm that the product in front has prepared: x = bf16(h * gain), ssq_in its
     shares of the rows' sums of squares (up to 64 rows)."""
     n, k = x.shape
+    lp = _lowp(w.data, "gated_linear_bf16_link.w")
     if w.cols != k or w.halves != 2:
         raise KernelError(f"gated_linear_bf16_link: x [{n}, {k}] does not fit a packed matrix [{w.rows}, {w.cols}] x {w.halves}")
-    _chk(x, "gated_linear_bf16_link.x", torch.bfloat16)
-    _chk(w.data, "gated_linear_bf16_link.w", torch.bfloat16)
+    _chk(x, "gated_linear_bf16_link.x", lp)
+    _chk(w.data, "gated_linear_bf16_link.w", lp)
     _chk(out, "gated_linear_bf16_link.out", None, (n, w.rows))
     _chk(ssq_in, "gated_linear_bf16_link.ssq_in", torch.float32)
     if n > 64 or ssq_in.dim() != 2 or ssq_in.shape[1] != link_stride(n):
         raise KernelError(f"gated_linear_bf16_link: {n} rows, ssq_in of shape {tuple(ssq_in.shape)}: up to 64 rows and "
                           f"[shares, {link_stride(n)}]")
-    _run(load_lib("vt_gemm_bf16"), "vt_gated_linear_bf16_link", _ptr(x), _ptr(w.data), _ptr(out), _i(_code(out)), _i(n),
+    _run(load_lib("vt_gemm_bf16", half=_half(w.data, x, out)), "vt_gated_linear_bf16_link", _ptr(x), _ptr(w.data), _ptr(out), _i(_code(out)), _i(n),
          _i(w.rows), _i(k), _ptr(ssq_in), _i(ssq_in.shape[0]), _f(eps_in), _stream())
     return out
 
@@ -407,20 +441,21 @@ def gated_linear_bf16(x: torch.Tensor, w_gate_up, out: torch.Tensor, norm_gain: 
     the stacked [2 I, k] tensor, which is packed on the spot.  With norm_gain (up to 16 rows), x is the float32
     residual stream and rmsnorm(x; gain, eps) is what gets multiplied."""
     n, k = x.shape
+    lp = _lowp((w_gate_up.data if isinstance(w_gate_up, PackedMatrix) else w_gate_up), "gated_linear_bf16.w")
     if not isinstance(w_gate_up, PackedMatrix):
-        _chk(w_gate_up, "gated_linear_bf16.w", torch.bfloat16, (w_gate_up.shape[0], k))
+        _chk(w_gate_up, "gated_linear_bf16.w", lp, (w_gate_up.shape[0], k))
         w_gate_up = pack_matrix_bf16(w_gate_up, halves=2)
     w = w_gate_up
     if w.cols != k or w.halves != 2:
         raise KernelError(f"gated_linear_bf16: x [{n}, {k}] does not fit a packed matrix [{w.rows}, {w.cols}] x {w.halves}")
-    _chk(x, "gated_linear_bf16.x", torch.float32 if norm_gain is not None else torch.bfloat16)
-    _chk(w.data, "gated_linear_bf16.w", torch.bfloat16)
+    _chk(x, "gated_linear_bf16.x", torch.float32 if norm_gain is not None else lp)
+    _chk(w.data, "gated_linear_bf16.w", lp)
     _chk(out, "gated_linear_bf16.out", None, (n, w.rows))
     if norm_gain is not None:
         if n > 16 or k % 8:
             raise KernelError(f"gated_linear_bf16: the fused norm takes at most 16 rows and k a multiple of 8 (n={n}, k={k})")
         _chk(norm_gain, "gated_linear_bf16.norm_gain", torch.float32, (k,))
-    _run(load_lib("vt_gemm_bf16"), "vt_gated_linear_bf16", _ptr(x), _ptr(w.data), _ptr(out), _i(_code(out)), _i(n),
+    _run(load_lib("vt_gemm_bf16", half=_half(w.data, x, out)), "vt_gated_linear_bf16", _ptr(x), _ptr(w.data), _ptr(out), _i(_code(out)), _i(n),
          _i(w.rows), _i(k), _ptr(norm_gain), _f(norm_eps), _stream())
     return out
 
@@ -458,16 +493,17 @@ def attention_bf16(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor
     number of partial indices it used, checked against the workspace here."""
     n = q.shape[0]
     num_pages, kvh, page_size, d = k_pages.shape
+    lp = _lowp(k_pages, "attention_bf16.k_pages")
     if head_dim % 16 or not 16 <= head_dim <= 256:
         raise KernelError(f"attention_bf16: head size {head_dim} is not a multiple of 16 in 16..256")
     if rt not in (1, 2, 3):
         raise KernelError(f"attention_bf16: {rt} row tiles per item (1 or 2)")
-    _chk(q, "attention_bf16.q", torch.bfloat16, (n, n_heads * head_dim))
-    _chk(k_pages, "attention_bf16.k_pages", torch.bfloat16, (num_pages, n_kv, page_size, head_dim))
-    _chk(v_pages, "attention_bf16.v_pages", torch.bfloat16, (num_pages, n_kv, head_dim, page_size))
+    _chk(q, "attention_bf16.q", lp, (n, n_heads * head_dim))
+    _chk(k_pages, "attention_bf16.k_pages", lp, (num_pages, n_kv, page_size, head_dim))
+    _chk(v_pages, "attention_bf16.v_pages", lp, (num_pages, n_kv, head_dim, page_size))
     _chk(block_table, "attention_bf16.block_table", torch.int32)
     _chk(items, "attention_bf16.items", torch.int32)
-    _chk(out, "attention_bf16.out", torch.bfloat16, (n, n_heads * head_dim))
+    _chk(out, "attention_bf16.out", lp, (n, n_heads * head_dim))
     if items.numel() < n_items * ATTN_ITEM_INTS:
         raise KernelError("attention_bf16: item list shorter than n_items")
     if n_citems:
@@ -478,7 +514,7 @@ def attention_bf16(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor
             raise KernelError("attention_bf16: combine list shorter than n_citems")
         if part_o.numel() < max_part * rt * n_kv * 16 * head_dim or part_ml.numel() < max_part * rt * n_kv * 16 * 2:
             raise KernelError("attention_bf16: workspace for split keys is too small")
-    lib = load_lib("vt_attn_bf16", head_dim)
+    lib = load_lib("vt_attn_bf16", head_dim, half=_half(k_pages, v_pages, out))
     _run(lib, "vt_attn_bf16", _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(block_table), _ptr(items), _i(n_items), _i(rt),
          _ptr(citems), _i(n_citems), _ptr(out), _ptr(part_o), _ptr(part_ml), _i(n_heads), _i(n_kv), _i(page_size),
          _i(block_table.shape[1]), _i(num_pages), _i(window), _f(scale), _stream())
@@ -488,7 +524,7 @@ def attention_bf16(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor
 def attention_bf16_direct(head_dim: int) -> bool:
     """Whether the bfloat16 attention kernels of this head size load their key/value blocks straight into LDS; the
     host cuts their work differently then (parts.attention_plan)."""
-    return bool(load_lib("vt_attn_bf16", head_dim).vt_attn_bf16_direct())
+    return bool(_any_build("vt_attn_bf16", head_dim).vt_attn_bf16_direct())
 
 
 def attention_bf16_tiles(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
@@ -503,16 +539,17 @@ def attention_bf16_tiles(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
     16 * head_dim and n_parts * 4 * rt * n_kv * 32 elements."""
     n = q.shape[0]
     num_pages, kvh, page_size, d = k_pages.shape
+    lp = _lowp(k_pages, "attention_bf16_tiles.k_pages")
     if head_dim % 16 or not 16 <= head_dim <= 256:
         raise KernelError(f"attention_bf16_tiles: head size {head_dim} is not a multiple of 16 in 16..256")
     if rt not in (1, 2):
         raise KernelError(f"attention_bf16_tiles: {rt} row tiles per wave (1 or 2)")
-    _chk(q, "attention_bf16_tiles.q", torch.bfloat16, (n, n_heads * head_dim))
-    _chk(k_pages, "attention_bf16_tiles.k_pages", torch.bfloat16, (num_pages, n_kv, page_size, head_dim))
-    _chk(v_pages, "attention_bf16_tiles.v_pages", torch.bfloat16, (num_pages, n_kv, head_dim, page_size))
+    _chk(q, "attention_bf16_tiles.q", lp, (n, n_heads * head_dim))
+    _chk(k_pages, "attention_bf16_tiles.k_pages", lp, (num_pages, n_kv, page_size, head_dim))
+    _chk(v_pages, "attention_bf16_tiles.v_pages", lp, (num_pages, n_kv, head_dim, page_size))
     _chk(block_table, "attention_bf16_tiles.block_table", torch.int32)
     _chk(items, "attention_bf16_tiles.items", torch.int32)
-    _chk(out, "attention_bf16_tiles.out", torch.bfloat16, (n, n_heads * head_dim))
+    _chk(out, "attention_bf16_tiles.out", lp, (n, n_heads * head_dim))
     if items.numel() < n_items * ATTN_ITEM_INTS:
         raise KernelError("attention_bf16_tiles: item list shorter than n_items")
     if n_citems or n_parts:
@@ -525,7 +562,7 @@ def attention_bf16_tiles(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
             raise KernelError("attention_bf16_tiles: combine list shorter than n_citems")
         if part_o.numel() < n_parts * 4 * rt * n_kv * 16 * head_dim or part_ml.numel() < n_parts * 4 * rt * n_kv * 32:
             raise KernelError(f"attention_bf16_tiles: workspaces too small for {n_parts} partial results")
-    _run(load_lib("vt_attn_bf16", head_dim), "vt_attn_bf16_tiles", _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
+    _run(load_lib("vt_attn_bf16", head_dim, half=_half(k_pages, v_pages, out)), "vt_attn_bf16_tiles", _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
          _ptr(items), _i(n_items), _i(rt), _ptr(citems if n_citems else None), _i(n_citems), _ptr(out),
          _ptr(part_o if n_citems else None), _ptr(part_ml if n_citems else None), _i(n_heads), _i(n_kv), _i(page_size),
          _i(block_table.shape[1]), _i(num_pages), _i(window), _f(scale), _stream())
@@ -540,22 +577,23 @@ def attention_bf16_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch
     p_max items of dec_params[0] keys.  All that changes from step to step is read from device memory."""
     n = q.shape[0]
     num_pages, kvh, page_size, d = k_pages.shape
+    lp = _lowp(k_pages, "attention_bf16_decode.k_pages")
     if head_dim % 16 or not 16 <= head_dim <= 256:
         raise KernelError(f"attention_bf16_decode: head size {head_dim} is not a multiple of 16 in 16..256")
-    _chk(q, "attention_bf16_decode.q", torch.bfloat16, (n, n_heads * head_dim))
-    _chk(k_pages, "attention_bf16_decode.k_pages", torch.bfloat16, (num_pages, n_kv, page_size, head_dim))
-    _chk(v_pages, "attention_bf16_decode.v_pages", torch.bfloat16, (num_pages, n_kv, head_dim, page_size))
+    _chk(q, "attention_bf16_decode.q", lp, (n, n_heads * head_dim))
+    _chk(k_pages, "attention_bf16_decode.k_pages", lp, (num_pages, n_kv, page_size, head_dim))
+    _chk(v_pages, "attention_bf16_decode.v_pages", lp, (num_pages, n_kv, head_dim, page_size))
     _chk(block_table, "attention_bf16_decode.block_table", torch.int32)
     if block_table.shape[0] < n:
         raise KernelError("attention_bf16_decode: fewer block table rows than entries")
     _chk(entry_pos0, "attention_bf16_decode.entry_pos0", torch.int32, (n,))
     _chk(dec_params, "attention_bf16_decode.dec_params", torch.int32)
-    _chk(out, "attention_bf16_decode.out", torch.bfloat16, (n, n_heads * head_dim))
+    _chk(out, "attention_bf16_decode.out", lp, (n, n_heads * head_dim))
     _chk(part_o, "attention_bf16_decode.part_o", torch.float32)
     _chk(part_ml, "attention_bf16_decode.part_ml", torch.float32)
     if part_o.numel() < n * p_max * n_kv * 16 * head_dim or part_ml.numel() < n * p_max * n_kv * 32:
         raise KernelError("attention_bf16_decode: workspace too small")
-    _run(load_lib("vt_attn_bf16", head_dim), "vt_attn_bf16_decode", _ptr(q), _ptr(k_pages), _ptr(v_pages),
+    _run(load_lib("vt_attn_bf16", head_dim, half=_half(k_pages, v_pages, out)), "vt_attn_bf16_decode", _ptr(q), _ptr(k_pages), _ptr(v_pages),
          _ptr(block_table), _ptr(entry_pos0), _ptr(dec_params), _i(n), _i(p_max), _ptr(out), _ptr(part_o), _ptr(part_ml),
          _i(n_heads), _i(n_kv), _i(page_size), _i(block_table.shape[1]), _i(num_pages), _i(window), _f(scale), _stream())
     return out
@@ -570,6 +608,7 @@ def attention_bf16_decode_fused(qkv: torch.Tensor, cos: Optional[torch.Tensor], 
     the attention kernel rotates queries and the new key and writes key and value into the token's page itself."""
     n = qkv.shape[0]
     num_pages, kvh, page_size, d = k_pages.shape
+    lp = _lowp(k_pages, "attention_bf16_decode_fused.k_pages")
     if head_dim % 16 or not 16 <= head_dim <= 256:
         raise KernelError(f"attention_bf16_decode_fused: head size {head_dim} is not a multiple of 16 in 16..256")
     _chk(qkv, "attention_bf16_decode_fused.qkv", torch.float32)
@@ -583,19 +622,19 @@ def attention_bf16_decode_fused(qkv: torch.Tensor, cos: Optional[torch.Tensor], 
         rot = 2 * half
         if rot % 16 or rot > head_dim:
             raise KernelError(f"attention_bf16_decode_fused: {rot} rotated dims (a multiple of 16 up to {head_dim})")
-    _chk(k_pages, "attention_bf16_decode_fused.k_pages", torch.bfloat16, (num_pages, n_kv, page_size, head_dim))
-    _chk(v_pages, "attention_bf16_decode_fused.v_pages", torch.bfloat16, (num_pages, n_kv, head_dim, page_size))
+    _chk(k_pages, "attention_bf16_decode_fused.k_pages", lp, (num_pages, n_kv, page_size, head_dim))
+    _chk(v_pages, "attention_bf16_decode_fused.v_pages", lp, (num_pages, n_kv, head_dim, page_size))
     _chk(block_table, "attention_bf16_decode_fused.block_table", torch.int32)
     if block_table.shape[0] < n:
         raise KernelError("attention_bf16_decode_fused: fewer block table rows than entries")
     _chk(entry_pos0, "attention_bf16_decode_fused.entry_pos0", torch.int32, (n,))
     _chk(dec_params, "attention_bf16_decode_fused.dec_params", torch.int32)
-    _chk(out, "attention_bf16_decode_fused.out", torch.bfloat16, (n, n_heads * head_dim))
+    _chk(out, "attention_bf16_decode_fused.out", lp, (n, n_heads * head_dim))
     _chk(part_o, "attention_bf16_decode_fused.part_o", torch.float32)
     _chk(part_ml, "attention_bf16_decode_fused.part_ml", torch.float32)
     if part_o.numel() < n * p_max * n_kv * 16 * head_dim or part_ml.numel() < n * p_max * n_kv * 32:
         raise KernelError("attention_bf16_decode_fused: workspace too small")
-    _run(load_lib("vt_attn_bf16", head_dim), "vt_attn_bf16_decode_fused", _ptr(qkv), ctypes.c_longlong(qkv.stride(0)),
+    _run(load_lib("vt_attn_bf16", head_dim, half=_half(k_pages, v_pages, out)), "vt_attn_bf16_decode_fused", _ptr(qkv), ctypes.c_longlong(qkv.stride(0)),
          _ptr(cos), _ptr(sin), _i(rot), _i(max_pos), _ptr(k_pages), _ptr(v_pages), _ptr(block_table), _ptr(entry_pos0),
          _ptr(dec_params), _i(n), _i(p_max), _ptr(out), _ptr(part_o), _ptr(part_ml), _i(n_heads), _i(n_kv),
          _i(page_size), _i(block_table.shape[1]), _i(num_pages), _i(window), _f(scale), _stream())

@@ -48,8 +48,8 @@ class PagedAttention(Part):
         self.rt = rt
         self.width = int(width)
         self.nh, self.nkv, self.d = int(num_heads), int(num_kv_heads), int(head_dim)
-        if rt.dtype == torch.bfloat16 and (self.d % 16 or not 16 <= self.d <= 256):
-            raise ValueError(f"head size {self.d}: the bfloat16 attention kernels take multiples of 16 from 16 to 256 "
+        if rt.lowp and (self.d % 16 or not 16 <= self.d <= 256):
+            raise ValueError(f"head size {self.d}: the 16-bit attention kernels take multiples of 16 from 16 to 256 "
                              f"(float32 takes any)")
         self.qkv_bias, self.out_bias = bool(qkv_bias), bool(out_bias)
         self.window = int(window)
@@ -76,8 +76,8 @@ class PagedAttention(Part):
 
     # -- what the cache manager must hold for this mixer --------------------
     def cache_need(self) -> Optional[CacheNeed]:
-        # the bfloat16 kernels read keys 16 at a time, from one page
-        return CacheNeed(self.nkv, self.d, self.window, page_multiple=16 if self.rt.dtype == torch.bfloat16 else 1)
+        # the 16-bit kernels read keys 16 at a time, from one page
+        return CacheNeed(self.nkv, self.d, self.window, page_multiple=16 if self.rt.lowp else 1)
 
     def state_need(self) -> Optional[StateNeed]:
         return None
@@ -104,7 +104,7 @@ class PagedAttention(Part):
         self.w_qkv = torch.cat([rt.place(get(nm[k] + ".weight"), "matrix") for k in "qkv"], dim=0).contiguous()
         if self.qkv_bias:
             self.b_qkv = torch.cat([rt.place(get(nm[k] + ".bias"), "bias") for k in "qkv"], dim=0).contiguous()
-            self.b_qkv_lowp = self.b_qkv.to(torch.bfloat16)
+            self.b_qkv_lowp = self.b_qkv.to(rt.dtype)
         self.w_o = rt.place(get(nm["o"] + ".weight"), "matrix")
         if self.out_bias:
             self.b_o = rt.place(get(nm["o"] + ".bias"), "bias")
@@ -130,7 +130,7 @@ class PagedAttention(Part):
         (one token per entry): the number of keys per work item, one integer, so that a captured step can be
         replayed with another one.  Any other step: the work items of the planned kernels.  Layers of the same
         shape share one plan."""
-        if self.rt.dtype != torch.bfloat16:
+        if not self.rt.lowp:
             return None
         if ctx.single_token and self.nh // self.nkv <= DECODE_MAX_GROUP:
             key = self._decode_key()
@@ -181,7 +181,7 @@ class PagedAttention(Part):
                 qkv[:, nq:nq + nkv * d] = k2.reshape(n, nkv * d).to(qkv.dtype)
         cos, sin = tables if tables is not None else (None, None)
         plain_positions = tables is not None or getattr(self.position, "dim", 0) == 0
-        chunk = ctx.extra.get(self._decode_key()) if rt.dtype == torch.bfloat16 and ctx.single_token else None
+        chunk = ctx.extra.get(self._decode_key()) if rt.lowp and ctx.single_token else None
         p_max = decode_parts_max(ctx.n_positions)
         if (chunk is not None and cache.writes and qkv.dtype == torch.float32
                 and plain_positions and (cos is None or cos.shape[1] % 8 == 0)):

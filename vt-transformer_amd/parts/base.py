@@ -46,7 +46,7 @@ from ..config.base import ConfigError, PartSpec
 class TensorDecl:
     """A tensor that a part needs: its shape and what it is.
 
-    role "matrix": kept in the runtime's dtype (bfloat16 or float32);
+    role "matrix": kept in the runtime's dtype (bfloat16, float16 or float32);
     "gain", "bias": small vectors, kept in float32 (exact from bfloat16);
     "table": integers, kept as int32.  A tensor stored in 32-bit stays so."""
 
@@ -80,15 +80,18 @@ class Runtime:
     """Device, dtype and scratch buffers shared by the parts of one model."""
 
     def __init__(self, device: torch.device, dtype: torch.dtype, keep_row_major: bool = True):
-        if dtype not in (torch.bfloat16, torch.float32):
-            raise ValueError(f"dtype {dtype} is not supported (bfloat16 and float32 are)")
+        if dtype not in (torch.bfloat16, torch.float16, torch.float32):
+            raise ValueError(f"dtype {dtype} is not supported (bfloat16, float16 and float32 are)")
         self.device = device
         self.dtype = dtype
-        # bfloat16 keeps every matrix twice: row-major for the GEMM library (long portions) and packed for the
+        # a 16-bit type (bfloat16, or float16, the reference's own: v1/tensortype/hip_tensor.cpp:514-535): the
+        # matrix-core kernels; float32: the true 32-bit path
+        self.lowp = dtype != torch.float32
+        # a 16-bit model keeps every matrix twice: row-major for the GEMM library (long portions) and packed for the
         # few-row kernels.  False: the packed copy only, and long portions go through the few-row kernels 64 rows
         # at a time, which reads W once per 64 rows: several times slower on prompts, half the memory (a model
         # that fits the GPU once but not twice).
-        self.keep_row_major = bool(keep_row_major) or dtype != torch.bfloat16
+        self.keep_row_major = bool(keep_row_major) or not self.lowp
         self._buffers: Dict[str, torch.Tensor] = {}
         self._scope = ""
 
@@ -105,9 +108,9 @@ class Runtime:
         raise ValueError(f"unknown tensor role {role!r}")
 
     def pack(self, w: torch.Tensor, halves: int = 1):
-        """The bfloat16 matrix once more in the order the few-row matrix kernels read it (None in float32).  The
+        """The 16-bit matrix once more in the order the few-row matrix kernels read it (None in float32).  The
         row-major matrix stays for the GEMM library, which long portions go through."""
-        if self.dtype != torch.bfloat16:
+        if not self.lowp:
             return None
         from ..kernels import ops
         return ops.pack_matrix_bf16(w, halves)

@@ -69,7 +69,7 @@ class GatedMLP(Part):
                 (can_fuse(rt, n) and self.width % 8 == 0)
             if not ok:
                 x, normed = x.materialize(), False
-        if rt.dtype == torch.bfloat16 and (n <= GATED_MAX_ROWS or (self.w_gu is None and (rt.keep_row_major or n < UNPACK_MIN_ROWS))):
+        if rt.lowp and (n <= GATED_MAX_ROWS or (self.w_gu is None and (rt.keep_row_major or n < UNPACK_MIN_ROWS))):
             w = self.p_gu if self.p_gu is not None else self.w_gu
             if normed and x.prepared:
                 ops.gated_linear_bf16_link(x.xn, w, act, x.ssq, x.eps)

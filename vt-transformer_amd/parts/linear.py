@@ -44,23 +44,23 @@ FUSE_MAX_ROWS = ops.NORM_MAX_ROWS
 
 def can_fuse(rt: Runtime, n: int) -> bool:
     """Whether a product of n rows can take the residual stream with its norm still to be applied."""
-    return rt.dtype == torch.bfloat16 and n <= FUSE_MAX_ROWS
+    return rt.lowp and n <= FUSE_MAX_ROWS
 
 
 def can_add_residual(rt: Runtime, n: int, m: int, k: int) -> bool:
     """Whether the product of n rows with W [m, k] can add its result to the residual stream itself: it can where
     no k range is split over blocks (up to 16 rows; 17 to 64 for matrices that the kernel for it suits)."""
-    return rt.dtype == torch.bfloat16 and ops.linear_bf16_adds_residual(n, m, k)
+    return rt.lowp and ops.linear_bf16_adds_residual(n, m, k)
 
 
 def can_hand_norm_on(rt: Runtime, n: int, m: int, k: int) -> bool:
     """Whether the product of n rows with W [m, k], adding to the residual stream, can prepare the norm behind it."""
-    return rt.dtype == torch.bfloat16 and n <= ops.LINK_MAX_ROWS and ops.linear_bf16_link_shares(n, m, k) > 0
+    return rt.lowp and n <= ops.LINK_MAX_ROWS and ops.linear_bf16_link_shares(n, m, k) > 0
 
 
 def takes_prepared_norm(rt: Runtime, n: int, k: int) -> bool:
     """Whether a product of n rows over k can take a norm that the product in front has prepared."""
-    return rt.dtype == torch.bfloat16 and n <= ops.LINK_MAX_ROWS and k % 8 == 0
+    return rt.lowp and n <= ops.LINK_MAX_ROWS and k % 8 == 0
 
 
 def linear(rt: Runtime, x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], name: str,
@@ -68,7 +68,7 @@ def linear(rt: Runtime, x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.T
            packed=None, residual: Optional[torch.Tensor] = None, hand_on=None):
     """x [N, K] in the runtime's dtype -> [N, M].  `name` keys the output's scratch buffer.
     Output dtype: float32 from the hand-written kernels unless `out_dtype` says otherwise; the
-    library path returns bfloat16 (its bias, if any, is `bias_lowp`, the same values in bfloat16).
+    library path returns the 16-bit type (its bias, if any, is `bias_lowp`, the same values in that type).
     packed: W as rt.pack(w) made it, for the few-row kernel (made on the spot if missing: slow).
     x may be a NormedInput (the norm then happens inside the few-row kernel, or before the product as a kernel of
     its own where that is not possible).  residual (float32 [N, M]): the product is added to it in place and
@@ -96,7 +96,7 @@ def linear(rt: Runtime, x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.T
             if emits or (norm is not None and norm.prepared):
                 xn = ssq = None
                 if emits:
-                    xn = rt.buffer(name + ".xn", (n, m), torch.bfloat16)
+                    xn = rt.buffer(name + ".xn", (n, m), rt.dtype)
                     ssq = rt.buffer(name + ".ssq", (ops.linear_bf16_link_shares(n, m, k), ops.link_stride(n)), torch.float32)
                 ops.linear_bf16_link(norm.xn if norm else x, w_any, bias, out, residual=residual,
                                      ssq_in=norm.ssq if norm else None, eps_in=norm.eps if norm else 0.0,
@@ -113,16 +113,16 @@ def linear(rt: Runtime, x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.T
         return ops.linear_f32(x, w, bias, out)
     if w is None and not rt.keep_row_major and n >= UNPACK_MIN_ROWS:
         # every product's matrix in turn in the same scratch memory (the largest one's size)
-        w = ops.unpack_matrix_bf16(packed, rt.buffer("linear.unpacked", (packed.halves * packed.rows, packed.cols), torch.bfloat16))
+        w = ops.unpack_matrix_bf16(packed, rt.buffer("linear.unpacked", (packed.halves * packed.rows, packed.cols), rt.dtype))
     if w is None or n <= (packed_kernel_rows(m, k) if packed is not None else SKINNY_MAX_ROWS):
         out = rt.buffer(name, (n, m), out_dtype or torch.float32)
         need = ops.linear_bf16_workspace(n, m, k) if n > 16 else 0
         work = rt.buffer("linear.partials", (need,), torch.float32) if need else None
         return ops.linear_bf16(x, packed if packed is not None else w, bias, out, work)
-    out = rt.buffer(name + ".lib", (n, m), torch.bfloat16)
+    out = rt.buffer(name + ".lib", (n, m), rt.dtype)
     if bias is not None:
         if bias_lowp is None:
-            bias_lowp = bias.to(torch.bfloat16)
+            bias_lowp = bias.to(rt.dtype)
         torch.addmm(bias_lowp, x, w.t(), out=out)
     else:
         torch.mm(x, w.t(), out=out)
