@@ -45,8 +45,9 @@ def main() -> int:
     ap.add_argument("--prompt-len", type=int, default=1024)
     ap.add_argument("--sizes", choices=sorted(SIZES), default="7b",
                     help="layer sizes; 72b keeps one copy of the weights (long prompt portions unpack each matrix for the library)")
-    ap.add_argument("--dtype", choices=["bfloat16", "float16"], default="bfloat16",
-                    help="the 16-bit type of weights, activations and cache (the same kernels and rates either way)")
+    ap.add_argument("--dtype", choices=["bfloat16", "float16"], default="float16",
+                    help="the 16-bit type of weights, activations and cache: float16 as in the reference's "
+                         "inference_fp16.dag, or bfloat16 (the same kernels and rates either way)")
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the model has (named in config)")
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
