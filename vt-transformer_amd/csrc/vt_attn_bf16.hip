@@ -404,15 +404,15 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : (DECODE && !DIRECT ? 3 : 2)) voi
     // (late_first), or its second (late_second), is then asked for after that.
     const bool late_first = DECODE && a.qkv && dec_writes && min(j_first, j_end) + 16 > pos0;
     const bool late_second = DECODE && a.qkv && dec_writes && j_first + j_step + 16 > pos0;
-    if (DECODE && a.qkv) {
-        if constexpr (DIRECT) {
-            if (!late_first) {
-                if (j_first < key_hi) issue(j_first, page_at(j_first), 0);
-                if (j_first + j_step < key_hi && !late_second) issue(j_first + j_step, page_at(j_first + j_step), 1);
-            }
-        } else {
-            load_block<DECODE>(cur, a, page_at(j_first), spare, min(j_first, j_end), kvh, lane);
+    if constexpr (DIRECT) {
+        // (every wave does, decoding or not: the loads of the rows below are then younger than these, and where the
+        // compiler waits for them it waits for nothing that the first step does not need anyway)
+        if (!late_first) {
+            if (j_first < key_hi) issue(j_first, page_at(j_first), 0);
+            if (j_first + j_step < key_hi && !late_second) issue(j_first + j_step, page_at(j_first + j_step), 1);
         }
+    } else if (DECODE && a.qkv) {
+        load_block<DECODE>(cur, a, page_at(j_first), spare, min(j_first, j_end), kvh, lane);
     }
 
     bool row_ok[RT];
@@ -472,6 +472,15 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : (DECODE && !DIRECT ? 3 : 2)) voi
             } else {
 #pragma unroll
                 for (int s = 0; s < QSTEPS; ++s) { U8 t; t.u = *(const uint2*)(qrow + s * 16 + g * 4); q4[rt][s] = t.v; }
+            }
+            if constexpr (DIRECT) {
+                // The compiler does not know of the loads into LDS and counts only its own.  Left to itself it waits
+                // for these rows at their first use, inside the loop over the keys, with a count that is right for
+                // its loads alone: in every turn that wait takes the block that was only just asked for with it, and
+                // nothing is in flight while a block is multiplied.  So it is made to wait here, once: an empty
+                // statement that "rewrites" the registers.
+#pragma unroll
+                for (int s = 0; s < QSTEPS; ++s) asm volatile("" : "+v"(q8[rt][s]));
             }
         }
 #pragma unroll
@@ -565,7 +574,7 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : (DECODE && !DIRECT ? 3 : 2)) voi
         // which was asked for into the buffer that the last multiplication left.  (Nothing is tested around these
         // loads for the compiler's sake, which does not know of them: a block that the wave does not have is not
         // asked for, and the wait counts the loads that are.)
-        if (!(DECODE && a.qkv) || late_first) {
+        if (late_first) {
             if (j_first < key_hi) issue(j_first, page_at(j_first), 0);
             if (j_first + j_step < key_hi) issue(j_first + j_step, page_at(j_first + j_step), 1);
         } else if (late_second && j_first + j_step < key_hi) {
