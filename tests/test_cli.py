@@ -58,6 +58,20 @@ def test_generate_and_shell(model_folders):
     assert "Exiting shell..." in r.stdout
 
 
+def test_dtype_names_of_the_reference_are_understood():
+    """fp16, bf16 and fp32 as the reference's verify tool spells them
+    (vt-transformer/models/qwen3-0.6b/tools/verify/reference.py:42-46), beside torch's names."""
+    import torch
+    from vt_transformer_amd.engine import parse_dtype
+    assert parse_dtype("fp16") is parse_dtype("float16") is torch.float16
+    assert parse_dtype("bf16") is parse_dtype("bfloat16") is torch.bfloat16
+    assert parse_dtype("fp32") is parse_dtype("float32") is torch.float32
+    with pytest.raises(ValueError, match="int8"):
+        parse_dtype("int8")
+    r = run_cli("--help")
+    assert "fp16" in r.stdout and "float16" in r.stdout
+
+
 def test_bench_refuses_more_than_one_gpu():
     """bench.py measures one GPU: asked for more it says so in one line and exits with 2, before it touches a GPU."""
     import subprocess

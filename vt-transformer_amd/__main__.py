@@ -42,7 +42,8 @@ def build_parser() -> argparse.ArgumentParser:
     p.add_argument("--tokenizer-path", type=str, default="", help="folder or file of a tokenizer.json (default: the model folder)")
     p.add_argument("--model-name", type=str, default="vt_transformer_amd", help="name shown by the shell")
     p.add_argument("--shell-mode", action="store_true", help="interactive shell: a prompt per line, /reset, /exit")
-    p.add_argument("--dtype", choices=["bfloat16", "float16", "float32"], default="bfloat16")
+    # (the reference's tool spells them fp16, bf16 and fp32: vt-transformer/models/qwen3-0.6b/tools/verify/reference.py:42-46, 75)
+    p.add_argument("--dtype", choices=["bfloat16", "float16", "float32", "bf16", "fp16", "fp32"], default="bfloat16")
     # prompts
     p.add_argument("--prompt-ids", action="append", default=[], help="token ids, comma separated (may be repeated)")
     p.add_argument("--prompt-file", type=str, help="one prompt per line: token ids separated by commas or blanks")
