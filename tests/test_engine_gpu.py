@@ -407,6 +407,34 @@ def test_decoding_ahead_of_the_host_gives_the_same_tokens(cfg, tmp_path):
     assert "eos" in reasons and "max_tokens" in reasons                 # both ways of ending happened
 
 
+def test_decoding_ahead_stops_at_a_page_edge_when_no_page_is_free(model_folders):
+    """The only running request decodes ahead of the host with every page taken and crosses a page's edge: the step
+    ahead is not launched, and the request ends for want of pages (alone) or its neighbour is preempted (two of
+    them); Engine.step never raises."""
+    from vt_transformer_amd.engine import Engine
+    from vt_transformer_amd.sampling import SamplingParams
+    cfg = "A"
+    rs = np.random.RandomState(21)
+    vocab = TINY[cfg]["vocab_size"]
+    # alone: 2 pages of 16 tokens, a prompt of 23: token 33 has no page
+    eng = Engine(model_folders[cfg], dtype="bfloat16", num_pages=2, max_running_reqs=2, max_seq_len=128)
+    ahead = []
+    orig = eng._launch
+    eng._launch = lambda plan, ids: (ahead.append(ids is not None), orig(plan, ids))[1]
+    out = eng.generate([rs.randint(0, vocab, size=23).tolist()], SamplingParams(max_tokens=40, ignore_eos=True))
+    assert any(ahead) and eng.finish_reason(0) == "out_of_pages" and len(out[0]) == 10
+    assert sum(eng.runner.cache.held_pages()) == 0 and not eng.has_work()
+    # two requests and three pages: both stand at a page's edge with one page free; the younger gives way
+    eng = Engine(model_folders[cfg], dtype="bfloat16", num_pages=3, max_running_reqs=2, max_seq_len=128)
+    eng.pipeline_decode = True
+    prompts = [rs.randint(0, vocab, size=9).tolist() for _ in range(2)]
+    sp = SamplingParams(max_tokens=12, ignore_eos=True)
+    outs = eng.generate(prompts, sp)
+    assert [eng.finish_reason(i) for i in (0, 1)] == ["max_tokens"] * 2 and eng.requests[1].preemptions >= 1
+    one = Engine(model_folders[cfg], dtype="bfloat16", num_pages=4, max_running_reqs=1, max_seq_len=128)
+    assert outs == [one.generate(p, sp)[0] for p in prompts]
+
+
 def test_decoding_ahead_with_arrivals_aborts_and_few_pages(model_folders):
     """Steps started ahead while requests arrive, are aborted and are preempted for want of pages: every request
     ends with a reason, within its limit, no page or slot stays held, and requests that were never disturbed

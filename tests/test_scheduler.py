@@ -5,7 +5,8 @@ import random
 import pytest
 
 from vt_transformer_amd.cache import CacheManager, GroupSpec
-from vt_transformer_amd.engine.scheduler import (FINISHED, RUNNING, WAITING, Request, Scheduler, SchedulerConfig)
+from vt_transformer_amd.engine.scheduler import (FINISHED, RUNNING, WAITING, Request, Scheduled, Scheduler,
+                                                  SchedulerConfig)
 from vt_transformer_amd.sampling import SamplingParams
 
 EOS = 7
@@ -292,3 +293,113 @@ def test_random_load_always_drains(seed):
     for r in reqs:
         if r.finish_reason == "max_tokens":
             assert len(r.output) == r.params.max_tokens
+
+
+class AheadEngine(FakeEngine):
+    """FakeEngine whose step starts the step after it before it has the tokens, the way Engine.step does: the
+    stand-in for the step function reserves and commits the plan's pages when the plan is launched."""
+
+    def __init__(self, **kw):
+        super().__init__(**kw)
+        self.ahead = None
+        self.launched_ahead = 0
+
+    def _launch(self, plan):
+        items = [(s.request.uid, s.start + s.n_tokens) for s in plan]
+        assert self.cache.reserve(items), "a step was launched that the cache cannot hold"
+        for uid, n in items:
+            self.cache.commit(uid, n)
+        return plan
+
+    def step(self):
+        cur, self.ahead = self.ahead, None
+        if cur is None:
+            plan = self.sched.schedule()
+            self.plans.append([(s.request.uid, s.start, s.n_tokens, s.sample) for s in plan])
+            if not plan:
+                return self.sched.update(plan, {})
+            cur = self._launch(plan)
+        nxt = self.sched.plan_ahead(cur)
+        if nxt is not None:
+            self.ahead = self._launch(nxt)
+            self.launched_ahead += 1
+            self.plans.append([(s.request.uid, s.start, s.n_tokens, s.sample) for s in nxt])
+        sampled = {s.request.uid: self.token(s.request) for s in cur if s.sample}
+        out = self.sched.update(cur, sampled)
+        if self.ahead is not None and not any(s.request.state == RUNNING for s in self.ahead):
+            self.ahead = None
+        self.cache.check()
+        return out
+
+    def run(self, limit=10000):
+        results = []
+        for _ in range(limit):
+            if not (self.sched.has_work() or self.ahead is not None):
+                break
+            results.extend(self.step())
+        assert not self.sched.has_work(), "the scheduler did not finish"
+        return results
+
+
+def test_the_step_ahead_is_checked_against_the_length_after_it():
+    """A lone request crosses a page's edge while it decodes ahead of the host and no page is free: the step ahead
+    is not planned (the step in flight has committed start + 1 tokens, the step ahead needs room for start + 2),
+    and the plain way then ends the request for want of pages instead of raising."""
+    e = AheadEngine(num_pages=2, page_size=4, max_running_reqs=2, max_seq_len=64)
+    a = e.add("a", 7, max_tokens=20)
+    e.step()                                    # the prompt (a portion: nothing is started ahead of it)
+    assert e.launched_ahead == 0 and e.cache.get("a").length == 7
+    e.step()                                    # token 8 fills the second page; token 9 would need a third one
+    assert e.launched_ahead == 0 and e.ahead is None and e.cache.get("a").length == 8
+    plan = [Scheduled(a, 7, 1, True)]           # the step that has just run, as Engine.step hands it on
+    assert e.sched._fits([(a, 8)]) and not e.sched._fits([(a, 9)])
+    assert e.sched.plan_ahead(plan) is None
+    e.run()
+    assert a.finish_reason == "out_of_pages" and a.total_len == 9 and e.cache.held_pages() == [0]
+
+
+def test_decoding_ahead_gives_way_to_preemption_when_pages_run_out():
+    # 3 pages of 4: a and b decode ahead until both stand at a page's edge with one page free; nothing is launched
+    # ahead then, schedule() preempts b, and both finish with the tokens they get alone
+    token = lambda r: 1 + (len(r.output) * 5 + len(r.prompt)) % 4
+    e = AheadEngine(num_pages=3, page_size=4, token=token)
+    a = e.add("a", 2, max_tokens=8)
+    b = e.add("b", 2, max_tokens=8)
+    e.run(limit=200)
+    assert e.launched_ahead > 0 and b.preemptions >= 1 and a.preemptions == 0
+    assert (a.finish_reason, b.finish_reason) == ("max_tokens", "max_tokens")
+    assert a.output == _alone(2, 8, token) and b.output == a.output
+    assert e.cache.held_pages() == [0]
+
+
+@pytest.mark.parametrize("seed", range(30))
+def test_random_load_decoding_ahead_always_drains(seed):
+    rng = random.Random(1000 + seed)
+    page_size = rng.choice([1, 2, 4, 16])
+    e = AheadEngine(num_pages=-(-rng.randint(20, 70) // page_size) + 1, page_size=page_size,
+                    max_running_reqs=rng.randint(1, 5), max_extend_tokens=rng.randint(4, 24),
+                    chunk_size=rng.randint(2, 12), max_seq_len=64, token=lambda r: rng.choice([1, 2, 3, EOS]))
+    reqs = []
+    for step in range(200):
+        if rng.random() < 0.15:
+            reqs.append(e.add(len(reqs), rng.randint(1, 30), max_tokens=rng.randint(1, 20), ignore_eos=rng.random() < 0.5))
+        if rng.random() < 0.03 and reqs:
+            e.sched.abort_request(rng.choice(reqs).uid)
+        e.step()
+    e.run()
+    assert all(r.state == FINISHED for r in reqs) and e.cache.held_pages() == [0]
+    for r in reqs:
+        if r.finish_reason == "max_tokens":
+            assert len(r.output) == r.params.max_tokens
+
+
+def test_random_loads_do_decode_ahead():
+    launched = 0
+    for seed in range(30):
+        rng = random.Random(1000 + seed)
+        e = AheadEngine(num_pages=40, page_size=4, token=lambda r: rng.choice([1, 2, 3]))
+        for i in range(3):
+            e.add(i, rng.randint(1, 20), max_tokens=rng.randint(3, 20))
+        e.run()
+        launched += e.launched_ahead
+    assert launched > 100

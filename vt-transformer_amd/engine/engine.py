@@ -168,24 +168,11 @@ class Engine:
         return plan, (self.sampler.launch(logits, rows) if rows else None)
 
     def _plan_ahead(self, plan: List[Scheduled]) -> Optional[List[Scheduled]]:
-        """The step after `plan`, if it can be told without `plan`'s tokens: `plan` is every running request's one
-        decoding token, nobody waits, nobody reaches a limit with the token it is about to get (an end-of-sequence
-        token may still finish a request: its part of the step ahead is then dropped), the pages are there, and
-        the step goes through a captured graph."""
-        sch = self.scheduler
-        if sch.waiting or sch.finished_early or len(plan) != len(sch.running) or not self.runner.replays(len(plan)):
+        """The step after `plan`, which is already queued on the GPU, if it can be told without `plan`'s tokens
+        (Scheduler.plan_ahead) and goes through a captured graph."""
+        if not self.runner.replays(len(plan)):
             return None
-        nxt = []
-        for s in plan:
-            r = s.request
-            if s.n_tokens != 1 or not s.sample or r.state != "running":
-                return None
-            if len(r.output) + 2 > r.params.max_tokens or r.total_len + 2 > sch.config.max_seq_len:
-                return None     # its last or last but one token: the plain way finishes it
-            nxt.append(Scheduled(r, s.start + 1, 1, True))
-        if not sch._fits([(s.request, s.start + 1) for s in nxt]):
-            return None
-        return nxt
+        return self.scheduler.plan_ahead(plan)
 
     # -- the whole loop --------------------------------------------------------
     def generate(self, prompts: Union[Sequence[int], Sequence[Sequence[int]]],

@@ -285,6 +285,28 @@ class Scheduler:
             budget -= n
         return plan
 
+    def plan_ahead(self, plan: List[Scheduled]) -> Optional[List[Scheduled]]:
+        """The step after `plan`, chosen before `plan`'s tokens are known, or None if it cannot be told yet.
+        `plan` has been handed to the step function (its pages are taken and its lengths committed) but `update`
+        has not seen it.  It can be told if `plan` is every running request's one decoding token, nobody waits,
+        nobody reaches a limit with the token it is about to get (an end-of-sequence token may still finish a
+        request: its part of the step ahead is then dropped), and the pages for one more token each are free: a
+        request that holds start + 1 tokens after `plan` holds start + 2 after the step ahead."""
+        if self.waiting or self.finished_early or len(plan) != len(self.running):
+            return None
+        ahead: List[Scheduled] = []
+        for s in plan:
+            r = s.request
+            if s.n_tokens != 1 or not s.sample or r.state != RUNNING:
+                return None
+            if len(r.output) + 2 > r.params.max_tokens or r.total_len + 2 > self.config.max_seq_len:
+                return None     # its last or last but one token: the plain way finishes it
+            ahead.append(Scheduled(r, s.start + 1, 1, True))
+        lengths_after = [(a.request, a.start + a.n_tokens) for a in ahead]
+        if not self._fits(lengths_after):
+            return None         # a page is missing: the next schedule() preempts or finishes somebody
+        return ahead
+
     # -- after the step ------------------------------------------------------
     def update(self, plan: List[Scheduled], sampled: Dict[Hashable, int]) -> List[ReqResult]:
         """Record what the step stored and the tokens sampled for the portions that asked; finish and free."""
