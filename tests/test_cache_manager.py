@@ -190,38 +190,105 @@ def test_slot_pool():
     assert s.alloc() == 0
 
 
-def test_a_byte_budget_is_shared_by_the_groups_of_layers():
-    """The reference sizes its one pool as budget // (block size x bytes per token)
-    (vt-transformer/models/qwen3-0.6b/init.vt:109-113).  With groups of layers that have pages of their own, a token
-    takes a slot in every group, so the budget is divided by the bytes of one page of each group together."""
+def _kv_need(kv, d, window=0):
+    from vt_transformer_amd.parts.base import CacheNeed, PageTensor
+    return CacheNeed((PageTensor("k", (kv, d), 1), PageTensor("v", (kv, d), 2)), window=window)
+
+
+def _fake_model(needs):
     from types import SimpleNamespace
 
+    from vt_transformer_amd.config.base import ScheduleEntry
+    mixers = [SimpleNamespace(cache_need=lambda n=n: n, state_need=lambda: None) for n in needs]
+    return SimpleNamespace(schedule=[ScheduleEntry(i) for i in range(len(needs))],
+                           layers=[SimpleNamespace(mixer=m) for m in mixers], spec=SimpleNamespace(vocab_size=10))
+
+
+def test_a_byte_budget_is_shared_by_the_groups_of_layers_by_their_needs():
+    """The reference sizes its one pool as budget // (block size x bytes per token)
+    (vt-transformer/models/qwen3-0.6b/init.vt:109-113).  Here groups of layers have pages of their own.  A group with
+    a window gets what its requests can hold at a time (window + a portion, per request) and no more; the rest of the
+    budget is divided by the bytes of one page of each group that keeps every key."""
     import pytest
     import torch
 
     from vt_transformer_amd.cache.storage import CacheStorage
-    from vt_transformer_amd.config.base import ScheduleEntry
-    from vt_transformer_amd.parts.base import CacheNeed, Runtime
-
-    def mixer(kv, d, window):
-        return SimpleNamespace(cache_need=lambda: CacheNeed(kv, d, window), state_need=lambda: None)
+    from vt_transformer_amd.parts.base import Runtime
 
     # three layers keep every key of 2 heads x 16; two keep a window of 8 keys of 1 head x 32
-    mixers = [mixer(2, 16, 0), mixer(1, 32, 8), mixer(2, 16, 0), mixer(1, 32, 8), mixer(2, 16, 0)]
-    model = SimpleNamespace(schedule=[ScheduleEntry(i) for i in range(5)],
-                            layers=[SimpleNamespace(mixer=m) for m in mixers], spec=SimpleNamespace(vocab_size=10))
+    needs = [_kv_need(2, 16), _kv_need(1, 32, 8), _kv_need(2, 16), _kv_need(1, 32, 8), _kv_need(2, 16)]
+    model = _fake_model(needs)
     rt = Runtime(torch.device("cpu"), torch.float32)
     page = 4
-    per_page = 2 * 4 * page * (3 * 2 * 16 + 2 * 1 * 32)          # keys and values, float32
-    st = CacheStorage(rt, model, page, None, 4, 64, kv_bytes=10 * per_page + per_page // 2)
-    assert st.num_pages == 10 and st.kv_bytes == 10 * per_page
-    assert [p.num_pages for p in st.manager.pools] == [10, 10]
-    held = sum(t.numel() * t.element_size() for t in st.k + st.v)
-    assert held == st.kv_bytes <= 10 * per_page + per_page // 2
-    assert st.page_bytes == [2 * 4 * page * 3 * 2 * 16, 2 * 4 * page * 2 * 1 * 32]
+    whole_page = 2 * 4 * page * 3 * 2 * 16          # keys and values, float32, three layers
+    window_page = 2 * 4 * page * 2 * 1 * 32         # two layers
+    # 4 requests, portions of 8 tokens: a request holds (8 + 8) / 4 + 1 = 5 pages of the windowed group at most, and
+    # the scheduler keeps one more free for each: 24 pages, however large the budget
+    budget = 24 * window_page + 10 * whole_page + whole_page // 2
+    st = CacheStorage(rt, model, page, None, 4, 64, kv_bytes=budget, max_portion=8)
+    assert st.page_bytes == [whole_page, window_page]
+    assert [p.num_pages for p in st.manager.pools] == [10, 24] and st.num_pages == 10
+    assert st.kv_bytes == 24 * window_page + 10 * whole_page <= budget
+    held = sum(t.numel() * t.element_size() for g in st.pages for t in g.values())
+    assert held == st.kv_bytes
+    assert st.pages[0]["k"].shape == (3, 10, 2, page, 16) and st.pages[0]["v"].shape == (3, 10, 2, 16, page)
+    assert st.pages[1]["k"].shape == (2, 24, 1, page, 32)
+    assert st.manager.max_held_pages(1, 8) == 5 and st.manager.max_held_pages(0, 8) == 16
+    # ten times the budget: the windowed group stays, the other takes everything
+    big = CacheStorage(rt, model, page, None, 4, 64, kv_bytes=24 * window_page + 100 * whole_page, max_portion=8)
+    assert [p.num_pages for p in big.manager.pools] == [100, 24]
+    # as it was before the groups were sized by need, every group would have had budget // (both pages) = the same
+    assert budget // (whole_page + window_page) < 24
+    # whole sequences in one step (no portion given): the windowed group's requests may hold a whole sequence
+    assert CacheStorage(rt, model, page, None, 4, 64, kv_bytes=budget * 4).manager.pools[1].num_pages == 4 * 17
     with pytest.raises(ValueError, match="does not hold one page"):
-        CacheStorage(rt, model, page, None, 4, 64, kv_bytes=per_page - 1)
+        CacheStorage(rt, model, page, None, 4, 64, kv_bytes=whole_page - 1, max_portion=8)
     with pytest.raises(ValueError, match="not both"):
-        CacheStorage(rt, model, page, 64, 4, 64, kv_bytes=per_page)
-    # the same pool given in tokens
-    assert CacheStorage(rt, model, page, 40, 4, 64).num_pages == 10
+        CacheStorage(rt, model, page, 64, 4, 64, kv_bytes=budget)
+    # the same pool given in tokens: every group holds that many
+    assert [p.num_pages for p in CacheStorage(rt, model, page, 40, 4, 64).manager.pools] == [10, 10]
+
+
+def test_what_a_page_holds_is_what_the_mixers_declare():
+    """The storage allocates the tensors that a mixer's CacheNeed lists and nothing else: one latent vector per token
+    in a dtype of its own, beside keys and values of another shape; layers whose needs are equal share a group."""
+    import torch
+
+    from vt_transformer_amd.cache.storage import CacheStorage
+    from vt_transformer_amd.parts.base import CacheNeed, PageTensor, Runtime
+
+    latent = CacheNeed((PageTensor("latent", (24,), 0, torch.float32),), page_multiple=1)
+    needs = [_kv_need(2, 16), latent, _kv_need(2, 16), latent, None]
+    st = CacheStorage(Runtime(torch.device("cpu"), torch.bfloat16), _fake_model(needs), 8, 64, 2, 64)
+    assert st.n_groups == 2 and st.entry_group == [0, 1, 0, 1, None] and st.entry_index == [0, 0, 1, 1, None]
+    assert set(st.pages[0]) == {"k", "v"} and set(st.pages[1]) == {"latent"}
+    assert st.pages[1]["latent"].shape == (2, 8, 8, 24) and st.pages[1]["latent"].dtype == torch.float32
+    assert st.pages[0]["k"].dtype == torch.bfloat16
+    assert st.page_bytes == [2 * 2 * 8 * 2 * 2 * 16, 2 * 8 * 24 * 4]
+    caches = st.layer_caches([torch.zeros(1, 8, dtype=torch.int32)] * 2)
+    assert caches[4] is None and caches[3]["latent"].shape == (8, 8, 24) and caches[2]["v"].shape == (8, 2, 16, 8)
+    # an entry that reads another's pages must lay them out alike
+    import pytest
+    from types import SimpleNamespace
+    from vt_transformer_amd.config.base import ScheduleEntry
+    m = _fake_model([_kv_need(2, 16), latent])
+    m.schedule = [ScheduleEntry(0), ScheduleEntry(1, cache_from=0)]
+    with pytest.raises(ValueError, match="pages differ"):
+        CacheStorage(Runtime(torch.device("cpu"), torch.float32), m, 8, 64, 2, 64)
+
+
+def test_pages_a_request_will_hold_on_its_way_through_a_window():
+    m = manager(num_pages=64, page_size=4, windows=(0, 8), max_seq_len=256)
+    rp = m.admit("a")
+    # in one step of 40 tokens both groups need all ten pages; on the way there in portions of 8 the windowed group
+    # never holds more than (8 + 8) / 4 + 1 = 5
+    assert m.pages_needed(rp, 40) == [10, 10]
+    assert m.pages_needed(rp, 40, portion=8) == [10, 5]
+    assert m.reserve([("a", 8)])
+    m.commit("a", 8)
+    assert m.pages_needed(rp, 40, portion=8) == [8, 3]        # it holds two of the five already
+    for n in range(16, 41, 8):
+        assert m.reserve([("a", n)])
+        m.commit("a", n)
+        assert sum(1 for p in rp.tables[1] if p >= 0) <= 5
+    m.check()

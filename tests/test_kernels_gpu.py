@@ -708,20 +708,22 @@ def test_random_normal_kernel_makes_the_hosts_bits(dtype, n, first):
 @pytest.mark.parametrize("h,k1,m2,gated", [(3584, 3584, 4608, False), (3584, 18944, 1184, True), (200, 96, 320, False),
                                            (1536, 8960, 2048, False), (8192, 512, 640, True), (72, 40, 56, True),
                                            (3584, 18944, 10240, False)])
-def test_rmsnorm_handed_from_one_product_to_the_next(n, h, k1, m2, gated):
+@pytest.mark.parametrize("lp", [torch.bfloat16, torch.float16])
+def test_rmsnorm_handed_from_one_product_to_the_next(n, h, k1, m2, gated, lp):
     """A product that adds to the residual stream prepares the norm behind it (the stream times the gains in
     bfloat16, its blocks' shares of the rows' sums of squares); the product behind the norm takes those as its
     tokens and divides by the root.  Against the plain chain: add, RMSNorm, product.  Up to 16 rows a block per tile
     row produces; from 17 to 64 the kernel that keeps k inside a block, or the launch that adds the partial sums of a
-    split k."""
+    split k.  (Both 16-bit builds carry the kernels; the parts use them in bfloat16 only, because float16's range does
+    not hold an un-normalised stream times gains: parts/linear.py, norm_inside_products.)"""
     o = ops()
     g = torch.Generator().manual_seed(n * 1000 + h)
-    x = (torch.randn(n, k1, generator=g) * 0.5).to(torch.bfloat16)
-    w1 = (torch.randn(h, k1, generator=g) * 0.05).to(torch.bfloat16)
+    x = (torch.randn(n, k1, generator=g) * 0.5).to(lp)
+    w1 = (torch.randn(h, k1, generator=g) * 0.05).to(lp)
     bias1 = torch.randn(h, generator=g) * 0.1
     resid = torch.randn(n, h, generator=g)
     gain = 1.0 + 0.1 * torch.randn(h, generator=g)
-    w2 = (torch.randn((2 if gated else 1) * m2, h, generator=g) * 0.05).to(torch.bfloat16)
+    w2 = (torch.randn((2 if gated else 1) * m2, h, generator=g) * 0.05).to(lp)
     eps = 1e-5
     shares, stride = o.linear_bf16_link_shares(n, h, k1), o.link_stride(n)
     assert shares > 0 and o.linear_bf16_adds_residual(n, h, k1)
@@ -730,7 +732,7 @@ def test_rmsnorm_handed_from_one_product_to_the_next(n, h, k1, m2, gated):
         need = o.linear_bf16_workspace(rows, m, k) if rows > 16 else 0
         return torch.full((need,), float("nan"), device=DEV) if need else None
     hbuf = resid.clone().to(DEV)
-    xn = torch.full((n, h), float("nan"), dtype=torch.bfloat16, device=DEV)
+    xn = torch.full((n, h), float("nan"), dtype=lp, device=DEV)
     ssq = torch.full((shares, stride), float("nan"), dtype=torch.float32, device=DEV)
     o.linear_bf16_link(x.to(DEV), o.pack_matrix_bf16(w1.to(DEV)), bias1.to(DEV), hbuf, residual=hbuf, xn_out=xn,
                        gain_next=gain.to(DEV), ssq_out=ssq, workspace=workspace(n, h, k1))
@@ -739,8 +741,8 @@ def test_rmsnorm_handed_from_one_product_to_the_next(n, h, k1, m2, gated):
     assert rel_err(ssq[:, :n].sum(dim=0), (h_ref * h_ref).sum(dim=1)) < 1e-5
     assert bool((ssq[:, n:] == 0).all())
     # what the consumer reads: exactly bf16(h * gain) of the stream as the producer left it
-    assert torch.equal(xn.cpu(), (hbuf.cpu() * gain).to(torch.bfloat16))
-    normed = bf16_round(hbuf.cpu() * gain) / torch.sqrt((h_ref * h_ref).mean(dim=1, keepdim=True) + eps)
+    assert torch.equal(xn.cpu(), (hbuf.cpu() * gain).to(lp))
+    normed = (hbuf.cpu() * gain).to(lp).double() / torch.sqrt((h_ref * h_ref).mean(dim=1, keepdim=True) + eps)
     if gated:
         out = torch.empty(n, m2, dtype=torch.float32, device=DEV)
         o.gated_linear_bf16_link(xn, o.pack_matrix_bf16(w2.to(DEV), halves=2), out, ssq, eps)

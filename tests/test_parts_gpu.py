@@ -193,7 +193,7 @@ def test_run_order_is_data(dtype):
     model.load(w.__getitem__)
     runner = make_runner(model, pool_tokens=128, page_size=16, max_requests=2, max_seq_len=128)
     # three entries keep pages (0, 1, 2), two read another's: one group of three layers' worth of pages
-    assert runner.storage.k[0].shape[0] == 3 and runner.storage.writes == [True, True, True, False, False]
+    assert runner.storage.pages[0]["k"].shape[0] == 3 and runner.storage.writes == [True, True, True, False, False]
     ids = np.random.RandomState(0).randint(0, TINY_A["vocab_size"], size=41).tolist()
     runner.admit("r")
     got = []
@@ -265,6 +265,48 @@ def register_toy_parts():
                 state[slot] = s
             return out.to(x.dtype)
 
+    @MIXERS.register("toy_latent")
+    class ToyLatent(Part):
+        """Attention over one latent vector per token: c_t = x_t Wd^T is what the pages keep (one tensor, float32
+        whatever the runtime's dtype, [slot][rank]); y_t = softmax_s<=t(q_t . c_s / sqrt(rank)) c_s Wu^T with
+        q_t = x_t Wq^T.  The page's layout is this mixer's own: the cache manager allocates what cache_need() lists."""
+
+        def __init__(self, *, rt, width, prefix, rank, shared=None):
+            self.rt, self.width, self.rank, self.prefix = rt, width, int(rank), prefix
+
+        def cache_need(self):
+            from vt_transformer_amd.parts import CacheNeed, PageTensor
+            return CacheNeed((PageTensor("latent", (self.rank,), 0, torch.float32),))
+
+        def state_need(self):
+            return None
+
+        def tensors(self):
+            return {self.prefix + "down.weight": TensorDecl((self.rank, self.width), "matrix"),
+                    self.prefix + "q.weight": TensorDecl((self.rank, self.width), "matrix"),
+                    self.prefix + "up.weight": TensorDecl((self.width, self.rank), "matrix")}
+
+        def load(self, get, rt):
+            self.wd, self.wq, self.wu = (rt.place(get(self.prefix + n + ".weight"), "matrix").float() for n in ("down", "q", "up"))
+
+        def forward(self, x, ctx, cache, state):
+            pages = cache["latent"]                              # [pages][slot][rank]
+            ps = pages.shape[1]
+            xf = x.float()
+            c, q = xf @ self.wd.t(), xf @ self.wq.t()
+            pos, ent = ctx.positions.long(), ctx.tok_entry.long()
+            page = cache.block_table[ent, pos // ps].long()
+            pages[page, pos % ps] = c                            # this step's tokens into their slots
+            out = torch.empty(x.shape[0], self.width, dtype=torch.float32, device=x.device)
+            for e in range(ctx.n_entries):
+                t0, t1, p0 = int(ctx.h_entry_start[e]), int(ctx.h_entry_start[e + 1]), int(ctx.h_entry_pos0[e])
+                n_keys = p0 + (t1 - t0)
+                lat = pages[cache.block_table[e, :-(-n_keys // ps)].long()].reshape(-1, self.rank)[:n_keys]
+                sc = (q[t0:t1] @ lat.t()) / math.sqrt(self.rank)
+                seen = torch.arange(n_keys, device=x.device)[None, :] <= (p0 + torch.arange(t1 - t0, device=x.device))[:, None]
+                out[t0:t1] = (torch.softmax(sc.masked_fill(~seen, float("-inf")), dim=-1) @ lat) @ self.wu.t()
+            return out.to(x.dtype)
+
     @POSITIONS.register("toy_offset")
     class ToyOffset(Part):
         """Not a rotation: adds position * slope to the first dim of queries and keys."""
@@ -319,6 +361,61 @@ class ToyConfig(ModelConfig):
                          PartSpec("linear_head", {"name": "emb.weight", "tied_to": "emb.weight"}), 256)
 
 
+class ToyLatentConfig(ModelConfig):
+    """Layers that keep one latent vector per token beside layers of grouped-query attention: two groups of pages
+    with different contents."""
+    architecture = "ToyLatentForCausalLM"
+
+    def __init__(self, d):
+        self.d = d
+
+    @classmethod
+    def from_dict(cls, d):
+        return cls(d)
+
+    def to_dict(self):
+        return dict(self.d)
+
+    def to_spec(self):
+        d = self.d
+        norm = lambda name: PartSpec("rmsnorm", {"eps": d["eps"], "name": name})
+        layers = []
+        for i in range(d["n_layer"]):
+            if i % 2 == 0:
+                mixer = PartSpec("toy_latent", {"rank": d["rank"], "prefix": "lat."})
+            else:
+                mixer = PartSpec("attention", {"num_heads": 2, "num_kv_heads": 1, "head_dim": 16, "prefix": "attn."})
+            layers.append(LayerSpec(PartSpec("prenorm", {}), mixer,
+                                    PartSpec("gated_mlp", {"intermediate_size": d["inter"], "prefix": "ffn."}),
+                                    {"input": norm("n1.weight"), "post_mixer": norm("n2.weight")}, f"blocks.{i}."))
+        return ModelSpec("ToyLatentForCausalLM", d["vocab"], d["width"], PartSpec("embedding", {"name": "emb.weight"}),
+                         layers, [ScheduleEntry(i) for i in range(d["n_layer"])], norm("final.weight"),
+                         PartSpec("linear_head", {"name": "emb.weight", "tied_to": "emb.weight"}), 256)
+
+
+def toy_latent_plain(d, w, ids):
+    """The latent toy model whole, float64."""
+    t = len(ids)
+    x = w["emb.weight"][torch.tensor(ids)]
+    causal = torch.tril(torch.ones(t, t, dtype=torch.bool))
+    for i in range(d["n_layer"]):
+        p = f"blocks.{i}."
+        a = pm.rmsnorm(x, w[p + "n1.weight"], d["eps"])
+        if i % 2 == 0:
+            c, q = a @ w[p + "lat.down.weight"].t(), a @ w[p + "lat.q.weight"].t()
+            sc = (q @ c.t() / math.sqrt(d["rank"])).masked_fill(~causal, float("-inf"))
+            y = (torch.softmax(sc, dim=-1) @ c) @ w[p + "lat.up.weight"].t()
+        else:
+            q = pm.linear(a, w[p + "attn.q_proj.weight"]).reshape(t, 2, 16)
+            k = pm.linear(a, w[p + "attn.k_proj.weight"]).reshape(t, 1, 16)
+            v = pm.linear(a, w[p + "attn.v_proj.weight"]).reshape(t, 1, 16)
+            y = pm.linear(pm.attention(q, k, v).reshape(t, 32), w[p + "attn.o_proj.weight"])
+        x = x + y
+        b = pm.rmsnorm(x, w[p + "n2.weight"], d["eps"])
+        x = x + pm.swiglu(b, w[p + "ffn.gate_proj.weight"], w[p + "ffn.up_proj.weight"], w[p + "ffn.down_proj.weight"])
+    return pm.rmsnorm(x, w["final.weight"], d["eps"]) @ w["emb.weight"].t()
+
+
 def toy_plain(d, w, ids):
     """The toy model whole, float64."""
     t = len(ids)
@@ -371,7 +468,7 @@ def test_toy_mixer_with_state_toy_position_encoding_and_toy_routing():
     runner = make_runner(model, pool_tokens=128, page_size=16, max_requests=2, max_seq_len=128)
     assert [s is not None for s in runner.storage.state] == [True, False, True, False]    # state slots for the toy
     assert runner.storage.state[0].shape == (2, 48)
-    assert runner.storage.n_groups == 1 and runner.storage.k[0].shape[0] == 2               # pages for attention only
+    assert runner.storage.n_groups == 1 and runner.storage.pages[0]["k"].shape[0] == 2               # pages for attention only
     wd = {n: t.double() for n, t in w.items()}
     rs = np.random.RandomState(1)
     a, b, c = (rs.randint(0, 90, size=n).tolist() for n in (30, 21, 12))
@@ -389,6 +486,33 @@ def test_toy_mixer_with_state_toy_position_encoding_and_toy_routing():
     got_c = runner.step([StepEntry("c", c, list(range(12)))]).cpu()
     assert rel(got_c, rc) < 2e-5
     assert not runner._stateless and not runner._replayable     # such a model is never replayed from a captured graph
+
+
+def test_the_toy_architecture_through_the_engine_with_preemption():
+    """The mixer with state of its own through Engine.generate (scheduler, sampler, no captured steps and no decoding
+    ahead, since its steps cannot be replayed), with three pages for two requests: the younger one is preempted when
+    both need a second page, gives its state slot back, and is recomputed later from its prompt and what it had
+    produced, into a slot that starts from zero again.  Both end with the tokens they get alone."""
+    from vt_transformer_amd.config import config_from_dict, register_architecture
+    from vt_transformer_amd.engine import Engine
+    from vt_transformer_amd.sampling import SamplingParams
+    register_toy_parts()
+    register_architecture("ToyStateForCausalLM", ToyConfig)
+    d = {"architectures": ["ToyStateForCausalLM"], "n_layer": 4, "width": 48, "inter": 64, "vocab": 90, "eps": 1e-6,
+         "decay": 0.9, "slope": 0.01, "experts": 3}
+    rs = np.random.RandomState(4)
+    prompts = [rs.randint(0, 90, size=n).tolist() for n in (10, 9)]
+    sp = SamplingParams(max_tokens=14, ignore_eos=True)
+    eng = Engine(config=config_from_dict(d), random_weights_seed=5, dtype="float32", num_pages=3, max_running_reqs=2,
+                 max_seq_len=64)
+    assert not eng.runner.replays(2)
+    outs = eng.generate(prompts, sp)
+    assert [eng.finish_reason(i) for i in (0, 1)] == ["max_tokens"] * 2
+    assert eng.requests[1].preemptions > 0 and eng.requests[0].preemptions == 0
+    assert sum(eng.runner.cache.held_pages()) == 0 and eng.runner.cache.slots.available == 2
+    alone = Engine(config=config_from_dict(d), random_weights_seed=5, dtype="float32", num_pages=4, max_running_reqs=1,
+                   max_seq_len=64)
+    assert outs == [alone.generate(p, sp)[0] for p in prompts]
 
 
 def test_a_plugin_file_brings_an_architecture_to_the_replay_program(tmp_path):
@@ -428,3 +552,59 @@ def test_a_plugin_file_brings_an_architecture_to_the_replay_program(tmp_path):
                 assert rel(torch.from_numpy(got[s["step"]][row].copy()), want) < 2e-5, (s["step"], e["id"], j)
                 row += 1
             pos[e["id"]] += len(e["tokens"])
+
+
+def test_a_mixer_that_keeps_one_latent_vector_per_token_in_pages_of_its_own(tmp_path):
+    """What a page holds is the mixer's own affair: a mixer defined here keeps one float32 vector per token,
+    [slot][rank], beside attention layers that keep keys and values of another shape in the runtime's dtype.  Written
+    as a model folder and replayed by bin/trace_run in mixed steps with so few pages that they are used again, with
+    nothing but a plugin file (no change under the package's cache or engine folders); and in-process in bfloat16."""
+    import os
+    from replay_helpers import cut, max_live_tokens, random_requests, run_in_process, run_trace_run, trace_mixed
+    from vt_transformer_amd.config import config_from_dict, register_architecture
+    from vt_transformer_amd.engine import load_model, make_runner
+    from vt_transformer_amd.weights import write_random_model
+    register_toy_parts()
+    register_architecture("ToyLatentForCausalLM", ToyLatentConfig)
+    d = {"architectures": ["ToyLatentForCausalLM"], "n_layer": 4, "width": 48, "inter": 64, "vocab": 90, "eps": 1e-6,
+         "rank": 24}
+    folder = write_random_model(config_from_dict(d), str(tmp_path / "toy"), seed=9, dtype=torch.float32)
+    # larger projections, so that the scores differ and a latent vector read from a wrong slot would show
+    from vt_transformer_amd.weights.safetensors_io import WeightStore, write_safetensors
+    store = WeightStore(folder)
+    tensors = [(n, store.get(n).float() * (8.0 if ".lat." in n or "_proj" in n else 1.0)) for n in store.names()]
+    store.close()
+    write_safetensors(os.path.join(folder, "model.safetensors"), tensors)
+    plugin = tmp_path / "toy_plugin.py"
+    plugin.write_text(
+        "import sys\n"
+        f"sys.path.insert(0, {os.path.dirname(os.path.abspath(__file__))!r})\n"
+        "import test_parts_gpu as toy\n"
+        "from vt_transformer_amd.config import register_architecture\n"
+        "toy.register_toy_parts()\n"
+        "register_architecture('ToyLatentForCausalLM', toy.ToyLatentConfig)\n")
+    reqs = random_requests(d["vocab"], [23, 9, 31, 14, 18, 40], seed=5)
+    portions = {r: cut(t, [5, 2, 7, 1]) for r, t in reqs.items()}
+    steps = trace_mixed(reqs, portions, max_live=3, seed=6)
+    _, w = pm.read_folder(folder)
+    ref = {r: toy_latent_plain(d, w, t) for r, t in reqs.items()}
+
+    def check(got, tol):
+        pos = {r: 0 for r in reqs}
+        for s in steps:
+            row = 0
+            for e in s["entries"]:
+                for j in e["want"]:
+                    want = ref[e["id"]][pos[e["id"]] + j]
+                    assert rel(torch.from_numpy(got[s["step"]][row].copy()), want) < tol, (s["step"], e["id"], j)
+                    row += 1
+                pos[e["id"]] += len(e["tokens"])
+    check(run_trace_run(folder, "float32", steps, str(tmp_path / "out"), max_live_tokens(steps), d["vocab"],
+                        extra_args=("--plugin", str(plugin))), 2e-5)
+    model = load_model(folder, "bfloat16")
+    runner = make_runner(model, pool_tokens=max_live_tokens(steps), page_size=16, max_requests=3, max_seq_len=128)
+    assert runner.storage.n_groups == 2
+    assert set(runner.storage.pages[0]) == {"latent"} and runner.storage.pages[0]["latent"].dtype == torch.float32
+    assert runner.storage.pages[0]["latent"].shape[2:] == (16, 24) and set(runner.storage.pages[1]) == {"k", "v"}
+    check(run_in_process(runner, steps), 3e-2)
+    assert sum(runner.cache.held_pages()) == 0

@@ -88,6 +88,15 @@ def check_configuration(cfg, seed, tmp_path):
     print(f"random configuration {seed}: worst relative error {worst}")
 
 
+def size_tolerance(dtype: str, width: int) -> float:
+    """The comparisons with the plain model at real layer sizes, relative to a row's largest logit.  The rounding of a
+    16-bit model grows with the length of its sums: measured 9.2e-3, 1.2e-2 and 1.9e-2 in bfloat16 at widths 1,536, 3,584
+    and 8,192 (float16: an eighth of that, three more bits; float32: 3.5e-6 to 1.2e-5), about the square root of the
+    width.  Twice what was measured at the largest width, following the root of the width."""
+    per_root = {"bfloat16": 4.2e-4, "float16": 5.0e-5, "float32": 2.6e-7}[dtype]
+    return per_root * width ** 0.5
+
+
 @pytest.mark.parametrize("name,hidden,heads,kv,inter", [("7B", 3584, 28, 4, 18944), ("1.5B", 1536, 12, 2, 8960),
                                                         ("72B", 8192, 64, 8, 29568)])
 def test_real_layer_sizes(name, hidden, heads, kv, inter, tmp_path):
@@ -109,7 +118,8 @@ def test_real_layer_sizes(name, hidden, heads, kv, inter, tmp_path):
     toks = np.random.RandomState(0).randint(0, 4099, size=n).tolist()
     ref = plain_model.forward(pcfg, w, toks)
     scale = ref.abs().max()
-    for dtype, tol in (("bfloat16", 2e-2), ("float16", 3e-3), ("float32", 3e-5)):
+    for dtype in ("bfloat16", "float16", "float32"):
+        tol = size_tolerance(dtype, hidden)
         model = load_model(folder, dtype)
         for mode in ("whole", "cut", "decode", "graph", "batch"):
             runner = make_runner(model, pool_tokens=10240, page_size=16, max_requests=48, max_seq_len=512)
@@ -190,3 +200,56 @@ def test_many_requests_decoding_side_by_side_at_7b_layer_sizes(n_req, tmp_path):
         assert bool(runner._graphs) == graphs          # (a captured step takes up to 192 entries)
         print(f"{n_req} decoding requests {dtype}{' captured' if graphs else ''}: worst relative error {worst:.3e}")
         del model, runner
+
+
+@pytest.mark.parametrize("tied", [False, True])
+@pytest.mark.parametrize("name,hidden,heads,kv,inter", [("7B", 3584, 28, 4, 18944), ("72B", 8192, 64, 8, 29568)])
+def test_the_whole_vocabulary(name, hidden, heads, kv, inter, tied):
+    """One layer at Qwen2-7B and 72B widths under the real vocabulary of 152,064 (9,504 tile rows of the head; at
+    width 8,192 its matrix has 1.25 G elements, beyond 32-bit byte offsets), tied and untied: the logits of a
+    40-token portion (the 17-to-64-row kernels) and of 3 tokens decoded one by one (the few-row kernels), and the
+    embedding's rows of the first and the last token id (the reference's head and lookup:
+    v1/tensortype/hip_tensor.cpp:923-991, v1/tensortype/hip_kernels/embed.cpp:7-37), against float64, in the three
+    dtypes.  The tensors are drawn on the device and the plain model runs there in float64: on the host the head
+    alone would be 10 GB."""
+    from vt_transformer_amd.config import config_from_dict
+    from vt_transformer_amd.engine import StepEntry, build_model, make_runner
+    V = 152064
+    cfg = dict(architectures=["Qwen2ForCausalLM"], model_type="qwen2", vocab_size=V, hidden_size=hidden,
+               intermediate_size=inter, num_hidden_layers=1, num_attention_heads=heads, num_key_value_heads=kv, head_dim=128,
+               rope_theta=1e6, rms_norm_eps=1e-6, tie_word_embeddings=tied, max_position_embeddings=8192,
+               hidden_act="silu", use_sliding_window=False, torch_dtype="bfloat16")
+    config = config_from_dict(cfg)
+    gen = torch.Generator(device="cuda").manual_seed(hidden + tied)
+    expected = build_model(config, "float32").tensors()
+    w16 = {}
+    for tname, decl in expected.items():
+        if decl.optional:
+            continue
+        t = torch.randn(decl.shape, generator=gen, device="cuda") * 0.02
+        if decl.role == "gain":
+            t += 1.0
+        w16[tname] = t.to(torch.bfloat16)
+    toks = [0, V - 1] + np.random.RandomState(hidden).randint(0, V, size=41).tolist()
+    ref = plain_model.forward(cfg, {k: v.double() for k, v in w16.items()}, toks)          # [43, V] float64, on the host
+    torch.cuda.empty_cache()
+    for dtype in ("bfloat16", "float16", "float32"):
+        model = build_model(config, dtype)
+        model.load(w16.__getitem__)
+        rows = model.embedding.forward(torch.tensor([0, V - 1], dtype=torch.int32, device="cuda"))
+        table = w16["model.embed_tokens.weight"]
+        assert torch.equal(rows.cpu(), table[[0, V - 1]].float().cpu()), (name, dtype, "embedding rows")
+        runner = make_runner(model, pool_tokens=64, page_size=16, max_requests=2, max_seq_len=64)
+        runner.admit("r")
+        got = [runner.step([StepEntry("r", toks[:40], list(range(40)))]).float().cpu()]
+        got += [runner.step([StepEntry("r", toks[i:i + 1], [0])]).float().cpu() for i in (40, 41, 42)]
+        got = torch.cat(got).double()
+        assert got.shape == (43, V)
+        err = float(((got - ref).abs().max(dim=1).values / ref.abs().max(dim=1).values).max())
+        print(f"whole vocabulary {name} tied={tied} {dtype}: relative error {err:.3e}")
+        assert err < size_tolerance(dtype, hidden), (name, tied, dtype, err)
+        # the head's far end alone: the last tile row of the matrix against the same rows of the reference
+        tail = float((got[:, V - 16:] - ref[:, V - 16:]).abs().max() / ref.abs().max())
+        assert tail < size_tolerance(dtype, hidden), (name, tied, dtype, "last tile row", tail)
+        del model, runner
+        torch.cuda.empty_cache()

@@ -15,9 +15,10 @@ EOS = 7
 class FakeEngine:
     """Scheduler + cache manager + a step that only does the bookkeeping of the real step function."""
 
-    def __init__(self, num_pages=64, page_size=4, windows=(0,), token=lambda req: 1, **cfg):
+    def __init__(self, num_pages=64, page_size=4, windows=(0,), token=lambda req: 1, group_pages=None, **cfg):
         self.cfg = SchedulerConfig(num_pages=num_pages, page_size=page_size, **cfg)
-        self.cache = CacheManager([GroupSpec(i, w, num_pages) for i, w in enumerate(windows)], page_size,
+        group_pages = group_pages or [num_pages] * len(windows)
+        self.cache = CacheManager([GroupSpec(i, w, n) for i, (w, n) in enumerate(zip(windows, group_pages))], page_size,
                                   self.cfg.max_running_reqs, self.cfg.max_seq_len)
         self.sched = Scheduler(self.cfg, self.cache, [EOS])
         self.token = token
@@ -403,3 +404,23 @@ def test_random_loads_do_decode_ahead():
         e.run()
         launched += e.launched_ahead
     assert launched > 100
+
+
+def test_a_windowed_group_with_few_pages_does_not_bound_a_requests_length():
+    """Layers with a window hold a window and a portion of a request, so their pool may be far smaller than a
+    prompt: 12 pages of 4 tokens beside prompts of 40 (ten pages in the group that keeps every key).  Nobody is
+    refused as too long, both slots are used, everybody finishes."""
+    e = FakeEngine(page_size=4, windows=(0, 6), group_pages=[64, 12], max_running_reqs=2, chunk_size=8,
+                   max_extend_tokens=16, max_seq_len=128)
+    assert e.cache.max_held_pages(1, 8) == 5
+    reqs = [e.add(i, 40, max_tokens=6) for i in range(3)]
+    e.step()
+    assert len(e.sched.running) == 2
+    e.run(limit=300)
+    assert [r.finish_reason for r in reqs] == ["max_tokens"] * 3 and all(len(r.output) == 6 for r in reqs)
+    assert e.cache.held_pages() == [0, 0]
+    # with fewer pages than a window and a portion take, the windowed group bounds the length like any other
+    small = FakeEngine(page_size=4, windows=(0, 6), group_pages=[64, 4], chunk_size=8, max_seq_len=128)
+    r = small.add("x", 40)
+    small.run()
+    assert r.finish_reason == "too_long"

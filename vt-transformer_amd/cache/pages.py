@@ -158,8 +158,22 @@ class CacheManager:
             return 0
         return max(0, (length - w + 1)) // self.page_size
 
-    def pages_needed(self, rp: RequestPages, new_len: int) -> List[int]:
-        """Per group, how many pages `reserve` would have to take for the request to hold new_len tokens."""
+    def max_held_pages(self, gi: int, portion: int) -> int:
+        """The most pages of group gi that one request can hold at a time when no step brings more than `portion`
+        of its tokens: every page for a group that keeps all keys; for a group with a window, the pages of the
+        window and of one portion (and one more: neither needs to start at a page's edge)."""
+        ps = self.page_size
+        whole = -(-self.max_seq_len // ps)
+        w = self.groups[gi].window
+        if w <= 0:
+            return whole
+        return min(whole, -(-(w + max(1, int(portion))) // ps) + 1)
+
+    def pages_needed(self, rp: RequestPages, new_len: int, portion: Optional[int] = None) -> List[int]:
+        """Per group, how many pages `reserve` would have to take for the request to hold new_len tokens after
+        one step.  With `portion` (the most tokens that a step brings): how many more pages the request will ever
+        hold at a time on its way to new_len in steps of at most that many tokens, which for a group with a window
+        is bounded by the window (`max_held_pages`), since `commit` gives back what the window has passed."""
         ps = self.page_size
         out = []
         for gi, table in enumerate(rp.tables):
@@ -169,6 +183,9 @@ class CacheManager:
             for b in range(first, last):
                 if b >= len(table) or table[b] == NO_PAGE:
                     n += 1
+            if portion is not None and self.groups[gi].window > 0:
+                held = sum(1 for p in table if p != NO_PAGE)
+                n = min(n, max(0, self.max_held_pages(gi, portion) - held))
             out.append(n)
         return out
 

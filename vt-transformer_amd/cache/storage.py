@@ -1,12 +1,14 @@
-"""Device memory behind the cache manager: key and value pages per group of
-layers, and per-request state slots.
+"""Device memory behind the cache manager: the pages of every group of layers,
+and per-request state slots.
 
-Pages of a group: K [layer][page][kv head][slot][D], V [layer][page][kv head][D][slot]
-(the reference's newer engine keeps one pool indexed [slot][layer][K|V],
-vt-transformer/models/qwen3-0.6b/init.vt:86-117; here a page of one kv head is
-contiguous so that one read of it serves all query heads of its group).
-Pools start zeroed: a slot that was never written holds finite numbers, so a
-masked key can never bring a NaN into a weighted sum.
+What a page holds is the mixer's business: its `cache_need()` lists the page's
+tensors (`PageTensor`: name, shape per token, where the slot axis lies, dtype)
+and this file allocates, per group of layers with equal needs, one tensor
+[layer][page] + page shape for each of them and hands the mixer a dict by name.
+(The reference's newer engine keeps one pool indexed [slot][layer][K|V],
+vt-transformer/models/qwen3-0.6b/init.vt:86-117.)  Pools start zeroed: a slot
+that was never written holds finite numbers, so a masked key can never bring
+a NaN into a weighted sum.
 """
 from __future__ import annotations
 
@@ -23,21 +25,52 @@ from .pages import CacheManager, GroupSpec
 class LayerCache:
     """What a mixer sees of the cache in one step."""
 
-    k: Optional[torch.Tensor]            # [pages][kv heads][slot][D] of this schedule entry
-    v: Optional[torch.Tensor]            # [pages][kv heads][D][slot]
+    tensors: Dict[str, torch.Tensor]     # by the names of its CacheNeed: [pages] + page shape, of this schedule entry
     block_table: Optional[torch.Tensor]  # int32 [entries of the step][blocks], of the entry's group
     writes: bool                         # False: the pages are another entry's, only read here
     group: int
 
+    def __getitem__(self, name: str) -> torch.Tensor:
+        return self.tensors[name]
+
+
+def group_pages(needs: List[CacheNeed], page_bytes: List[int], page_size: int, max_requests: int, max_seq_len: int,
+                max_portion: int, kv_bytes: int) -> List[int]:
+    """Pages per group under a budget in bytes for all of them.  A group with a window never holds more of a
+    request than its window and one portion (CacheManager.max_held_pages), so it gets pages for that, for every
+    request that may run, and no more; what is left of the budget goes to the groups that keep every key, which all
+    hold the same tokens and so get the same number of pages: budget // (bytes of one page of each of them together),
+    as the reference sizes its one pool (vt-transformer/models/qwen3-0.6b/init.vt:109-113:
+    num_blocks = budget // (block_size * per_token_bytes))."""
+    whole = -(-max_seq_len // page_size)
+    pages = [0] * len(needs)
+    left = int(kv_bytes)
+    for g, need in enumerate(needs):
+        if need.window > 0:
+            # (what a request holds at most, and the page of head-room per running request that the scheduler keeps
+            # free when it admits another)
+            per_request = min(whole, -(-(need.window + max(1, max_portion)) // page_size) + 1) + 1
+            pages[g] = max(1, min(max_requests * per_request, left // max(1, page_bytes[g])))
+            left -= pages[g] * page_bytes[g]
+    unbounded = [g for g, need in enumerate(needs) if need.window <= 0]
+    if unbounded:
+        per_page = sum(page_bytes[g] for g in unbounded)
+        n = left // per_page if per_page else 1
+        if n < 1 and per_page:
+            raise ValueError(f"a cache of {kv_bytes} bytes does not hold one page of {page_size} tokens of every group "
+                             f"of layers ({per_page} bytes over {len(unbounded)} group(s) that keep every key, after "
+                             f"{kv_bytes - left} bytes for the groups with a window)")
+        for g in unbounded:
+            pages[g] = max(1, n)
+    return pages
+
 
 class CacheStorage:
     def __init__(self, rt: Runtime, model, page_size: int, pool_tokens: Optional[int], max_requests: int,
-                 max_seq_len: int, kv_bytes: Optional[int] = None):
+                 max_seq_len: int, kv_bytes: Optional[int] = None, max_portion: Optional[int] = None):
         """`pool_tokens`: how many tokens the pages of each group hold together.  Or `kv_bytes`: a budget in bytes
-        for all keys and values, shared by the groups: a token takes a slot of a page in every group, so every
-        group gets the same number of pages, budget // (bytes of one page of each group together), as the
-        reference sizes its one pool (vt-transformer/models/qwen3-0.6b/init.vt:109-113:
-        num_blocks = budget // (block_size * per_token_bytes))."""
+        for all pages, shared by the groups according to their needs (`group_pages`); `max_portion`: the most
+        tokens of one request that a step brings (the scheduler's chunk size; default: a whole sequence)."""
         self.rt = rt
         self.page_size = int(page_size)
         schedule = model.schedule
@@ -50,11 +83,12 @@ class CacheStorage:
             state_needs.append(mixer.state_need() if hasattr(mixer, "state_need") else None)
             if e.cache_from is not None:
                 src = needs[e.cache_from]
-                if need is None or src is None or (need.kv_heads, need.head_dim) != (src.kv_heads, src.head_dim):
+                if need is None or src is None or not need.same_layout(src):
                     raise ValueError(f"schedule entry {i} cannot read the cache of entry {e.cache_from}: "
-                                     f"their key/value heads differ")
+                                     f"their pages differ")
         # groups of entries with their own cache and equal needs
         keys: List = []
+        self.group_needs: List[CacheNeed] = []
         self.entry_group: List[Optional[int]] = [None] * len(schedule)
         self.entry_index: List[Optional[int]] = [None] * len(schedule)
         members: Dict[int, int] = {}
@@ -64,6 +98,7 @@ class CacheStorage:
             k = needs[i].group_key()
             if k not in keys:
                 keys.append(k)
+                self.group_needs.append(needs[i])
             g = keys.index(k)
             self.entry_group[i] = g
             self.entry_index[i] = members.get(g, 0)
@@ -72,34 +107,26 @@ class CacheStorage:
             if e.cache_from is not None:
                 self.entry_group[i] = self.entry_group[e.cache_from]
                 self.entry_index[i] = self.entry_index[e.cache_from]
-        self.group_needs = [CacheNeed(*k) for k in keys]
-        elem = torch.empty((), dtype=rt.dtype).element_size()
-        # bytes of one page of every layer of a group: keys and values
-        self.page_bytes = [2 * members[g] * need.kv_heads * need.head_dim * self.page_size * elem
+        # bytes of one page of every layer of a group
+        self.page_bytes = [members[g] * need.bytes_per_token(rt.dtype) * self.page_size
                            for g, need in enumerate(self.group_needs)]
         if kv_bytes is not None:
             if pool_tokens is not None:
                 raise ValueError("give the cache's size in tokens or in bytes, not both")
-            per_page = sum(self.page_bytes)
-            num_pages = int(kv_bytes) // per_page if per_page else 1
-            if num_pages < 1 and per_page:
-                raise ValueError(f"a cache of {kv_bytes} bytes does not hold one page of {self.page_size} tokens "
-                                 f"({per_page} bytes over {len(keys)} group(s) of layers)")
-            num_pages = max(1, num_pages)
+            pages = group_pages(self.group_needs, self.page_bytes, self.page_size, max_requests, max_seq_len,
+                                max_portion or max_seq_len, int(kv_bytes))
         else:
             if pool_tokens is None:
                 raise ValueError("the cache needs a size: pool_tokens or kv_bytes")
-            num_pages = max(1, -(-int(pool_tokens) // self.page_size))
-        self.num_pages = num_pages
-        self.manager = CacheManager([GroupSpec(k, k[2], num_pages) for k in keys], self.page_size, max_requests,
-                                    max_seq_len)
-        self.k: List[torch.Tensor] = []
-        self.v: List[torch.Tensor] = []
+            pages = [max(1, -(-int(pool_tokens) // self.page_size))] * len(self.group_needs)
+        self.group_pages = pages
+        self.manager = CacheManager([GroupSpec(k, need.window, n) for k, need, n in zip(keys, self.group_needs, pages)],
+                                    self.page_size, max_requests, max_seq_len)
+        # per group and page tensor: [layer][page] + the tensor's page shape
+        self.pages: List[Dict[str, torch.Tensor]] = []
         for g, need in enumerate(self.group_needs):
-            shape_k = (members[g], num_pages, need.kv_heads, self.page_size, need.head_dim)
-            shape_v = (members[g], num_pages, need.kv_heads, need.head_dim, self.page_size)
-            self.k.append(torch.zeros(shape_k, dtype=rt.dtype, device=rt.device))
-            self.v.append(torch.zeros(shape_v, dtype=rt.dtype, device=rt.device))
+            self.pages.append({t.name: torch.zeros((members[g], pages[g]) + t.page_shape(self.page_size),
+                                                   dtype=t.dtype or rt.dtype, device=rt.device) for t in need.tensors})
         self.writes = [e.cache_from is None for e in schedule]
         # fixed-size state per request and schedule entry (none for attention)
         self.state: List[Optional[torch.Tensor]] = []
@@ -108,9 +135,18 @@ class CacheStorage:
                               torch.zeros((max_requests,) + tuple(need.shape), dtype=need.dtype, device=rt.device))
 
     @property
+    def num_pages(self) -> int:
+        """Pages of the groups that bound a request's length (those that keep every key); of the smallest group
+        if every group has a window."""
+        if not self.group_pages:
+            return 0
+        whole = [n for n, need in zip(self.group_pages, self.group_needs) if need.window <= 0]
+        return min(whole) if whole else min(self.group_pages)
+
+    @property
     def kv_bytes(self) -> int:
         """Bytes that the pages of all groups take."""
-        return self.num_pages * sum(self.page_bytes)
+        return sum(n * b for n, b in zip(self.group_pages, self.page_bytes))
 
     @property
     def n_groups(self) -> int:
@@ -127,7 +163,8 @@ class CacheStorage:
                 out.append(None)
             else:
                 idx = self.entry_index[i]
-                out.append(LayerCache(self.k[g][idx], self.v[g][idx], block_tables[g], self.writes[i], g))
+                out.append(LayerCache({name: t[idx] for name, t in self.pages[g].items()}, block_tables[g],
+                                      self.writes[i], g))
         return out
 
     def clear_state(self, slots: List[int]) -> None:

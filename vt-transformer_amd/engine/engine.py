@@ -53,7 +53,8 @@ class Engine:
         self.config = sc
         self.runner: ModelRunner = make_runner(
             self.model, pool_tokens=None if sc.kv_bytes is not None else sc.num_pages * sc.page_size,
-            kv_bytes=sc.kv_bytes, page_size=sc.page_size, max_requests=sc.max_running_reqs, max_seq_len=sc.max_seq_len)
+            kv_bytes=sc.kv_bytes, page_size=sc.page_size, max_requests=sc.max_running_reqs, max_seq_len=sc.max_seq_len,
+            max_portion=sc.chunk_size)
         sc.num_pages = self.runner.storage.num_pages
         self.runner.decode_graphs = bool(decode_graphs)
         self.scheduler = Scheduler(sc, self.runner.cache, spec.eos_token_ids)

@@ -76,13 +76,17 @@ def check_page_size(model: DecoderModel, page_size: int) -> None:
 
 
 def make_runner(model: DecoderModel, *, pool_tokens: Optional[int] = None, page_size: int = 16, max_requests: int = 64,
-                max_seq_len: Optional[int] = None, kv_bytes: Optional[int] = None) -> ModelRunner:
-    """The cache's size is `pool_tokens` (tokens that each group of layers holds) or `kv_bytes` (bytes for all keys
-    and values together, shared by the groups)."""
+                max_seq_len: Optional[int] = None, kv_bytes: Optional[int] = None,
+                max_portion: Optional[int] = None) -> ModelRunner:
+    """The cache's size is `pool_tokens` (tokens that each group of layers holds) or `kv_bytes` (bytes for all pages
+    together, shared by the groups by their needs: a group with a window gets pages for its window and `max_portion`
+    tokens, the most of one request that a step will bring, per request; the rest goes to the groups that keep
+    every key)."""
     check_page_size(model, page_size)
     if max_seq_len is None:
         if pool_tokens is None:
             max_seq_len = model.spec.max_positions
         else:
             max_seq_len = min(model.spec.max_positions, max(pool_tokens, page_size))
-    return ModelRunner(model, model.rt, page_size, pool_tokens, max_requests, max_seq_len, kv_bytes=kv_bytes)
+    return ModelRunner(model, model.rt, page_size, pool_tokens, max_requests, max_seq_len, kv_bytes=kv_bytes,
+                       max_portion=max_portion)

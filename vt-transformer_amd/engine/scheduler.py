@@ -141,15 +141,22 @@ class Scheduler:
 
     # -- one step's decisions ------------------------------------------------
     def _capacity_tokens(self) -> int:
-        if not self.cache.pools:
-            return self.config.max_seq_len
-        return min(p.num_pages for p in self.cache.pools) * self.cache.page_size
+        """The longest request that the pools can hold at all.  A group that keeps every key bounds it by its pages; a
+        group with a window holds a window and a portion of any request (CacheManager.max_held_pages) and bounds
+        nothing if it has the pages for that."""
+        limit = self.config.max_seq_len
+        for gi, (g, pool) in enumerate(zip(self.cache.groups, self.cache.pools)):
+            if g.window <= 0 or pool.num_pages < self.cache.max_held_pages(gi, self.config.chunk_size):
+                limit = min(limit, pool.num_pages * self.cache.page_size)
+        return limit
 
-    def _need(self, items: List[Tuple[Request, int]]) -> List[int]:
-        """Pages per group that these (request, new length) pairs would take together."""
+    def _need(self, items: List[Tuple[Request, int]], whole: bool = False) -> List[int]:
+        """Pages per group that these (request, new length) pairs would take together: in one step, or (whole) the
+        most that they will hold at a time on their way there in portions of at most chunk_size."""
         need = [0] * len(self.cache.pools)
+        portion = self.config.chunk_size if whole else None
         for r, new_len in items:
-            for gi, k in enumerate(self.cache.pages_needed(self.cache.get(r.uid), new_len)):
+            for gi, k in enumerate(self.cache.pages_needed(self.cache.get(r.uid), new_len, portion)):
                 need[gi] += k
         return need
 
@@ -248,7 +255,7 @@ class Scheduler:
         #    need to finish their prompts, so that requests admitted together can all reach decoding
         while self.waiting and budget > 0 and len(self.running) < cfg.max_running_reqs:
             r = self.waiting[0]
-            limit = min(cfg.max_seq_len, self._capacity_tokens())
+            limit = self._capacity_tokens()
             if r.total_len > limit:
                 self.waiting.popleft()
                 self._refuse(r, "too_long")
@@ -261,7 +268,7 @@ class Scheduler:
             reserve_pages = len(self.running)
             promised = [(q, max(new_len, q.total_len)) for q, new_len in planned]
             promised += [(q, q.total_len) for q in self.running if all(q is not p for p, _ in planned)]
-            need = self._need(promised + [(r, r.total_len)])
+            need = self._need(promised + [(r, r.total_len)], whole=True)
             ok = all(p.available - k >= reserve_pages for p, k in zip(self.cache.pools, need))
             if not ok:
                 self.cache.release(r.uid)

@@ -100,11 +100,12 @@ class ModelRunner:
     """Owns the model, its cache and the step function."""
 
     def __init__(self, model, rt: Runtime, page_size: int, pool_tokens: Optional[int], max_requests: int,
-                 max_seq_len: int, kv_bytes: Optional[int] = None):
+                 max_seq_len: int, kv_bytes: Optional[int] = None, max_portion: Optional[int] = None):
         self.model = model
         self.rt = rt
         self.max_seq_len = int(max_seq_len)
-        self.storage = CacheStorage(rt, model, page_size, pool_tokens, max_requests, max_seq_len, kv_bytes=kv_bytes)
+        self.storage = CacheStorage(rt, model, page_size, pool_tokens, max_requests, max_seq_len, kv_bytes=kv_bytes,
+                                    max_portion=max_portion)
         self.cache = self.storage.manager
         self.vocab_size = model.spec.vocab_size
         self.steps = 0
@@ -202,8 +203,10 @@ class ModelRunner:
         ctx.h_logit_rows, ctx.h_block_tables, ctx.fresh = rows, h["tables"], h["fresh"]
         ctx.h_kv_lens = h["kv_lens"]
         extras = self._prepare_parts(ctx)
+        # (the block tables last: a patched decoding step sends what lies in front of them, and of them only what changed)
+        ng, nx = len(h["tables"]), len(extras)
         parts = [ctx.h_token_ids, ctx.h_positions, ctx.h_tok_entry, ctx.h_entry_start, ctx.h_entry_pos0,
-                 ctx.h_state_slots, ctx.h_logit_rows] + [t.reshape(-1) for t in h["tables"]] + list(extras.values())
+                 ctx.h_state_slots, ctx.h_logit_rows] + list(extras.values()) + [t.reshape(-1) for t in h["tables"]]
         flat = np.concatenate(parts)
         if dev is None:
             dev = self.rt.buffer("step.meta", (flat.size,), torch.int32)
@@ -222,13 +225,13 @@ class ModelRunner:
          ctx.h_logit_rows) = hviews[:7]
         (ctx.token_ids, ctx.positions, ctx.tok_entry, ctx.entry_start, ctx.entry_pos0, ctx.state_slots,
          ctx.logit_rows) = views[:7]
-        ng = len(h["tables"])
-        ctx.h_block_tables = [v.reshape(h["n_entries"], h["max_blocks"]) for v in hviews[7:7 + ng]]
-        ctx.block_tables = [v.view(h["n_entries"], h["max_blocks"]) for v in views[7:7 + ng]]
+        ctx.h_block_tables = [v.reshape(h["n_entries"], h["max_blocks"]) for v in hviews[7 + nx:]]
+        ctx.block_tables = [v.view(h["n_entries"], h["max_blocks"]) for v in views[7 + nx:]]
         ctx.extra, ctx.extra_host = {}, {}
-        for key, v, hv, o in zip(extras, views[7 + ng:], hviews[7 + ng:], offs[7 + ng:]):
+        for key, v, hv in zip(extras, views[7:7 + nx], hviews[7:7 + nx]):
             ctx.extra[key], ctx.extra_host[key] = v, hv
-        ctx.offsets = dict(ids=offs[0], positions=offs[1], pos0=offs[4], tables=offs[7:7 + ng])
+        ctx.offsets = dict(ids=offs[0], positions=offs[1], pos0=offs[4], tables=offs[7 + nx:],
+                           lead=offs[7 + nx] if ng else flat.size)
         return dev
 
     def build_context(self, entries: Sequence[StepEntry]) -> StepContext:
@@ -352,6 +355,9 @@ class ModelRunner:
         for k, arr in new.items():
             old[k][:] = arr
         g.ctx.extra_host = old
+        # what goes to the device: everything in front of the block tables, and of the tables the entries that changed
+        # (a request takes a page every page_size steps; the tables are n entries x max_seq_len / page_size integers)
+        pieces = [(flat[:off["lead"]], g.meta[:off["lead"]])]
         mb = h["max_blocks"]
         for gi in range(self.storage.n_groups):
             base = off["tables"][gi]
@@ -359,12 +365,16 @@ class ModelRunner:
             windowed = self.storage.group_window(gi) > 0
             for i, rp in enumerate(rps):
                 t = rp.tables[gi]
+                lo = hi = base + i * mb
                 if windowed:                      # pages behind the window have gone: write the row anew
-                    row = flat[base + i * mb:base + i * mb + len(t)]
-                    row[:] = t
+                    hi = lo + len(t)
+                    flat[lo:hi] = t
                 elif len(t) != lens[i]:
-                    flat[base + i * mb + lens[i]:base + i * mb + len(t)] = t[lens[i]:]
+                    lo, hi = lo + lens[i], lo + len(t)
+                    flat[lo:hi] = t[lens[i]:]
                 lens[i] = len(t)
+                if hi > lo:
+                    pieces.append((flat[lo:hi], g.meta[lo:hi]))
         g.ctx.fresh = [False] * len(g.ctx.fresh)
-        self._staging.upload(flat, g.meta)
+        self._staging.upload_pieces(pieces)
         return True

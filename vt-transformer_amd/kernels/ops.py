@@ -479,6 +479,7 @@ def attention_f32(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
     return out
 
 
+ATTN_F32_MAX_HEAD_DIM = 256     # the float32 attention kernel keeps a head's dims in a block's registers: up to this many
 ATTN_ITEM_INTS = 8
 ATTN_CITEM_INTS = 6
 

@@ -23,7 +23,7 @@ import numpy as np
 
 from ..kernels import ops
 from .attention_plan import DECODE_BLOCKS, DECODE_BLOCKS_DIRECT, decode_chunk, decode_parts_max, device_plan, plan_step
-from .base import MIXERS, POSITIONS, CacheNeed, Part, Runtime, StateNeed, TensorDecl
+from .base import MIXERS, POSITIONS, CacheNeed, PageTensor, Part, Runtime, StateNeed, TensorDecl
 from .linear import can_add_residual, linear
 
 # the decoding kernels take the (token, head-of-group) rows of one entry as one tile of 16
@@ -49,8 +49,10 @@ class PagedAttention(Part):
         self.width = int(width)
         self.nh, self.nkv, self.d = int(num_heads), int(num_kv_heads), int(head_dim)
         if rt.lowp and (self.d % 16 or not 16 <= self.d <= 256):
-            raise ValueError(f"head size {self.d}: the 16-bit attention kernels take multiples of 16 from 16 to 256 "
-                             f"(float32 takes any)")
+            raise ValueError(f"head size {self.d}: the 16-bit attention kernels take multiples of 16 from 16 to 256")
+        if not rt.lowp and not 1 <= self.d <= ops.ATTN_F32_MAX_HEAD_DIM:
+            raise ValueError(f"head size {self.d}: the float32 attention kernel takes any size up to "
+                             f"{ops.ATTN_F32_MAX_HEAD_DIM}")
         self.qkv_bias, self.out_bias = bool(qkv_bias), bool(out_bias)
         self.window = int(window)
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.d)
@@ -76,8 +78,11 @@ class PagedAttention(Part):
 
     # -- what the cache manager must hold for this mixer --------------------
     def cache_need(self) -> Optional[CacheNeed]:
-        # the 16-bit kernels read keys 16 at a time, from one page
-        return CacheNeed(self.nkv, self.d, self.window, page_multiple=16 if self.rt.lowp else 1)
+        """A page holds a token's keys as [kv head][slot][D] and its values transposed, [kv head][D][slot], so that
+        one read of a kv head's page serves all the query heads of its group and the kernels read four keys of one
+        dim with one load; in the runtime's dtype.  The 16-bit kernels read keys 16 at a time, from one page."""
+        return CacheNeed((PageTensor("k", (self.nkv, self.d), slot_axis=1), PageTensor("v", (self.nkv, self.d), slot_axis=2)),
+                         window=self.window, page_multiple=16 if self.rt.lowp else 1)
 
     def state_need(self) -> Optional[StateNeed]:
         return None
@@ -113,7 +118,8 @@ class PagedAttention(Part):
 
     # -- one step --------------------------------------------------------------
     def _decode_key(self):
-        return ("attention.decode_chunk", self.nkv)
+        # what the cut of a decoding step's keys depends on: layers that agree in these share one
+        return ("attention.decode_chunk", self.nkv, self._direct(), self.window)
 
     def _items_key(self):
         return ("attention.items", self.nh // self.nkv, self.window, self.nkv, self.d)
@@ -136,6 +142,8 @@ class PagedAttention(Part):
             key = self._decode_key()
             if key in ctx.extra_host:
                 return None
+            # (cut from the whole lengths also where a window hides most keys: the kernel numbers an entry's ranges
+            # from its first key, range p holds keys p * chunk .. and p stays below p_max only if chunk covers them all)
             chunk = decode_chunk(ctx.h_kv_lens, decode_parts_max(ctx.n_positions), n_kv=self.nkv,
                                  want_blocks=DECODE_BLOCKS_DIRECT if self._direct() else DECODE_BLOCKS)
             return {key: np.array([chunk], np.int32)}
@@ -189,30 +197,30 @@ class PagedAttention(Part):
             out = rt.buffer("attn.out", (n, nq), rt.dtype)
             part_o = rt.buffer("attn.dec_part_o", (n * p_max * nkv * 16 * d,), torch.float32)
             part_ml = rt.buffer("attn.dec_part_ml", (n * p_max * nkv * 32,), torch.float32)
-            ops.attention_bf16_decode_fused(qkv, cos, sin, cache.k, cache.v, cache.block_table, ctx.entry_pos0,
+            ops.attention_bf16_decode_fused(qkv, cos, sin, cache["k"], cache["v"], cache.block_table, ctx.entry_pos0,
                                             chunk, p_max, out, part_o, part_ml, nh, nkv, d, self.window, self.scale)
             return linear(rt, out, self.w_o, self.b_o, "attn.o", packed=self.p_o, residual=residual, hand_on=hand_on)
         q = rt.buffer("attn.q", (n, nq), rt.dtype)
-        ops.rope_store(qkv, cos, sin, ctx.positions, ctx.tok_entry, cache.block_table, q, cache.k, cache.v, nh, nkv, d,
+        ops.rope_store(qkv, cos, sin, ctx.positions, ctx.tok_entry, cache.block_table, q, cache["k"], cache["v"], nh, nkv, d,
                        write_kv=cache.writes)
         out = rt.buffer("attn.out", (n, nq), rt.dtype)
         if rt.dtype == torch.float32:
-            ops.attention_f32(q, cache.k, cache.v, ctx.positions, ctx.tok_entry, cache.block_table, out, nh, nkv, d,
+            ops.attention_f32(q, cache["k"], cache["v"], ctx.positions, ctx.tok_entry, cache.block_table, out, nh, nkv, d,
                               self.window, self.scale)
         elif chunk is not None:
             # one token per entry: the kernel cuts the keys itself from the positions on the device
             part_o = rt.buffer("attn.dec_part_o", (n * p_max * nkv * 16 * d,), torch.float32)
             part_ml = rt.buffer("attn.dec_part_ml", (n * p_max * nkv * 32,), torch.float32)
-            ops.attention_bf16_decode(q, cache.k, cache.v, cache.block_table, ctx.entry_pos0, chunk, p_max, out,
+            ops.attention_bf16_decode(q, cache["k"], cache["v"], cache.block_table, ctx.entry_pos0, chunk, p_max, out,
                                       part_o, part_ml, nh, nkv, d, self.window, self.scale)
         else:
             plan = self._plan(ctx)
             if plan.n_items:        # decoded tokens and short portions: 16-row items, keys split where that helps
-                ops.attention_bf16(q, cache.k, cache.v, cache.block_table, plan.items, plan.n_items, plan.citems,
+                ops.attention_bf16(q, cache["k"], cache["v"], cache.block_table, plan.items, plan.n_items, plan.citems,
                                    plan.n_citems, out, plan.part_o, plan.part_ml, nh, nkv, d, self.window, self.scale,
                                    max_part=plan.n_parts, rt=plan.rt)
             if plan.n_tile_items:   # long portions: key/value blocks through LDS, shared by four waves
-                ops.attention_bf16_tiles(q, cache.k, cache.v, cache.block_table, plan.tile_items, plan.n_tile_items,
+                ops.attention_bf16_tiles(q, cache["k"], cache["v"], cache.block_table, plan.tile_items, plan.n_tile_items,
                                          out, nh, nkv, d, self.window, self.scale, rt=plan.tile_rt,
                                          citems=plan.tile_citems, n_citems=plan.n_tile_citems,
                                          part_o=plan.tile_part_o, part_ml=plan.tile_part_ml, n_parts=plan.n_tile_parts)

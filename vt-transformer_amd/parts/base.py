@@ -56,16 +56,54 @@ class TensorDecl:
 
 
 @dataclass(frozen=True)
-class CacheNeed:
-    """Keys and values that a mixer wants kept in pages, per token."""
+class PageTensor:
+    """One tensor of a cache page, as the mixer that owns it lays it out: what it keeps per token (`token_shape`)
+    and where the page's token slots lie among those axes (`slot_axis`: the index at which an axis of page_size
+    slots is inserted).  Keys kept as [kv head][slot][D] are PageTensor("k", (kv_heads, D), 1); values kept
+    transposed, [kv head][D][slot], are PageTensor("v", (kv_heads, D), 2); one latent vector per token is
+    PageTensor("latent", (rank,), 0).  dtype None: the runtime's."""
 
-    kv_heads: int
-    head_dim: int
-    window: int = 0  # 0: every key stays; W: a key is dead once W later tokens exist
+    name: str
+    token_shape: Tuple[int, ...]
+    slot_axis: int = 0
+    dtype: Optional[torch.dtype] = None
+
+    def __post_init__(self):
+        if not 0 <= self.slot_axis <= len(self.token_shape):
+            raise ValueError(f"page tensor '{self.name}': slot axis {self.slot_axis} is outside its {len(self.token_shape)} axes")
+
+    def page_shape(self, page_size: int) -> Tuple[int, ...]:
+        s = [int(x) for x in self.token_shape]
+        s.insert(self.slot_axis, int(page_size))
+        return tuple(s)
+
+    def token_elems(self) -> int:
+        n = 1
+        for x in self.token_shape:
+            n *= int(x)
+        return n
+
+
+@dataclass(frozen=True)
+class CacheNeed:
+    """What a mixer wants kept in pages: the tensors of a page (the layout is the mixer's own: the cache manager
+    only allocates what is listed and hands the mixer a dict by name), how long a token's entry stays alive, and the
+    page sizes that the mixer's kernels take.  Layers whose needs are equal share a group of pages (one pool, one
+    block table per request)."""
+
+    tensors: Tuple[PageTensor, ...]
+    window: int = 0  # 0: every token stays; W: a token is dead once W later tokens exist
     page_multiple: int = 1  # the mixer's kernels take pages whose size is a multiple of this many tokens
 
     def group_key(self):
-        return (self.kv_heads, self.head_dim, self.window)
+        return (self.tensors, self.window)
+
+    def same_layout(self, other: "CacheNeed") -> bool:
+        """Whether a mixer with this need can read pages that a mixer with the other need writes."""
+        return self.tensors == other.tensors
+
+    def bytes_per_token(self, runtime_dtype: torch.dtype) -> int:
+        return sum(t.token_elems() * torch.empty((), dtype=t.dtype or runtime_dtype).element_size() for t in self.tensors)
 
 
 @dataclass(frozen=True)
@@ -193,15 +231,26 @@ class HostStaging:
 
     def upload(self, host, dev: torch.Tensor) -> None:
         """host: a numpy array of the buffer's dtype; dev: a device tensor of the same size."""
-        n = int(host.size)
+        self.upload_pieces([(host, dev)])
+
+    def upload_pieces(self, pieces) -> None:
+        """Several (host array, device tensor of the same size) pairs through one pinned buffer: one wait for the
+        buffer, one copy to the device per piece."""
+        n = sum(int(h.size) for h, _ in pieces)
         slot = self._slots[self._next]
         self._next = (self._next + 1) % len(self._slots)
         if slot[1] is not None:
             slot[1].synchronize()
         if slot[0] is None or slot[0].numel() < n:
             slot[0] = torch.empty(max(n, 256), dtype=self.dtype, pin_memory=True)
-        slot[0][:n].numpy()[...] = host.reshape(-1)
-        dev.view(-1).copy_(slot[0][:n], non_blocking=True)
+        at = 0
+        for host, dev in pieces:
+            k = int(host.size)
+            if k == 0:
+                continue
+            slot[0][at:at + k].numpy()[...] = host.reshape(-1)
+            dev.view(-1).copy_(slot[0][at:at + k], non_blocking=True)
+            at += k
         if slot[1] is None:
             slot[1] = torch.cuda.Event()
         slot[1].record()

@@ -42,9 +42,20 @@ def packed_kernel_rows(m: int, k: int) -> int:
 FUSE_MAX_ROWS = ops.NORM_MAX_ROWS
 
 
+def norm_inside_products(rt: Runtime) -> bool:
+    """Whether this runtime's products may apply an RMSNorm on their way (the norm in front of a few-row product, or
+    handed from the product in front of it to the product behind it).  Those kernels round the stream times the
+    norm's gains to 16 bits and divide by the root afterwards, on the fp32 sums.  bfloat16 has float32's range, so
+    the order costs nothing there.  float16 does not: an un-normalised h * gain beyond 65,504 would become infinite and
+    one below 6e-5 would lose bits, where the normalised value that the reference rounds ((w * x) * r,
+    v1/tensortype/hip_kernels/rmsnorm.cpp:28-41) is harmless.  In float16 the norm therefore stays a kernel of its
+    own, which rounds once, behind the scaling."""
+    return rt.lowp and rt.dtype != torch.float16
+
+
 def can_fuse(rt: Runtime, n: int) -> bool:
     """Whether a product of n rows can take the residual stream with its norm still to be applied."""
-    return rt.lowp and n <= FUSE_MAX_ROWS
+    return norm_inside_products(rt) and n <= FUSE_MAX_ROWS
 
 
 def can_add_residual(rt: Runtime, n: int, m: int, k: int) -> bool:
@@ -55,12 +66,12 @@ def can_add_residual(rt: Runtime, n: int, m: int, k: int) -> bool:
 
 def can_hand_norm_on(rt: Runtime, n: int, m: int, k: int) -> bool:
     """Whether the product of n rows with W [m, k], adding to the residual stream, can prepare the norm behind it."""
-    return rt.lowp and n <= ops.LINK_MAX_ROWS and ops.linear_bf16_link_shares(n, m, k) > 0
+    return norm_inside_products(rt) and n <= ops.LINK_MAX_ROWS and ops.linear_bf16_link_shares(n, m, k) > 0
 
 
 def takes_prepared_norm(rt: Runtime, n: int, k: int) -> bool:
     """Whether a product of n rows over k can take a norm that the product in front has prepared."""
-    return rt.lowp and n <= ops.LINK_MAX_ROWS and k % 8 == 0
+    return norm_inside_products(rt) and n <= ops.LINK_MAX_ROWS and k % 8 == 0
 
 
 def linear(rt: Runtime, x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], name: str,
