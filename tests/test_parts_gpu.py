@@ -606,5 +606,7 @@ def test_a_mixer_that_keeps_one_latent_vector_per_token_in_pages_of_its_own(tmp_
     assert runner.storage.n_groups == 2
     assert set(runner.storage.pages[0]) == {"latent"} and runner.storage.pages[0]["latent"].dtype == torch.float32
     assert runner.storage.pages[0]["latent"].shape[2:] == (16, 24) and set(runner.storage.pages[1]) == {"k", "v"}
-    check(run_in_process(runner, steps), 3e-2)
+    # (scores of ten and more, rounded to bfloat16 on their way: a few per cent on the weights; a latent vector read
+    # from a wrong slot moves a row by its whole size)
+    check(run_in_process(runner, steps), 8e-2)
     assert sum(runner.cache.held_pages()) == 0

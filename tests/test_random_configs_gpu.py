@@ -238,7 +238,8 @@ def test_the_whole_vocabulary(name, hidden, heads, kv, inter, tied):
         model.load(w16.__getitem__)
         rows = model.embedding.forward(torch.tensor([0, V - 1], dtype=torch.int32, device="cuda"))
         table = w16["model.embed_tokens.weight"]
-        assert torch.equal(rows.cpu(), table[[0, V - 1]].float().cpu()), (name, dtype, "embedding rows")
+        # (as the model holds them: float16 has subnormals where bfloat16 still has eight bits)
+        assert torch.equal(rows.cpu(), table[[0, V - 1]].to(model.rt.dtype).float().cpu()), (name, dtype, "embedding rows")
         runner = make_runner(model, pool_tokens=64, page_size=16, max_requests=2, max_seq_len=64)
         runner.admit("r")
         got = [runner.step([StepEntry("r", toks[:40], list(range(40)))]).float().cpu()]
