@@ -437,12 +437,18 @@ def test_attention_fp32_one_key_is_value_row_and_zero_query_is_mean():
 # ---------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("nh,kvh,d,page_size", [(4, 2, 16, 16), (5, 1, 48, 32), (28, 4, 128, 16), (64, 8, 128, 16)])
-def test_rope_store(dtype, nh, kvh, d, page_size):
+@pytest.mark.parametrize("many", [False, True])
+def test_rope_store(dtype, nh, kvh, d, page_size, many):
+    """many: enough tokens for the kernel that takes sixteen tokens to a block and writes the values' page rows
+    through LDS; portions that start at a page's edge (whole rows in one store) and in the middle of a page, a single
+    token, a portion that ends in the middle of a group of sixteen."""
     from vt_transformer_amd.parts.rotary import rotary_table
     o = ops()
     g = torch.Generator().manual_seed(12)
     theta = 10000.0
     entries = [(0, 20), (33, 1), (page_size - 1, 3)]
+    if many:
+        entries = [(5, 70), (0, 48), (page_size - 3, 37), (64, 1), (2 * page_size, 21)]
     n = sum(x[1] for x in entries)
     width = (nh + 2 * kvh) * d
     qkv = torch.randn(n, width, generator=g)
@@ -456,7 +462,7 @@ def test_rope_store(dtype, nh, kvh, d, page_size):
     for e, t in enumerate(lens):
         for b in range(-(-t // page_size)):
             bt[e, b] = int(perm[nxt]); nxt += 1
-    cos, sin = rotary_table(64, d, theta)
+    cos, sin = rotary_table(256, d, theta)
     kp = torch.zeros(n_pages, kvh, page_size, d, dtype=dtype, device=DEV)
     vp = torch.zeros(n_pages, kvh, d, page_size, dtype=dtype, device=DEV)
     q_out = torch.empty(n, nh * d, dtype=dtype, device=DEV)
@@ -487,6 +493,7 @@ def test_rope_store(dtype, nh, kvh, d, page_size):
         e, p = int(tok_entry[t]), int(positions[t])
         written[int(bt[e, p // page_size]), p % page_size] = True
     assert float(kp.abs().sum(dim=(1, 3))[~written].sum()) == 0.0
+    assert float(vp.abs().sum(dim=(1, 2))[~written].sum()) == 0.0
 
 
 # ---------------------------------------------------------------------------
@@ -740,9 +747,15 @@ def test_rmsnorm_handed_from_one_product_to_the_next(n, h, k1, m2, gated, lp):
     assert rel_err(hbuf, h_ref) < 1e-5
     assert rel_err(ssq[:, :n].sum(dim=0), (h_ref * h_ref).sum(dim=1)) < 1e-5
     assert bool((ssq[:, n:] == 0).all())
-    # what the consumer reads: exactly bf16(h * gain) of the stream as the producer left it
-    assert torch.equal(xn.cpu(), (hbuf.cpu() * gain).to(lp))
-    normed = (hbuf.cpu() * gain).to(lp).double() / torch.sqrt((h_ref * h_ref).mean(dim=1, keepdim=True) + eps)
+    # what the consumer reads: h * gain of the stream as the producer left it, rounded to 16 bits.  bfloat16: the very
+    # bits of rounding the float32 product; float16: within half a unit in the last place of the product (the compiler
+    # may round the product to 16 bits in one instruction, where the host rounds it to float32 first)
+    prod = hbuf.cpu() * gain
+    if lp == torch.bfloat16:
+        assert torch.equal(xn.cpu(), prod.to(lp))
+    else:
+        assert bool(((xn.cpu().double() - prod.double()).abs() <= prod.double().abs() * 2.0 ** -11 * 1.001 + 2.0 ** -25).all())
+    normed = xn.cpu().double() / torch.sqrt((h_ref * h_ref).mean(dim=1, keepdim=True) + eps)
     if gated:
         out = torch.empty(n, m2, dtype=torch.float32, device=DEV)
         o.gated_linear_bf16_link(xn, o.pack_matrix_bf16(w2.to(DEV), halves=2), out, ssq, eps)
@@ -759,7 +772,8 @@ def test_rmsnorm_handed_from_one_product_to_the_next(n, h, k1, m2, gated, lp):
     if gated and n <= 16:
         same = torch.empty(n, m2, dtype=torch.float32, device=DEV)
         o.gated_linear_bf16(hbuf, o.pack_matrix_bf16(w2.to(DEV), halves=2), same, norm_gain=gain.to(DEV), norm_eps=eps)
-        assert rel_err(out, same) < 2e-6
+        # (float16: the two kernels may round h * gain to 16 bits with different instructions, once or twice)
+        assert rel_err(out, same) < (2e-6 if lp == torch.bfloat16 else 3e-5)
 
 
 def test_rmsnorm_hand_over_is_refused_where_it_cannot_work():

@@ -134,14 +134,98 @@ __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(float* __restrict__ h,
     }
 }
 
+// The same over many rows (a prompt portion): a block takes rows blockIdx.x, + gridDim.x, ... and asks for its next
+// row's values before it adds up and writes the row it holds, so that the memory always has this block's loads to
+// work on; the gains are read once per block.  The stream and the addend pass once and are loaded non-temporal, the
+// stream is stored so (the next norm reads it several large products later); the normed row is what the next kernel
+// reads and is stored plainly.  The sums are taken in the order of rmsnorm_vec_kernel: the same bits.
+typedef float ew_f32x4_t __attribute__((ext_vector_type(4)));
+typedef unsigned ew_u32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float4 load4_once(const float* p) {
+    const ew_f32x4_t v = __builtin_nontemporal_load((const ew_f32x4_t*)p);
+    return make_float4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ float4 load4_once(const bf16_t* p) {
+    const ew_u32x2_t u = __builtin_nontemporal_load((const ew_u32x2_t*)p);
+    return make_float4(lowp_lo(u.x), lowp_hi(u.x), lowp_lo(u.y), lowp_hi(u.y));
+}
+__device__ __forceinline__ void store4_once(float* p, float4 v) {
+    const ew_f32x4_t t = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(t, (ew_f32x4_t*)p);
+}
+
+template <typename TD, typename TO, bool HAS_DELTA, int NV>
+__global__ __launch_bounds__(256) void rmsnorm_rows_kernel(float* __restrict__ h, const TD* __restrict__ delta,
+                                                          const float* __restrict__ gain, TO* __restrict__ out,
+                                                          int n_rows, int hidden, float eps, int update) {
+    __shared__ float red[16];
+    const int tid = threadIdx.x, nq = hidden >> 2;
+    int r = blockIdx.x;
+    if (r >= n_rows) return;
+    float4 gn[NV], x[NV], nh[NV], nd[NV];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        const int qi = tid + v * 256;
+        if (qi < nq) gn[v] = load4(gain + 4 * qi);
+    }
+    auto fetch = [&](int row) __attribute__((always_inline)) {
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int qi = tid + v * 256;
+            if (qi < nq) {
+                nh[v] = load4_once(h + (size_t)row * hidden + 4 * qi);
+                if (HAS_DELTA) nd[v] = load4_once(delta + (size_t)row * hidden + 4 * qi);
+            }
+        }
+    };
+    fetch(r);
+    for (; r < n_rows; r += gridDim.x) {
+        float* hr = h + (size_t)r * hidden;
+        float ss = 0.f;
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int qi = tid + v * 256;
+            if (qi < nq) {
+                x[v] = nh[v];
+                if (HAS_DELTA) {
+                    x[v].x += nd[v].x; x[v].y += nd[v].y; x[v].z += nd[v].z; x[v].w += nd[v].w;
+                    if (update) store4_once(hr + 4 * qi, x[v]);
+                }
+                ss += x[v].x * x[v].x + x[v].y * x[v].y + x[v].z * x[v].z + x[v].w * x[v].w;
+            }
+        }
+        if (r + (int)gridDim.x < n_rows) fetch(r + gridDim.x);      // on their way while this row is added up and written
+        ss = block_sum(ss, red);
+        const float rinv = 1.0f / sqrtf(ss / (float)hidden + eps);
+        TO* o = out + (size_t)r * hidden;
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int qi = tid + v * 256;
+            if (qi < nq) {
+                const float4 g = gn[v];
+                store4(o + 4 * qi, make_float4((g.x * x[v].x) * rinv, (g.y * x[v].y) * rinv, (g.z * x[v].z) * rinv,
+                                               (g.w * x[v].w) * rinv));
+            }
+        }
+    }
+}
+
 template <typename TD, typename TO, bool HD>
 static void launch_rmsnorm(float* h, const void* delta, const float* gain, void* out, const int* rows, int n_out,
                            int hidden, float eps, int update_h, hipStream_t stream) {
     const bool aligned = (hidden % 4 == 0) && !((uintptr_t)h & 15) && !((uintptr_t)gain & 15) && !((uintptr_t)out & 15) &&
                          !((uintptr_t)delta & 15);
     const int nq = hidden / 4;
-#define VT_RNV(NV) rmsnorm_vec_kernel<TD, TO, HD, NV><<<n_out, 256, 0, stream>>>(h, (const TD*)delta, gain, (TO*)out, \
-                                                                               rows, hidden, eps, update_h)
+    // many rows and no row list: blocks that go on to further rows (about four blocks per compute unit)
+    const int row_blocks = 1024;
+#define VT_RNV(NV) do { \
+        if (!rows && n_out > row_blocks) \
+            rmsnorm_rows_kernel<TD, TO, HD, NV><<<row_blocks, 256, 0, stream>>>(h, (const TD*)delta, gain, (TO*)out, n_out, \
+                                                                                 hidden, eps, update_h); \
+        else \
+            rmsnorm_vec_kernel<TD, TO, HD, NV><<<n_out, 256, 0, stream>>>(h, (const TD*)delta, gain, (TO*)out, rows, hidden, \
+                                                                           eps, update_h); \
+    } while (0)
     if (aligned && nq <= 256 * 1) VT_RNV(1);
     else if (aligned && nq <= 256 * 2) VT_RNV(2);
     else if (aligned && nq <= 256 * 4) VT_RNV(4);
@@ -249,42 +333,37 @@ __global__ __launch_bounds__(256) void silu_mul_vec_kernel(const TI* __restrict_
     }
 }
 
-// bfloat16 in and out, widths that are a multiple of 8: 16 bytes per access, two accesses of gate and of up in
-// flight per thread.
+// 16-bit in and out, widths that are a multiple of 8.  A thread takes one group of eight columns in four rows: eight
+// 16-byte loads (gate and up of each row) are asked for before any is used, a wave's load is 1 KB of one row.  Loads
+// and stores are marked non-temporal: every byte passes once, and the memory delivers more to accesses so marked.
+// The gate's division is one reciprocal instruction (1 ulp, far below the 16-bit rounding of the result).
+typedef unsigned ew_u32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float silu_gate(float g, float u) { return g * __builtin_amdgcn_rcpf(1.f + __expf(-g)) * u; }
 __device__ __forceinline__ unsigned silu_mul_pair(unsigned g, unsigned u) {
-    const float g0 = lowp_lo(g), g1 = lowp_hi(g);
-    const float u0 = lowp_lo(u), u1 = lowp_hi(u);
-    return (unsigned)f32_to_bf16(g0 / (1.f + __expf(-g0)) * u0) | ((unsigned)f32_to_bf16(g1 / (1.f + __expf(-g1)) * u1) << 16);
+    return vt_pack2(silu_gate(lowp_lo(g), lowp_lo(u)), silu_gate(lowp_hi(g), lowp_hi(u)));
 }
+#define SILU_ROWS 4
 __global__ __launch_bounds__(256) void silu_mul_bf16x8_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ out,
                                                              int inter, int n) {
-    const int opr = inter >> 3;                                   // groups of 8 per row
-    const long long total = (long long)opr * n;
-    const long long stride = (long long)gridDim.x * 256;
-    for (long long base = (long long)blockIdx.x * 256 + threadIdx.x; base < total; base += 2 * stride) {
-        uint4 g[2], u[2];
-        long long idx[2];
+    const int c = (blockIdx.x * 256 + threadIdx.x) * 8;           // first of the thread's eight columns
+    if (c >= inter) return;
+    const int t0 = blockIdx.y * SILU_ROWS;
+    ew_u32x4_t g[SILU_ROWS], u[SILU_ROWS];
 #pragma unroll
-        for (int k = 0; k < 2; ++k) {
-            idx[k] = base + k * stride;
-            if (idx[k] < total) {
-                const long long t = idx[k] / opr;
-                const int i = (int)(idx[k] - t * opr) * 8;
-                const bf16_t* row = gu + (size_t)t * 2 * inter;
-                g[k] = *(const uint4*)(row + i);
-                u[k] = *(const uint4*)(row + inter + i);
-            }
+    for (int k = 0; k < SILU_ROWS; ++k) {
+        if (t0 + k < n) {
+            const bf16_t* row = gu + (size_t)(t0 + k) * 2 * inter + c;
+            g[k] = __builtin_nontemporal_load((const ew_u32x4_t*)row);
+            u[k] = __builtin_nontemporal_load((const ew_u32x4_t*)(row + inter));
         }
+    }
 #pragma unroll
-        for (int k = 0; k < 2; ++k) {
-            if (idx[k] < total) {
-                const long long t = idx[k] / opr;
-                const int i = (int)(idx[k] - t * opr) * 8;
-                uint4 o;
-                o.x = silu_mul_pair(g[k].x, u[k].x); o.y = silu_mul_pair(g[k].y, u[k].y);
-                o.z = silu_mul_pair(g[k].z, u[k].z); o.w = silu_mul_pair(g[k].w, u[k].w);
-                *(uint4*)(out + (size_t)t * inter + i) = o;
-            }
+    for (int k = 0; k < SILU_ROWS; ++k) {
+        if (t0 + k < n) {
+            ew_u32x4_t o;
+            o.x = silu_mul_pair(g[k].x, u[k].x); o.y = silu_mul_pair(g[k].y, u[k].y);
+            o.z = silu_mul_pair(g[k].z, u[k].z); o.w = silu_mul_pair(g[k].w, u[k].w);
+            __builtin_nontemporal_store(o, (ew_u32x4_t*)(out + (size_t)(t0 + k) * inter + c));
         }
     }
 }
@@ -293,10 +372,8 @@ template <typename TI, typename TO>
 static void launch_silu_mul(const void* gu, void* out, int n, int inter, hipStream_t stream) {
     if constexpr (sizeof(TI) == 2 && sizeof(TO) == 2) {
         if (inter % 8 == 0 && !((uintptr_t)gu & 15) && !((uintptr_t)out & 15)) {
-            const long long total = (long long)(inter / 8) * n;
-            long long blocks = (total + 511) / 512;
-            if (blocks > 8192) blocks = 8192;
-            silu_mul_bf16x8_kernel<<<(unsigned)(blocks < 1 ? 1 : blocks), 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, inter, n);
+            const dim3 grid((inter / 8 + 255) / 256, (n + SILU_ROWS - 1) / SILU_ROWS);
+            silu_mul_bf16x8_kernel<<<grid, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, inter, n);
             return;
         }
     }
@@ -449,6 +526,138 @@ __global__ __launch_bounds__(256) void rope_store_vec_kernel(RopeStoreArgs a) {
     }
 }
 
+// Many tokens, 16-bit pages (a prompt portion): a block takes sixteen consecutive tokens of the step and either one
+// kv head (its keys and its values) or RG_QH query heads.  The pages hold values transposed ([D][slot]), so a token
+// alone writes its D values two bytes at a time, a page row apart; here the sixteen tokens' values meet in LDS
+// ([D][token]) and a thread per dim writes the slots that are consecutive in one page with one store of up to 16 bytes
+// (a whole page row when the sixteen tokens are a page's, as in a prompt cut at page edges).  Runs are found from
+// the tokens' own pages and slots, so any mixture of entries and positions is written correctly, only less wide.
+// Rows that are rotated go four pieces of four dims per thread at a time, all their loads asked for first.
+#define RG_TOK 16
+#define RG_PAD 18       // halfwords per tile row: a thread per row reads them without bank conflicts
+#define RG_QH 4         // query heads of a block that rotates queries
+#define RG_U 4          // pieces in flight per thread
+template <typename TI>
+__global__ __launch_bounds__(256) void rope_store_group_kernel(RopeStoreArgs a, int n) {
+    extern __shared__ unsigned short rg_tile[];        // [D][RG_PAD]
+    __shared__ int s_page[RG_TOK], s_slot[RG_TOK], s_pos[RG_TOK];
+    const int tid = threadIdx.x;
+    const int t0 = blockIdx.x * RG_TOK, cnt = min(RG_TOK, n - t0);
+    const int D = a.D, half = a.rot >> 1, qd = D >> 2;
+    const bool kv_block = (int)blockIdx.y < a.n_kv;
+    const int kvh = blockIdx.y;                                         // (a kv block's head)
+    const int head0 = kv_block ? a.n_heads + kvh : ((int)blockIdx.y - a.n_kv) * RG_QH;
+    const int n_rot_heads = kv_block ? 1 : min(RG_QH, a.n_heads - head0);
+    if (tid < RG_TOK) {
+        int page = -1, slot = 0, pos = 0;
+        if (tid < cnt) {
+            pos = a.positions[t0 + tid];
+            if (kv_block) {
+                const int e = a.tok_entry[t0 + tid];
+                const int blk = pos / a.page_size;
+                slot = pos - blk * a.page_size;
+                const int pg = (blk >= 0 && blk < a.max_blocks) ? a.block_table[(size_t)e * a.max_blocks + blk] : -1;
+                if (pg >= 0 && pg < a.num_pages) page = pg;      // (no page: the host never asks for this)
+            }
+        }
+        s_page[tid] = page; s_slot[tid] = slot; s_pos[tid] = pos;
+    }
+    __syncthreads();
+    // the block's query heads, or its kv head's keys: rotated, a row of D at a time.  32 lanes along a row (four dims
+    // each), 8 rows side by side; row r is head r % n_rot_heads of token r / n_rot_heads (a product and a shift: the
+    // quotient of r < 64 by a number up to RG_QH), so that no piece costs an integer division.
+    const int lane_q = tid & 31, lane_r = tid >> 5;
+    const int n_rows = cnt * n_rot_heads;
+    const unsigned inv = (65536u + n_rot_heads - 1) / n_rot_heads;
+    for (int q0 = lane_q; q0 < qd; q0 += 32) {
+        const int i = q0 * 4;
+        const bool rotated = i < a.rot, low = i < half;
+        const int ip = low ? i : i - half, iy = low ? i + half : i - half;
+        for (int r0 = lane_r; r0 < n_rows; r0 += 8 * RG_U) {
+            float4 x[RG_U], y[RG_U], cc[RG_U], sn[RG_U];
+#pragma unroll
+            for (int u = 0; u < RG_U; ++u) {
+                const int r = r0 + 8 * u;
+                if (r < n_rows) {
+                    const int j = (int)((r * inv) >> 16), h = r - j * n_rot_heads;
+                    const int pos = s_pos[j];
+                    const int tp = pos < a.max_pos ? (pos < 0 ? 0 : pos) : a.max_pos - 1;
+                    const TI* hp = (const TI*)a.qkv + (size_t)(t0 + j) * a.in_stride + (size_t)(head0 + h) * D;
+                    x[u] = load4(hp + i);
+                    if (rotated) {
+                        y[u] = load4(hp + iy);
+                        cc[u] = load4(a.cos_t + (size_t)tp * half + ip);
+                        sn[u] = load4(a.sin_t + (size_t)tp * half + ip);
+                    }
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < RG_U; ++u) {
+                const int r = r0 + 8 * u;
+                if (r >= n_rows) continue;
+                const int j = (int)((r * inv) >> 16), h = r - j * n_rot_heads;
+                float4 o = x[u];
+                if (rotated)
+                    o = make_float4(rotate_pair(cc[u].x, sn[u].x, x[u].x, y[u].x, low), rotate_pair(cc[u].y, sn[u].y, x[u].y, y[u].y, low),
+                                    rotate_pair(cc[u].z, sn[u].z, x[u].z, y[u].z, low), rotate_pair(cc[u].w, sn[u].w, x[u].w, y[u].w, low));
+                if (!kv_block) store4((bf16_t*)a.q_out + ((size_t)(t0 + j) * a.n_heads + head0 + h) * D + i, o);
+                else if (s_page[j] >= 0)
+                    store4((bf16_t*)a.k_pages + (((size_t)s_page[j] * a.n_kv + kvh) * a.page_size + s_slot[j]) * D + i, o);
+            }
+        }
+    }
+    if (!kv_block) return;
+    // the head's values into the tile, a column per token
+    for (int q0 = lane_q; q0 < qd; q0 += 32) {
+        const int i = q0 * 4;
+        for (int j = lane_r; j < cnt; j += 8) {
+            const TI* hp = (const TI*)a.qkv + (size_t)(t0 + j) * a.in_stride + (size_t)(a.n_heads + a.n_kv + kvh) * D;
+            const float4 x = load4(hp + i);
+            rg_tile[(i + 0) * RG_PAD + j] = f32_to_bf16(x.x);
+            rg_tile[(i + 1) * RG_PAD + j] = f32_to_bf16(x.y);
+            rg_tile[(i + 2) * RG_PAD + j] = f32_to_bf16(x.z);
+            rg_tile[(i + 3) * RG_PAD + j] = f32_to_bf16(x.w);
+        }
+    }
+    __syncthreads();
+    // a thread per dim: the runs of tokens whose slots follow each other in one page, each in the widest stores
+    // that the slot's alignment allows (page rows start at multiples of 16 bytes: page sizes are multiples of 8)
+    for (int d = tid; d < D; d += 256) {
+        const unsigned short* src = rg_tile + d * RG_PAD;
+        int j = 0;
+        while (j < cnt) {
+            const int page = s_page[j], slot = s_slot[j];
+            int m = 1;
+            while (j + m < cnt && s_page[j + m] == page && s_slot[j + m] == slot + m) ++m;
+            if (page >= 0) {
+                bf16_t* dst = (bf16_t*)a.v_pages + (((size_t)page * a.n_kv + kvh) * D + d) * a.page_size + slot;
+                int k = 0;
+                while (k < m) {
+                    const int sl = slot + k, left = m - k;
+                    const unsigned short* sp = src + j + k;
+                    if (!(sl & 7) && left >= 8) {
+                        uint4 v;
+                        v.x = sp[0] | ((unsigned)sp[1] << 16); v.y = sp[2] | ((unsigned)sp[3] << 16);
+                        v.z = sp[4] | ((unsigned)sp[5] << 16); v.w = sp[6] | ((unsigned)sp[7] << 16);
+                        *(uint4*)(dst + k) = v;
+                        k += 8;
+                    } else if (!(sl & 3) && left >= 4) {
+                        *(uint2*)(dst + k) = make_uint2(sp[0] | ((unsigned)sp[1] << 16), sp[2] | ((unsigned)sp[3] << 16));
+                        k += 4;
+                    } else if (!(sl & 1) && left >= 2) {
+                        *(unsigned*)(dst + k) = sp[0] | ((unsigned)sp[1] << 16);
+                        k += 2;
+                    } else {
+                        dst[k] = sp[0];
+                        k += 1;
+                    }
+                }
+            }
+            j += m;
+        }
+    }
+}
+
 extern "C" int vt_rope_store(const void* qkv, int in_dtype, long long in_stride, const float* cos_t, const float* sin_t,
                              int rot, int max_pos, const int* positions, const int* tok_entry, const int* block_table,
                              int max_blocks, void* q_out, void* k_pages, void* v_pages, int out_dtype, int page_size,
@@ -471,9 +680,16 @@ extern "C" int vt_rope_store(const void* qkv, int in_dtype, long long in_stride,
     dim3 grid(n, n_heads + (write_kv ? 2 * n_kv : 0));
     VT_REQUIRE(grid.y <= 65535, "vt_rope_store: too many heads (%u)", grid.y);
     int threads = D <= 64 ? 64 : (D <= 128 ? 128 : 256);
+    // sixteen tokens and a kv head per block, the values through LDS: 16-bit pages, a portion of many tokens
+    const bool grouped = vec && write_kv && out_dtype == VT_BF16 && n >= 4 * RG_TOK && page_size % 8 == 0 &&
+                         n_kv + n_heads <= 65535 && !((uintptr_t)v_pages & 15);
+    const dim3 ggrid((n + RG_TOK - 1) / RG_TOK, n_kv + (n_heads + RG_QH - 1) / RG_QH);
+    const size_t glds = (size_t)D * RG_PAD * sizeof(unsigned short);
+    VT_REQUIRE(!grouped || glds <= 48 * 1024, "vt_rope_store: head size %d is too large for the grouped kernel", D);
 #define VT_RS(TI, TO)                                                                    \
     do {                                                                                 \
-        if (vec) rope_store_vec_kernel<TI, TO><<<n, 256, 0, stream>>>(a);                \
+        if (grouped && sizeof(TO) == 2) rope_store_group_kernel<TI><<<ggrid, 256, glds, stream>>>(a, n); \
+        else if (vec) rope_store_vec_kernel<TI, TO><<<n, 256, 0, stream>>>(a);           \
         else rope_store_kernel<TI, TO><<<grid, threads, 0, stream>>>(a);                 \
     } while (0)
     if (in_dtype == VT_F32 && out_dtype == VT_F32) VT_RS(float, float);
