@@ -17,6 +17,7 @@ layers.
 """
 from __future__ import annotations
 
+import gc
 from dataclasses import dataclass
 from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
@@ -306,8 +307,17 @@ class ModelRunner:
                 self.model.forward(g.ctx, caches, self.storage.state)
                 torch.cuda.synchronize()
                 g.graph = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(g.graph):
-                    g.logits = self.model.forward(g.ctx, caches, self.storage.state)
+                # No cyclic garbage collection while the step is recorded: it may destroy an object that owns device
+                # or pinned memory, events or another recorded graph (an engine that the caller has dropped), and
+                # freeing those is not allowed while a stream records.  (Entering the recording collects first.)
+                gc_was_on = gc.isenabled()
+                gc.disable()
+                try:
+                    with torch.cuda.graph(g.graph):
+                        g.logits = self.model.forward(g.ctx, caches, self.storage.state)
+                finally:
+                    if gc_was_on:
+                        gc.enable()
                 self._graphs[b] = g
             else:
                 self._fill_context(g.ctx, h, all_rows, g.meta)
