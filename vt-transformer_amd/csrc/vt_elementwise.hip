@@ -334,8 +334,8 @@ __global__ __launch_bounds__(256) void silu_mul_vec_kernel(const TI* __restrict_
 }
 
 // 16-bit in and out, widths that are a multiple of 8.  A thread takes one group of eight columns in four rows: eight
-// 16-byte loads (gate and up of each row) are asked for before any is used, a wave's load is 1 KB of one row.  Loads
-// and stores are marked non-temporal: every byte passes once, and the memory delivers more to accesses so marked.
+// 16-byte loads (gate and up of each row) are asked for before any is used, a wave's load is 1 KB of one row.  The
+// loads are marked non-temporal: every byte passes once, and the memory delivers more to loads so marked.
 // The gate's division is one reciprocal instruction (1 ulp, far below the 16-bit rounding of the result).
 typedef unsigned ew_u32x4_t __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ float silu_gate(float g, float u) { return g * __builtin_amdgcn_rcpf(1.f + __expf(-g)) * u; }
@@ -363,7 +363,8 @@ __global__ __launch_bounds__(256) void silu_mul_bf16x8_kernel(const bf16_t* __re
             ew_u32x4_t o;
             o.x = silu_mul_pair(g[k].x, u[k].x); o.y = silu_mul_pair(g[k].y, u[k].y);
             o.z = silu_mul_pair(g[k].z, u[k].z); o.w = silu_mul_pair(g[k].w, u[k].w);
-            __builtin_nontemporal_store(o, (ew_u32x4_t*)(out + (size_t)(t0 + k) * inter + c));
+            // (stored plainly: the product behind reads it next, out of the memory-side cache if it is left there)
+            *(ew_u32x4_t*)(out + (size_t)(t0 + k) * inter + c) = o;
         }
     }
 }
