@@ -134,98 +134,14 @@ __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(float* __restrict__ h,
     }
 }
 
-// The same over many rows (a prompt portion): a block takes rows blockIdx.x, + gridDim.x, ... and asks for its next
-// row's values before it adds up and writes the row it holds, so that the memory always has this block's loads to
-// work on; the gains are read once per block.  The stream and the addend pass once and are loaded non-temporal, the
-// stream is stored so (the next norm reads it several large products later); the normed row is what the next kernel
-// reads and is stored plainly.  The sums are taken in the order of rmsnorm_vec_kernel: the same bits.
-typedef float ew_f32x4_t __attribute__((ext_vector_type(4)));
-typedef unsigned ew_u32x2_t __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ float4 load4_once(const float* p) {
-    const ew_f32x4_t v = __builtin_nontemporal_load((const ew_f32x4_t*)p);
-    return make_float4(v.x, v.y, v.z, v.w);
-}
-__device__ __forceinline__ float4 load4_once(const bf16_t* p) {
-    const ew_u32x2_t u = __builtin_nontemporal_load((const ew_u32x2_t*)p);
-    return make_float4(lowp_lo(u.x), lowp_hi(u.x), lowp_lo(u.y), lowp_hi(u.y));
-}
-__device__ __forceinline__ void store4_once(float* p, float4 v) {
-    const ew_f32x4_t t = {v.x, v.y, v.z, v.w};
-    __builtin_nontemporal_store(t, (ew_f32x4_t*)p);
-}
-
-template <typename TD, typename TO, bool HAS_DELTA, int NV>
-__global__ __launch_bounds__(256) void rmsnorm_rows_kernel(float* __restrict__ h, const TD* __restrict__ delta,
-                                                          const float* __restrict__ gain, TO* __restrict__ out,
-                                                          int n_rows, int hidden, float eps, int update) {
-    __shared__ float red[16];
-    const int tid = threadIdx.x, nq = hidden >> 2;
-    int r = blockIdx.x;
-    if (r >= n_rows) return;
-    float4 gn[NV], x[NV], nh[NV], nd[NV];
-#pragma unroll
-    for (int v = 0; v < NV; ++v) {
-        const int qi = tid + v * 256;
-        if (qi < nq) gn[v] = load4(gain + 4 * qi);
-    }
-    auto fetch = [&](int row) __attribute__((always_inline)) {
-#pragma unroll
-        for (int v = 0; v < NV; ++v) {
-            const int qi = tid + v * 256;
-            if (qi < nq) {
-                nh[v] = load4_once(h + (size_t)row * hidden + 4 * qi);
-                if (HAS_DELTA) nd[v] = load4_once(delta + (size_t)row * hidden + 4 * qi);
-            }
-        }
-    };
-    fetch(r);
-    for (; r < n_rows; r += gridDim.x) {
-        float* hr = h + (size_t)r * hidden;
-        float ss = 0.f;
-#pragma unroll
-        for (int v = 0; v < NV; ++v) {
-            const int qi = tid + v * 256;
-            if (qi < nq) {
-                x[v] = nh[v];
-                if (HAS_DELTA) {
-                    x[v].x += nd[v].x; x[v].y += nd[v].y; x[v].z += nd[v].z; x[v].w += nd[v].w;
-                    if (update) store4_once(hr + 4 * qi, x[v]);
-                }
-                ss += x[v].x * x[v].x + x[v].y * x[v].y + x[v].z * x[v].z + x[v].w * x[v].w;
-            }
-        }
-        if (r + (int)gridDim.x < n_rows) fetch(r + gridDim.x);      // on their way while this row is added up and written
-        ss = block_sum(ss, red);
-        const float rinv = 1.0f / sqrtf(ss / (float)hidden + eps);
-        TO* o = out + (size_t)r * hidden;
-#pragma unroll
-        for (int v = 0; v < NV; ++v) {
-            const int qi = tid + v * 256;
-            if (qi < nq) {
-                const float4 g = gn[v];
-                store4(o + 4 * qi, make_float4((g.x * x[v].x) * rinv, (g.y * x[v].y) * rinv, (g.z * x[v].z) * rinv,
-                                               (g.w * x[v].w) * rinv));
-            }
-        }
-    }
-}
-
 template <typename TD, typename TO, bool HD>
 static void launch_rmsnorm(float* h, const void* delta, const float* gain, void* out, const int* rows, int n_out,
                            int hidden, float eps, int update_h, hipStream_t stream) {
     const bool aligned = (hidden % 4 == 0) && !((uintptr_t)h & 15) && !((uintptr_t)gain & 15) && !((uintptr_t)out & 15) &&
                          !((uintptr_t)delta & 15);
     const int nq = hidden / 4;
-    // many rows and no row list: blocks that go on to further rows (about four blocks per compute unit)
-    const int row_blocks = 1024;
-#define VT_RNV(NV) do { \
-        if (!rows && n_out > row_blocks) \
-            rmsnorm_rows_kernel<TD, TO, HD, NV><<<row_blocks, 256, 0, stream>>>(h, (const TD*)delta, gain, (TO*)out, n_out, \
-                                                                                 hidden, eps, update_h); \
-        else \
-            rmsnorm_vec_kernel<TD, TO, HD, NV><<<n_out, 256, 0, stream>>>(h, (const TD*)delta, gain, (TO*)out, rows, hidden, \
-                                                                           eps, update_h); \
-    } while (0)
+#define VT_RNV(NV) rmsnorm_vec_kernel<TD, TO, HD, NV><<<n_out, 256, 0, stream>>>(h, (const TD*)delta, gain, (TO*)out, \
+                                                                               rows, hidden, eps, update_h)
     if (aligned && nq <= 256 * 1) VT_RNV(1);
     else if (aligned && nq <= 256 * 2) VT_RNV(2);
     else if (aligned && nq <= 256 * 4) VT_RNV(4);

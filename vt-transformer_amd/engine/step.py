@@ -114,7 +114,9 @@ class ModelRunner:
         self._staging = HostStaging(torch.int32)
         # Decoding steps of a 16-bit model are captured once per batch size and replayed, unless a mixer keeps
         # state of its own between steps (the warm-up run before a capture would advance it twice) or a part does
-        # not declare that its step can be replayed.
+        # not declare that its step can be replayed.  This is decided here, once, for the whole model: one part that
+        # is stateful or says nothing keeps every step of the model on the launch-by-launch path (and the engine,
+        # which asks `replays()`, then never starts a step ahead of the host); the other parts lose nothing but that.
         self.decode_graphs = False
         self._graphs: Dict[int, _DecodeGraph] = {}
         self._stateless = all(s is None for s in self.storage.state)
