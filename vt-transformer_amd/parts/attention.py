@@ -179,14 +179,16 @@ class PagedAttention(Part):
                          packed=self.p_qkv.first_rows(nq) if self.p_qkv is not None else None)
         tables = self.position.rotary_tables(ctx.n_positions)
         if tables is None and hasattr(self.position, "apply") and self.position.dim != 0:
-            # a position encoding that is not a plain rotation: let it rewrite queries and keys, then store unrotated
-            qv = qkv[:, :nq].reshape(n, nh, d)
-            kv = qkv[:, nq:nq + nkv * d].reshape(n, nkv, d) if cache.writes else None
+            # a position encoding that is not a plain rotation: it rewrites queries and keys with whatever it brings
+            # (kernels of its own, or torch as the tests' toy does), in the projection's scratch buffer; they are then
+            # stored unrotated
+            qv = qkv[:, :nq].view(n, nh, d)
+            kv = qkv[:, nq:nq + nkv * d].view(n, nkv, d) if cache.writes else None
             q2, k2 = self.position.apply(qv, kv, ctx.positions)
-            qkv = qkv.clone()
-            qkv[:, :nq] = q2.reshape(n, nq).to(qkv.dtype)
-            if cache.writes:
-                qkv[:, nq:nq + nkv * d] = k2.reshape(n, nkv * d).to(qkv.dtype)
+            if q2 is not qv:
+                qv.copy_(q2)
+            if cache.writes and k2 is not kv:
+                kv.copy_(k2)
         cos, sin = tables if tables is not None else (None, None)
         plain_positions = tables is not None or getattr(self.position, "dim", 0) == 0
         chunk = ctx.extra.get(self._decode_key()) if rt.lowp and ctx.single_token else None
