@@ -714,6 +714,9 @@ constexpr int KBUF = DIRECT ? KB * D : KB * KROW;        // elements of a key bu
 constexpr int VBUF = DIRECT ? D * KB : D * VROW;
 constexpr int TILE_LDS_BYTES = 2 * (KBUF + VBUF) * (int)sizeof(bf16_t);
 
+constexpr int AHEAD = 4;                       // LDS operands on their way before the products that use them
+constexpr int SCHED_MFMA = 0x008, SCHED_LDS_READ = 0x100;      // instruction classes of sched_group_barrier
+
 // key (relative to the block's first) of score tile kt, lane group g, register i
 __device__ __forceinline__ int tile_key(int kt, int g, int i) { return 32 * (kt >> 1) + 8 * g + 4 * (kt & 1) + i; }
 
@@ -878,55 +881,50 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_tile_kernel(At
     const char* const v_base = (const char*)(a.v_pages + (size_t)kvh * ps * D);
     // (a native vector type: copies of HIP's uint4 struct become memcpy calls that keep the stage in scratch memory)
     u32x4_t st_k[KT][NP], st_v[KT][NP];
-    // Direct path: wave w brings the key pieces w, w + 4, ... (four LDS rows each: four consecutive keys of one
-    // page, 1 KB in a row) and the value pieces KT w .. KT w + KT - 1 (a group of 16 keys has four pieces of 32 dims).
-    const unsigned dma_k_off = (unsigned)(lane >> 4) * (2 * D) + ((unsigned)((lane & 15) ^ ((4 * wv + (lane >> 4)) & 15)) << 4);
-    const unsigned dma_v_off = (unsigned)((lane & 15) + 16 * (lane >> 5)) * (unsigned)(2 * ps) + (unsigned)((lane >> 4) & 1) * 16u;
-    // This wave's three groups of 16 keys of the next block to fetch (two for its key pieces, one for its values):
-    // the entry's page they lie in and the offset in it, moved on by KB keys per fetch without a division; the page
-    // ids are read from the block table a step ahead, through the constant address space (the kernel never writes
-    // the table): only so are they scalar loads, which do not wait for the loads into LDS that are in flight.
+    // Direct path: wave w brings the block's keys 16 w .. 16 w + 15 and their values: one group of 16 keys, which
+    // lies in one page, so a step costs the wave one page id and two addresses.  Its four key pieces (four keys
+    // each, 1 KB) go to the LDS rows that the score tiles read them from (see tile_key); its four value pieces are
+    // 32 dims each.  What differs from lane to lane and from piece to piece is fixed for the walk and kept in
+    // registers; what changes from step to step is the same in every lane and kept in scalar registers.
+    unsigned dma_k_off[4], dma_v_off[4];
+    unsigned dma_k_lds[4], dma_v_lds[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const int sw = (8 * (wv & 1) + 4 * (c >> 1) + (lane >> 4)) & 15;
+        dma_k_off[c] = (unsigned)(4 * c + (lane >> 4)) * (2 * D) + ((unsigned)((lane & 15) ^ sw) << 4);
+        dma_k_lds[c] = (unsigned)(8 * (wv >> 1) + 4 * (c & 1) + 2 * (wv & 1) + (c >> 1)) * 1024u;
+        dma_v_off[c] = (unsigned)((lane & 15) + 16 * (lane >> 5) + 32 * c) * (unsigned)(2 * ps) + (unsigned)((lane >> 4) & 1) * 16u;
+        dma_v_lds[c] = (unsigned)wv * 4096u + (unsigned)c * 1024u;
+    }
+    // The group's page and its offset there move on by KB keys per fetch without a division; the page id is read
+    // from the block table a step ahead, through the constant address space (the kernel never writes the table):
+    // only so is it a scalar load, which does not wait for the loads into LDS that are in flight.
     typedef const __attribute__((address_space(4))) int* const_int_ptr;
     const const_int_ptr btc = (const_int_ptr)(uintptr_t)bt;
     const unsigned lds_k0 = lds_address(k_lds), lds_v0 = lds_address(v_lds);
-    constexpr int NGW = KH + 1;                           // groups of a block that a wave touches
-    const int v_group = (wv * KT) >> 2;                   // the group whose values this wave brings
-    int g_blk[NGW], g_off[NGW], g_pg[NGW];
     const int adv_blk = KB / ps, adv_off = KB - adv_blk * ps;
-#pragma unroll
-    for (int i = 0; i < NGW; ++i) {
-        const int kp = key_lo + (i < KH ? 32 * i + 16 * (wv >> 1) : 16 * v_group);
-        g_blk[i] = kp / ps;
-        g_off[i] = kp - g_blk[i] * ps;
+    int g_blk, g_off, g_pg;
+    {
+        const int kp = key_lo + 16 * wv;
+        g_blk = kp / ps;
+        g_off = kp - g_blk * ps;
     }
-    auto dma_pages = [&]() __attribute__((always_inline)) {
-#pragma unroll
-        for (int i = 0; i < NGW; ++i) g_pg[i] = btc[min(g_blk[i], last_page)];
-    };
+    auto dma_pages = [&]() __attribute__((always_inline)) { g_pg = btc[min(g_blk, last_page)]; };
     auto fetch_dma = [&](int buf) __attribute__((always_inline)) {
         const unsigned kd = lds_k0 + buf * (KBUF * 2), vd = lds_v0 + buf * (VBUF * 2);     // byte addresses in LDS
+        const int pg = ((unsigned)g_pg < (unsigned)a.num_pages) ? g_pg : pg_spare;
+        const size_t pg_off = (size_t)(unsigned)pg * page_bytes;
+        const char* ksrc = k_base + (pg_off + (unsigned)(g_off * (2 * D)));
+        const char* vsrc = v_base + (pg_off + (unsigned)(g_off * 2));
 #pragma unroll
-        for (int n = 0; n < KT; ++n) {
-            const int h = n >> 1, key0 = 8 * (wv & 1) + 4 * (n & 1);
-            const int pg = (g_pg[h] >= 0 && g_pg[h] < a.num_pages) ? g_pg[h] : pg_spare;
-            const char* src = k_base + ((size_t)pg * page_bytes + (unsigned)((g_off[h] + key0) * (2 * D)));
-            load_to_lds16(src, dma_k_off, kd + (wv + 4 * n) * 1024);
-        }
-        const int pg = (g_pg[KH] >= 0 && g_pg[KH] < a.num_pages) ? g_pg[KH] : pg_spare;
-        const char* vsrc = v_base + ((size_t)pg * page_bytes + (unsigned)(g_off[KH] * 2));
+        for (int c = 0; c < 4; ++c) load_to_lds16(ksrc, dma_k_off[c], kd + dma_k_lds[c]);
 #pragma unroll
-        for (int m = 0; m < KT; ++m) {
-            const int u = (wv * KT + m) & 3;              // the piece of 32 dims
-            load_to_lds16(vsrc + (size_t)(u * 32) * (2 * ps), dma_v_off, vd + v_group * 4096 + u * 1024);
-        }
-#pragma unroll
-        for (int i = 0; i < NGW; ++i) {
-            g_blk[i] += adv_blk;
-            g_off[i] += adv_off;
-            const bool wrap = g_off[i] >= ps;
-            g_off[i] -= wrap ? ps : 0;
-            g_blk[i] += wrap ? 1 : 0;
-        }
+        for (int c = 0; c < 4; ++c) load_to_lds16(vsrc, dma_v_off[c], vd + dma_v_lds[c]);
+        g_blk += adv_blk;
+        g_off += adv_off;
+        const bool wrap = g_off >= ps;
+        g_off -= wrap ? ps : 0;
+        g_blk += wrap ? 1 : 0;
         dma_pages();
     };
     auto fetch = [&]() __attribute__((always_inline)) {   // this thread's pieces of the next KB keys, pages -> registers
@@ -996,19 +994,44 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_tile_kernel(At
                 }
             }
         }
+        // The order the compiler gives these on its own is "read an operand, wait for it, multiply"; asked for
+        // here: the reads of AHEAD operands first, then after every operand's products the read that is AHEAD
+        // operands further on, so that an operand has been on its way for that many products when it is needed.
+        // (Heads above 128, one block per compute unit: measured slower with it at one row tile.)
+        if constexpr (WIDE && (D <= 128 || RT == 2)) {
+#pragma unroll
+            for (int n = 0; n < AHEAD; ++n) __builtin_amdgcn_sched_group_barrier(SCHED_LDS_READ, 1, 0);
+#pragma unroll
+            for (int n = 0; n < KT * QSTEPS; ++n) {
+                __builtin_amdgcn_sched_group_barrier(SCHED_MFMA, RT, 0);
+                if (n + AHEAD < KT * QSTEPS) __builtin_amdgcn_sched_group_barrier(SCHED_LDS_READ, 1, 0);
+            }
+        }
         // s[rt][kt][i] is key j0 + tile_key(kt, g, i) against row r of tile rt.  A tile with no visible key in
         // this block keeps its state: every probability is 0 and its factor 1.
         unsigned pk[RT][KT * 2];
+        float alpha[RT];
+        bool full = true;      // every key of the block is visible to every row of the wave
 #pragma unroll
-        for (int rt = 0; rt < RT; ++rt) {
-            const bool full = (j0 + KB - 1 <= tile_first_p[rt]) && (j0 >= tile_last_lo[rt]);
-            float alpha;
-            if (full) tile_softmax<true>(s[rt], j0, g, p[rt], p_lo[rt], a.scale_log2, m[rt], alpha, pk[rt]);
-            else tile_softmax<false>(s[rt], j0, g, p[rt], p_lo[rt], a.scale_log2, m[rt], alpha, pk[rt]);
-            if (__any(alpha != 1.f)) {      // the maximum of some row moved
+        for (int rt = 0; rt < RT; ++rt) full = full && (j0 + KB - 1 <= tile_first_p[rt]) && (j0 >= tile_last_lo[rt]);
+        if (full) {
+            // (the tiles one after the other in one stretch of code: each one's chain of dependent operations
+            // fills the other's waits)
 #pragma unroll
-                for (int t = 0; t < DT; ++t) o[rt][t] *= alpha;
-                ol[rt] *= alpha;
+            for (int rt = 0; rt < RT; ++rt) tile_softmax<true>(s[rt], j0, g, p[rt], p_lo[rt], a.scale_log2, m[rt], alpha[rt], pk[rt]);
+        } else {
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) tile_softmax<false>(s[rt], j0, g, p[rt], p_lo[rt], a.scale_log2, m[rt], alpha[rt], pk[rt]);
+        }
+        bool moved = false;
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) moved = moved || (alpha[rt] != 1.f);
+        if (__any(moved)) {      // the maximum of some row moved
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+#pragma unroll
+                for (int t = 0; t < DT; ++t) o[rt][t] *= alpha[rt];
+                ol[rt] *= alpha[rt];
             }
         }
 #pragma unroll
@@ -1027,6 +1050,17 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void attn_bf16_tile_kernel(At
 #pragma unroll
                 for (int rt = 0; rt < RT; ++rt)
                     o[rt][t] = VT_MFMA_16X16X32(vf.v, pf[rt].v, o[rt][t]);
+            }
+        }
+        // (the same order for the value operands; a half's products begin with its row sums)
+        if constexpr (D <= 128 || RT == 2) {
+#pragma unroll
+            for (int n = 0; n < AHEAD; ++n) __builtin_amdgcn_sched_group_barrier(SCHED_LDS_READ, 1, 0);
+#pragma unroll
+            for (int n = 0; n < KH * DT; ++n) {
+                if (n % DT == 0) __builtin_amdgcn_sched_group_barrier(SCHED_MFMA, RT, 0);
+                __builtin_amdgcn_sched_group_barrier(SCHED_MFMA, RT, 0);
+                if (n + AHEAD < KH * DT) __builtin_amdgcn_sched_group_barrier(SCHED_LDS_READ, 1, 0);
             }
         }
     };

@@ -69,6 +69,13 @@ DIRECT_START_US = 4.0
 DIRECT_BLOCK_US = 4.0
 DIRECT_SLOTS = 448
 DIRECT_MERGE_US = (8.0, 0.03)
+# ... and the cuts it is asked about: none, at TILE_CUT, and a finer one.  The finer one is for portions behind a long
+# context on few kv heads, whose items are few and long (2,048 tokens behind 30,720 on 12 / 2 heads: 192 blocks of 500
+# steps): two ranges each still leave a quarter of the slots empty, four fill them (476 -> 427 us; behind 14,336:
+# 246 -> 226).  Measured over 39 shapes (512 to 16,384 tokens, up to 30,720 earlier ones, 12 / 2, 28 / 4 and 64 / 8
+# heads, one to sixteen prompts): the model's choice among these is 1.0 % behind the best of the twelve on average
+# (1.4 % without the finer cut), at worst 4 us on a 29 us launch.
+DIRECT_CUTS = (0., 0.8, TILE_CUT)
 TILE_MIN_STEPS = 6      # no item's keys are cut into ranges of fewer steps than this
 TILE_MAX_PARTS = 8      # ... or into more ranges than this
 LONG_ENTRY_ROWS = 256   # entries with at least this many (token, head-of-group) rows go to the LDS-tiled kernel
@@ -96,7 +103,7 @@ def plan_tile_items(entry_start: np.ndarray, entry_pos0: np.ndarray, group: int,
     override the choice.
 
     `direct`: the kernel brings its key/value blocks from the pages straight into LDS (head size 128).  Then one and
-    two row tiles, with and without cuts at TILE_CUT, are priced with a model of the launch (DIRECT_*) and the
+    two row tiles, each with every cut of DIRECT_CUTS (no cut among them), are priced with a model of the launch (DIRECT_*) and the
     cheapest is taken.  Otherwise: two row tiles with cuts up to a head size of 128 (a block's step takes about as
     long with two row tiles as with one there, TILE_STEP_US), whole items and the cheaper row tiles above."""
     q_len = (entry_start[1:] - entry_start[:-1]).astype(np.int64)[entries]
@@ -150,7 +157,7 @@ def plan_tile_items(entry_start: np.ndarray, entry_pos0: np.ndarray, group: int,
             it = items_for(rt_)
             if it is None:
                 return none
-            for split_ in ((0., TILE_CUT) if split is None else (split,)):
+            for split_ in (DIRECT_CUTS if split is None else (split,)):
                 cost = direct_estimate(it, rt_, parts_of(steps_of(it), split_))
                 if best is None or cost < best[0]:
                     best = (cost, rt_, split_)
