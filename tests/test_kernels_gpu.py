@@ -391,6 +391,17 @@ def test_attention_page_sizes_and_edges(dtype, page_size):
     assert rel_err(got, ref) < ATT_TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("page_size,window", [(32, 0), (48, 100), (64, 0), (128, 33)])
+def test_attention_head_128_page_sizes(dtype, page_size, window):
+    """Head size 128: the tiled kernel's waves bring one group of 16 keys each from the pages straight into LDS, and
+    walk on by 64 keys without a division.  Pages that hold two, three, four and eight such groups; portions that
+    begin in the middle of a page and of a group; a window that frees the pages behind it."""
+    entries = [(0, 3 * page_size + 5), (page_size + 7, 300), (523, 90), (2 * page_size - 1, 1)]
+    got, ref = attention_case(dtype, 14, 2, 128, page_size, window, entries, seed=page_size + window, spike=window > 0)
+    assert rel_err(got, ref) < ATT_TOL[dtype]
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("window", [1, 5, 16, 40])
 def test_attention_window_edge(dtype, window):
