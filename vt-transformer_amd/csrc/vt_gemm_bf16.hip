@@ -196,7 +196,14 @@ __device__ __forceinline__ void link_row_scales(const NormLink& link, int K, flo
 // (rounded to bf16) as its tokens, adds up h^2 on the way (every block walks all of k, so every block has the whole
 // sum of every row) and multiplies the finished sums by 1/sqrt(mean(h^2) + eps): the norm costs no launch and no
 // pass over h of its own.  resid: fp32 [N][Mout] that the result is added to (y may be resid itself).
-template <int WPB, bool SWIGLU, bool NORM, typename TO>
+// PARTS = 2: a block owns half a tile row, 8 features; the lanes of the other 8 rows load nothing and multiply zeros.
+// Twice the blocks, for matrices with so few tile rows that whole ones would leave more than half of the compute
+// units without a block (Qwen2-1.5B's q/k/v, output and down projections: 128, 96 and 96 tile rows; a decoding step at
+// batch 8 1.42 -> 1.35 ms).  A tile's 16 rows x 32 k are packed as four stretches of 256 bytes, the first half of each
+// being rows 0 to 7: a half block reads whole 128-byte lines, and no line that its other half reads.  (Quarters read
+// half lines: 1.69 ms.  Halves for matrices of 224 and 288 tile rows, which fill the compute units unevenly: 3.05 ->
+// 3.36 ms at Qwen2-7B's sizes.  Halves with 8 waves a block where whole tile rows take 16: 1.39 ms.)
+template <int WPB, bool SWIGLU, bool NORM, typename TO, int PARTS = 1>
 __global__ __launch_bounds__(WPB * 64) void gemm_skinny_kernel(const void* __restrict__ xin, const bf16_t* __restrict__ wp,
                                                               const float* __restrict__ bias, TO* __restrict__ y, int N,
                                                               int Mout, int K, int KT, int up_tiles,
@@ -210,7 +217,11 @@ __global__ __launch_bounds__(WPB * 64) void gemm_skinny_kernel(const void* __res
     __shared__ float4 ssq_part[WPB][4];                       // consumer of a NormLink: the waves' sums of shares
     const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63;
     const int r = lane & 15, g = lane >> 4;
-    const int mt = blockIdx.x;
+    static_assert(!(PARTS > 1 && SWIGLU), "the gated product has tile rows enough");
+    constexpr int RB = 16 / PARTS;                    // features of the block
+    const int mt = blockIdx.x / PARTS, hb = blockIdx.x % PARTS;
+    const bool w_on = PARTS == 1 || r / RB == hb;     // this lane's row of W is one of the block's
+    auto load_w = [&](const bf16_t* p) __attribute__((always_inline)) { return w_on ? load_w_once(p) : make_uint4(0u, 0u, 0u, 0u); };
     // Consumer of a NormLink: thread t adds up rows 4 (t % 4) .. + 3 of shares t / 4, t / 4 + threads / 4, ...; the
     // first two loads are asked for here, ahead of everything, and used at the end.
     float4 sh0 = make_float4(0.f, 0.f, 0.f, 0.f), sh1 = sh0;
@@ -317,7 +328,7 @@ __global__ __launch_bounds__(WPB * 64) void gemm_skinny_kernel(const void* __res
                 for (int u = 0; u < 2; ++u)
 #pragma unroll
                     for (int a = 0; a < NW; ++a)
-                        wa[a][2 * up + u].u = load_w_once(wbase[a] + (size_t)(2 * (p + up) + u) * PK_TILE);
+                        wa[a][2 * up + u].u = load_w(wbase[a] + (size_t)(2 * (p + up) + u) * PK_TILE);
                 xa[up].v = load_x(xr_a, (p + up) * 64 + xpc, K);
                 if (two) xb[up].v = load_x(xr_b, (p + up) * 64 + xpc, K);
             }
@@ -334,7 +345,7 @@ __global__ __launch_bounds__(WPB * 64) void gemm_skinny_kernel(const void* __res
 #pragma unroll
             for (int u = 0; u < 2; ++u)
 #pragma unroll
-                for (int a = 0; a < NW; ++a) wa[a][u].u = load_w_once(wbase[a] + (size_t)(2 * p + u) * PK_TILE);
+                for (int a = 0; a < NW; ++a) wa[a][u].u = load_w(wbase[a] + (size_t)(2 * p + u) * PK_TILE);
             xa.v = load_x(xr_a, p * 64 + xpc, K);
             if (two) xb.v = load_x(xr_b, p * 64 + xpc, K);
             pair_exchange(xa, xb, 0, xf[0], xf[1]);
@@ -352,7 +363,7 @@ __global__ __launch_bounds__(WPB * 64) void gemm_skinny_kernel(const void* __res
 #pragma unroll
         for (int u = 0; u < U; ++u) {
 #pragma unroll
-            for (int a = 0; a < NW; ++a) wa[a][u].u = load_w_once(wbase[a] + (size_t)(t + u) * PK_TILE);
+            for (int a = 0; a < NW; ++a) wa[a][u].u = load_w(wbase[a] + (size_t)(t + u) * PK_TILE);
             xa[u] = load_piece(t + u);
         }
         if constexpr (NORM) __builtin_amdgcn_sched_barrier(0);
@@ -374,7 +385,7 @@ __global__ __launch_bounds__(WPB * 64) void gemm_skinny_kernel(const void* __res
 #pragma unroll
         for (int a = 0; a < NW; ++a) {
             Frag wa;
-            wa.u = load_w_once(wbase[a] + (size_t)t * PK_TILE);
+            wa.u = load_w(wbase[a] + (size_t)t * PK_TILE);
             acc[a] = VT_MFMA_16X16X32(wa.v, xa.f.v, acc[a]);
         }
     }
@@ -418,7 +429,7 @@ __global__ __launch_bounds__(WPB * 64) void gemm_skinny_kernel(const void* __res
         if (SWIGLU)
             for (int q = 0; q < WPB; ++q) u += red[NW - 1][q][c];
         float sq = 0.f;
-        if (m < Mout && n < N) {
+        if (m < Mout && n < N && (PARTS == 1 || (4 * (ln >> 4) + e) / RB == hb)) {
             if constexpr (NORM) {
                 float tot = 0.f;
                 for (int q = 0; q < WPB; ++q) tot += ssq[q][n];
@@ -917,6 +928,12 @@ static int mid_waves(int Mout, int rows_per_wave, int token_blocks) {
     return best;
 }
 
+// Up to 16 tokens: the parts of a tile row of W [Mout, .] that blocks take (gemm_skinny_kernel<PARTS>); by the shape of W
+// alone, so that a token's sums do not depend on the number of rows.
+static int skinny_parts(int Mout) {
+    return 2 * ((Mout + 15) / 16) <= compute_units() ? 2 : 1;
+}
+
 // 17 to 64 rows: tile rows per block (1 or 2) if gemm_rows_kernel takes the product, 0 if the 64-token kernel does.
 // The first lasts about 4 us + 0.026 us per k tile and token tile (every block takes in all the tokens, and that
 // is what its time goes to, however many rows of W it has); the second about 14 us, the launch that adds its
@@ -956,7 +973,7 @@ static const NormLink NO_LINK = {nullptr, nullptr, nullptr, nullptr, 0, 0.f};
 extern "C" int vt_linear_bf16_link_shares(int N, int M, int K) {
     if (N <= 0 || N > ROWS_MAX || M <= 0 || K <= 0 || K % 8 != 0 || M % 8 != 0) return 0;
     const int tiles = (M + 15) / 16;
-    if (N <= 16) return tiles;                                          // a block per tile row
+    if (N <= 16) return skinny_parts(M) * tiles;                       // a block per tile row, or per part of one
     const int rr = rows_tile_rows(N, M, K);
     if (rr) return (tiles + rr - 1) / rr;                               // a block per rr tile rows, whole k
     if (mid_splits(M, K, 128) > 1) return (M + SUM_COLS - 1) / SUM_COLS; // the launch that adds the partial sums
@@ -1057,9 +1074,19 @@ static int linear_bf16(const void* xv, const bf16_t* wp, const float* bias, TO* 
     const int tiles16 = (Mout + 15) / 16;
     const bool wide = tiles16 >= 512 || KT < 256;
 #define VT_SKINNY(W, NRM) gemm_skinny_kernel<W, SWIGLU, NRM, TO><<<tiles16, W * 64, 0, stream>>>(x, wp, bias, y, N, Mout, K, KT, up_tiles, gain, eps, resid, link)
+#define VT_SKINNY_PART(P, W, NRM) gemm_skinny_kernel<W, false, NRM, TO, P><<<P * tiles16, W * 64, 0, stream>>>(x, wp, bias, y, N, Mout, K, KT, up_tiles, gain, eps, resid, link)
+    if constexpr (!SWIGLU) {
+        if (skinny_parts(Mout) == 2) {
+            if (gain) { if (wide) VT_SKINNY_PART(2, 8, true); else VT_SKINNY_PART(2, 16, true); }
+            else { if (wide) VT_SKINNY_PART(2, 8, false); else VT_SKINNY_PART(2, 16, false); }
+            VT_CHECK_LAUNCH("vt_linear_bf16(half tile rows)");
+            return 0;
+        }
+    }
     if (gain) { if (wide) VT_SKINNY(8, true); else VT_SKINNY(16, true); }
     else { if (wide) VT_SKINNY(8, false); else VT_SKINNY(16, false); }
 #undef VT_SKINNY
+#undef VT_SKINNY_PART
     VT_CHECK_LAUNCH("vt_linear_bf16");
     return 0;
 }
