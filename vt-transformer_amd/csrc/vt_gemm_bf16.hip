@@ -916,10 +916,10 @@ static int mid_splits(int Mout, int K, int rows_per_block) {
 // the launch lasts (rounds of blocks over the compute units) x (work of a block); pick the smallest product.
 static int mid_waves(int Mout, int rows_per_wave, int token_blocks) {
     const int cus = compute_units();
-    const int choices[4] = {4, 5, 6, 8};
+    const int choices[5] = {3, 4, 5, 6, 8};
     int best = 4;
     long best_cost = -1;
-    for (int c = 0; c < 4; ++c) {
+    for (int c = 0; c < 5; ++c) {
         const int w = choices[c], rows = rows_per_wave * w;
         const long blocks = (long)((Mout + rows - 1) / rows) * token_blocks;
         const long cost = ((blocks + cus - 1) / cus) * w;
@@ -1044,7 +1044,8 @@ static int linear_bf16(const void* xv, const bf16_t* wp, const float* bias, TO* 
         } while (0)
 #define VT_MID_(W, O) do { if (tok == 64) VT_MID__(W, O, 4); else VT_MID__(W, O, 8); } while (0)
 #define VT_MID(W) do { if (grid.y == 1) VT_MID_(W, true); else VT_MID_(W, false); } while (0)
-        if (wm == 4) VT_MID(4);
+        if (wm == 3) VT_MID(3);
+        else if (wm == 4) VT_MID(4);
         else if (wm == 5) VT_MID(5);
         else if (wm == 6) VT_MID(6);
         else VT_MID(8);
