@@ -265,8 +265,10 @@ def test_gated_linear_bf16(n, inter, k, lp):
 # ---------------------------------------------------------------------------
 # paged cache helpers
 # ---------------------------------------------------------------------------
-def make_pages(k, v, lens, page_size, dtype, seed, extra_pages=3):
-    """k, v: lists of [T_e, KVH, D] per entry.  Pages in shuffled order.  Returns k_pages, v_pages, block_table."""
+def make_pages(k, v, lens, page_size, dtype, seed, extra_pages=3, free_before=None):
+    """k, v: lists of [T_e, KVH, D] per entry.  Pages in shuffled order.  Returns k_pages, v_pages, block_table.
+    free_before[e]: pages that lie wholly before this key have been given back (a window has passed them): the
+    table holds -1 there, as the cache manager leaves it."""
     kvh, d = k[0].shape[1], k[0].shape[2]
     n_blocks = [-(-t // page_size) for t in lens]
     total = sum(n_blocks) + extra_pages
@@ -277,6 +279,8 @@ def make_pages(k, v, lens, page_size, dtype, seed, extra_pages=3):
     nxt = 0
     for e, t in enumerate(lens):
         for b in range(n_blocks[e]):
+            if free_before is not None and (b + 1) * page_size <= free_before[e]:
+                continue
             pg = int(perm[nxt]); nxt += 1
             bt[e, b] = pg
             lo, hi = b * page_size, min(t, (b + 1) * page_size)
@@ -318,7 +322,9 @@ def attention_case(dtype, nh, kvh, d, page_size, window, entries, seed, spike=Fa
             vs[e][far] = 5.0
     if dtype != torch.float32:
         ks, vs, qs = ([t.to(dtype).float() for t in x] for x in (ks, vs, qs))
-    kp, vp, bt = make_pages(ks, vs, lens, page_size, dtype, seed)
+    # with a window: the pages that the entry's first new token no longer sees are gone
+    free_before = [max(0, c - window + 1) for c, _ in entries] if window > 0 else None
+    kp, vp, bt = make_pages(ks, vs, lens, page_size, dtype, seed, free_before=free_before)
     n_tok = sum(n for _, n in entries)
     q = torch.cat(qs).reshape(n_tok, nh * d).to(dtype).to(DEV)
     positions = torch.tensor([c + i for c, n in entries for i in range(n)], dtype=torch.int32)
