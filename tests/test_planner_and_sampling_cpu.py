@@ -161,4 +161,9 @@ def test_the_direct_kernels_launch_model_picks_what_was_measured():
         return rt, n_parts
     assert pick([2048], [0]) == (1, 0)
     assert pick([2048], [2048])[0] == 2
+    assert pick([2048], [2048])[1] == 0            # (cutting these costs a fifth: 112 -> 127 to 138 us)
     assert pick([1024] * 8, [0] * 8) == (2, 0)
+    # A 2,048-token portion behind 30,720 earlier tokens on 12 / 2 heads is 192 blocks of 500 steps: two key ranges
+    # each would leave a quarter of the 512 slots empty, four fill them (476 -> 427 us).
+    rt, n_parts = pick([2048], [30720], nh=12, nkv=2)
+    assert rt == 2 and n_parts == 4 * 96
